@@ -1,0 +1,153 @@
+// Internal declarations shared by the host-side C ABI (rt_api.hip) and the
+// kernel launchers (rt_kernels.hip, rt_gemm.hip).  Not installed; the public
+// surface is include/rustorch_hip.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <mutex>
+#include <string>
+
+#include "../../include/rustorch_hip.h"
+
+namespace rt {
+
+// Denominators every reported fraction is priced against (MI355X, gfx950 / CDNA4).
+constexpr double kHbmPeakBytesPerSec = 8.0e12;
+constexpr double kMfmaF16PeakFlops = 2.5e15;
+constexpr int kWave = 64;
+
+// ---- quantized activation vector ("xq"): what the GEMV kernels consume.
+// A vector of K floats (K % 32 == 0) is stored per 32-element block as
+//   q = rint(x * 16383 / amax_block)  in [-16383, 16383],   q = 128 * qh + ql,
+//   qh in [-128,127] (int8), ql in [0,127] (int8), scale s = amax_block / 16383,
+// so that an integer dot with int8 weights is exact:  sum w*q = 128*sum w*qh + sum w*ql.
+// Byte layout of one vector:
+//   [0, K)            qh   int8[K]
+//   [K, 2K)           ql   int8[K]
+//   [2K, 2K+K/8)      s    f32[K/32]
+//   [.., +K/4)        bsum f32[K/16] = s * (sum of q over each 16-element run)  (for the -8 / -32 / -min terms)
+// padded to a multiple of 16 bytes.
+__host__ __device__ inline size_t xq_stride(size_t K) { return (2 * K + K / 8 + K / 4 + 15) & ~(size_t)15; }
+
+struct GemvProb {
+    const uint8_t *w;    // raw GGUF blocks, row r at w + r * row_bytes
+    const uint8_t *xq;   // quantized activations, vector m at xq + m * xq_stride(K)
+    float *y;            // [batch, N]
+    const float *res;    // optional residual added to y (same shape), may alias y
+    size_t row_bytes;
+    int type, N, K;
+    int tile0;           // index of this problem's first tile in the launch
+    int rows_per_tile;
+};
+constexpr int kMaxGemvProbs = 8;
+struct GemvArgs {
+    GemvProb p[kMaxGemvProbs];
+    int n;
+};
+
+struct Llama;  // defined in rt_llama.hip
+
+// ---- launchers (all enqueue on `s`, return hipError_t of the launch)
+hipError_t launch_quantize_x(hipStream_t s, const float *x, uint8_t *xq, size_t K, size_t batch);
+hipError_t launch_qgemv(hipStream_t s, GemvArgs &args, int batch);  // fills tile0 / rows_per_tile
+hipError_t launch_dequant(hipStream_t s, int type, const uint8_t *w, size_t n_rows, size_t n_cols, float *out);
+hipError_t launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *y, uint8_t *xq, size_t rows,
+                          size_t n, float eps);
+hipError_t launch_swiglu(hipStream_t s, const float *gate, const float *up, float *out, uint8_t *xq, size_t n);
+hipError_t launch_rope(hipStream_t s, float *x, int n_heads, int head_dim, const int *pos_dev, int pos,
+                       const float *inv_freq_dev, float theta);
+hipError_t launch_kv_append(hipStream_t s, uint16_t *cache, const float *v, const int *pos_dev, size_t pos,
+                            size_t row_elems);
+hipError_t launch_rope_kv(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache,
+                          uint16_t *vcache, const int *pos_dev, int n_heads, int head_dim,
+                          const float *inv_freq_dev);
+hipError_t launch_attn_decode(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc,
+                              const int *pos_dev, int n_pos, int n_heads, int head_dim, float *out, uint8_t *xq);
+hipError_t launch_add(hipStream_t s, float *x, const float *y, size_t n);
+hipError_t launch_argmax(hipStream_t s, const float *v, size_t n, int *out_dev);
+hipError_t launch_embed_row(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,
+                            const int *token_dev, int vocab, float *out);
+hipError_t launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *c, size_t m, size_t n, size_t k);
+hipError_t launch_set_int(hipStream_t s, int *dst, int value);
+hipError_t launch_step_advance(hipStream_t s, int *pos_dev, int *token_dev, const int *pick_dev,
+                               const int *forced_dev, int *out_tokens_dev, int *step_dev);
+// prefill GEMM (rt_gemm.hip)
+hipError_t launch_qgemm(hipStream_t s, int type, const uint8_t *w, size_t N, size_t K, size_t row_bytes,
+                        const float *X, size_t M, float *Y, const float *res, void *scratch, size_t scratch_bytes);
+size_t qgemm_scratch_bytes(size_t M, size_t K);
+
+inline size_t type_block_bytes(int t) {
+    switch (t) {
+    case RT_GGML_F32: return 4;
+    case RT_GGML_F16: return 2;
+    case RT_GGML_Q4_0: return 18;
+    case RT_GGML_Q8_0: return 34;
+    case RT_GGML_Q4_K: return 144;
+    case RT_GGML_Q6_K: return 210;
+    default: return 0;
+    }
+}
+inline size_t type_block_elems(int t) {
+    switch (t) {
+    case RT_GGML_F32: case RT_GGML_F16: return 1;
+    case RT_GGML_Q4_0: case RT_GGML_Q8_0: return 32;
+    case RT_GGML_Q4_K: case RT_GGML_Q6_K: return 256;
+    default: return 0;
+    }
+}
+
+}  // namespace rt
+
+struct rt_hip_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::mutex mu;
+    std::string err;
+    // scratch owned by the context for the host-pointer entry points and the xq of *_dev GEMV calls
+    void *scratch = nullptr;
+    size_t scratch_bytes = 0;
+};
+
+struct rt_hip_qweight {
+    int type = 0;
+    size_t n_rows = 0, n_cols = 0, nbytes = 0, row_bytes = 0;
+    uint8_t *dev = nullptr;
+    bool owns = false;
+};
+
+struct rt_hip_event {
+    hipEvent_t ev = nullptr;
+};
+
+// ---- host-side helpers shared by the C-ABI translation units
+namespace rt {
+int fail(rt_hip_ctx *ctx, int code, const char *fmt, ...) __attribute__((format(printf, 3, 4)));
+int hip_fail(rt_hip_ctx *ctx, hipError_t e, const char *what);
+int ensure_scratch(rt_hip_ctx *ctx, size_t bytes);
+
+// Serialises calls on one context and makes its device current.
+struct Guard {
+    rt_hip_ctx *c;
+    explicit Guard(rt_hip_ctx *ctx) : c(ctx) {
+        c->mu.lock();
+        (void)hipSetDevice(c->device);
+    }
+    ~Guard() { c->mu.unlock(); }
+    Guard(const Guard &) = delete;
+    Guard &operator=(const Guard &) = delete;
+};
+}  // namespace rt
+
+#define RT_TRY_HIP(ctx, expr)                                        \
+    do {                                                             \
+        hipError_t e__ = (expr);                                     \
+        if (e__ != hipSuccess) return rt::hip_fail(ctx, e__, #expr); \
+    } while (0)
+
+#define RT_REQUIRE(ctx, cond, code, ...)                      \
+    do {                                                      \
+        if (!(cond)) return rt::fail(ctx, code, __VA_ARGS__); \
+    } while (0)

@@ -1,0 +1,333 @@
+// Llama-architecture decode loop on one GPU: weights stay in HBM as raw GGUF
+// blocks, the KV cache is fp16 [layer][pos][head][dim], and one decode step is a
+// fixed sequence of kernels driven by device-resident position / token state, so
+// consecutive steps need no host round trip.
+//
+// Step order (pre-norm residual block of example-cli/src/model/architectures/gpt.rs:43-55,192-215
+// with RMSNorm / RoPE / SwiGLU / causal cache in place of LayerNorm / sinusoidal PE / ReLU / full recompute):
+//   x = embd[token]
+//   per layer: h = rmsnorm(x); q,k,v = W h; rope(q,k); cache <- k,v; a = attn(q, cache);
+//              x += Wo a; h = rmsnorm(x); x += Wdown (up(h) * silu(gate(h)))
+//   logits = Wout rmsnorm(x)
+#include "rt_internal.h"
+
+#include <cmath>
+#include <cstring>
+#include <new>
+#include <vector>
+
+using rt::ensure_scratch;
+using rt::fail;
+using rt::Guard;
+using rt::hip_fail;
+
+struct rt_hip_llama {
+    struct T {
+        int type = -1;
+        size_t n_rows = 0, n_cols = 0, row_bytes = 0, nbytes = 0;
+        uint8_t *dev = nullptr;
+    };
+    rt_hip_llama_config cfg{};
+    int head_dim = 0;
+    T tok_embd, output;
+    float *out_norm = nullptr;
+    std::vector<T> wq, wk, wv, wo, wgate, wup, wdown;
+    std::vector<float *> attn_norm, ffn_norm;
+    uint16_t *kcache = nullptr, *vcache = nullptr;
+    float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *g = nullptr, *u = nullptr, *logits = nullptr;
+    uint8_t *xq_h = nullptr, *xq_a = nullptr, *xq_f = nullptr;
+    float *inv_freq = nullptr;
+    int *state = nullptr;  // [0] pos, [1] token, [2] pick, [3] step
+    int *forced_dev = nullptr, *out_tokens_dev = nullptr;
+    int n_fed = 0;
+    std::vector<void *> allocs;
+};
+
+namespace {
+
+int dev_alloc(rt_hip_ctx *ctx, rt_hip_llama *m, void **p, size_t bytes) {
+    RT_TRY_HIP(ctx, hipMalloc(p, bytes ? bytes : 1));
+    m->allocs.push_back(*p);
+    return RT_HIP_OK;
+}
+
+void free_all(rt_hip_llama *m) {
+    for (void *p : m->allocs) (void)hipFree(p);
+    m->allocs.clear();
+}
+
+void fill_prob(rt::GemvProb &p, const rt_hip_llama::T &t, const uint8_t *xq, float *y, const float *res) {
+    p.w = t.dev; p.xq = xq; p.y = y; p.res = res; p.row_bytes = t.row_bytes;
+    p.type = t.type; p.N = (int)t.n_rows; p.K = (int)t.n_cols;
+}
+
+int check_complete(rt_hip_ctx *ctx, const rt_hip_llama *m) {
+    RT_REQUIRE(ctx, m->tok_embd.dev && m->output.dev && m->out_norm, RT_HIP_ERR_INVALID_ARG,
+               "llama: token embedding / output head / output norm not uploaded");
+    for (int l = 0; l < m->cfg.n_layers; l++) {
+        bool ok = m->wq[l].dev && m->wk[l].dev && m->wv[l].dev && m->wo[l].dev && m->wgate[l].dev && m->wup[l].dev &&
+                  m->wdown[l].dev && m->attn_norm[l] && m->ffn_norm[l];
+        RT_REQUIRE(ctx, ok, RT_HIP_ERR_INVALID_ARG, "llama: layer %d has tensors that were not uploaded", l);
+    }
+    return RT_HIP_OK;
+}
+
+// One decode step driven by state[0] (pos) and state[1] (token). Enqueue only.
+int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
+    hipStream_t s = ctx->stream;
+    const rt_hip_llama_config &c = m->cfg;
+    const size_t H = (size_t)c.hidden, F = (size_t)c.ffn;
+    int *pos_dev = m->state, *tok_dev = m->state + 1;
+    RT_TRY_HIP(ctx, rt::launch_embed_row(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, tok_dev, c.vocab, m->x));
+    for (int l = 0; l < c.n_layers; l++) {
+        uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * H;
+        uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * H;
+        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, m->x, m->attn_norm[l], nullptr, m->xq_h, 1, H, c.rms_eps));
+        rt::GemvArgs a;
+        memset(&a, 0, sizeof a);
+        a.n = 3;
+        fill_prob(a.p[0], m->wq[l], m->xq_h, m->q, nullptr);
+        fill_prob(a.p[1], m->wk[l], m->xq_h, m->k, nullptr);
+        fill_prob(a.p[2], m->wv[l], m->xq_h, m->v, nullptr);
+        RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
+        RT_TRY_HIP(ctx, rt::launch_rope_kv(s, m->q, m->k, m->v, kc, vc, pos_dev, c.n_heads, m->head_dim, m->inv_freq));
+        RT_TRY_HIP(ctx, rt::launch_attn_decode(s, m->q, kc, vc, pos_dev, c.max_pos, c.n_heads, m->head_dim, nullptr, m->xq_a));
+        memset(&a, 0, sizeof a);
+        a.n = 1;
+        fill_prob(a.p[0], m->wo[l], m->xq_a, m->x, m->x);
+        RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
+        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, m->x, m->ffn_norm[l], nullptr, m->xq_h, 1, H, c.rms_eps));
+        memset(&a, 0, sizeof a);
+        a.n = 2;
+        fill_prob(a.p[0], m->wgate[l], m->xq_h, m->g, nullptr);
+        fill_prob(a.p[1], m->wup[l], m->xq_h, m->u, nullptr);
+        RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
+        RT_TRY_HIP(ctx, rt::launch_swiglu(s, m->g, m->u, nullptr, m->xq_f, F));
+        memset(&a, 0, sizeof a);
+        a.n = 1;
+        fill_prob(a.p[0], m->wdown[l], m->xq_f, m->x, m->x);
+        RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
+    }
+    if (want_logits) {
+        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, m->x, m->out_norm, nullptr, m->xq_h, 1, H, c.rms_eps));
+        rt::GemvArgs a;
+        memset(&a, 0, sizeof a);
+        a.n = 1;
+        fill_prob(a.p[0], m->output, m->xq_h, m->logits, nullptr);
+        RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
+    }
+    return RT_HIP_OK;
+}
+
+bool gemv_type_ok(int t) { return t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_K || t == RT_GGML_Q6_K; }
+
+}  // namespace
+
+extern "C" {
+
+int rt_hip_llama_create(rt_hip_ctx *ctx, const rt_hip_llama_config *cfg, rt_hip_llama **out) {
+    if (!ctx || !cfg || !out) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_create: NULL argument");
+    *out = nullptr;
+    RT_REQUIRE(ctx, cfg->n_layers > 0 && cfg->hidden > 0 && cfg->n_heads > 0 && cfg->ffn > 0 && cfg->vocab > 0 && cfg->max_pos > 0,
+               RT_HIP_ERR_SHAPE, "llama config has a non-positive dimension");
+    RT_REQUIRE(ctx, cfg->hidden % cfg->n_heads == 0, RT_HIP_ERR_SHAPE, "hidden=%d not divisible by n_heads=%d", cfg->hidden, cfg->n_heads);
+    int hd = cfg->hidden / cfg->n_heads;
+    RT_REQUIRE(ctx, hd == 64 || hd == 128, RT_HIP_ERR_SHAPE, "head_dim=%d (64 or 128 supported)", hd);
+    RT_REQUIRE(ctx, cfg->hidden % 256 == 0 && cfg->ffn % 256 == 0, RT_HIP_ERR_SHAPE, "hidden=%d and ffn=%d must be multiples of 256", cfg->hidden, cfg->ffn);
+    RT_REQUIRE(ctx, cfg->max_pos <= 16000, RT_HIP_ERR_SHAPE, "max_pos=%d exceeds 16000", cfg->max_pos);
+    RT_REQUIRE(ctx, rt::xq_stride((size_t)cfg->ffn) <= 64 * 1024 && rt::xq_stride((size_t)cfg->hidden) <= 64 * 1024, RT_HIP_ERR_SHAPE,
+               "hidden / ffn exceed the GEMV staging limit");
+    RT_REQUIRE(ctx, cfg->rms_eps >= 0.f && cfg->rope_theta > 0.f, RT_HIP_ERR_INVALID_ARG, "rms_eps=%g rope_theta=%g", (double)cfg->rms_eps,
+               (double)cfg->rope_theta);
+    Guard g(ctx);
+    rt_hip_llama *m = new (std::nothrow) rt_hip_llama();
+    if (!m) return fail(ctx, RT_HIP_ERR_OOM, "host allocation failed");
+    m->cfg = *cfg;
+    m->head_dim = hd;
+    size_t L = (size_t)cfg->n_layers, H = (size_t)cfg->hidden, F = (size_t)cfg->ffn, V = (size_t)cfg->vocab, P = (size_t)cfg->max_pos;
+    m->wq.resize(L); m->wk.resize(L); m->wv.resize(L); m->wo.resize(L); m->wgate.resize(L); m->wup.resize(L); m->wdown.resize(L);
+    m->attn_norm.assign(L, nullptr); m->ffn_norm.assign(L, nullptr);
+    int rc = RT_HIP_OK;
+    auto A = [&](void **p, size_t b) { if (rc == RT_HIP_OK) rc = dev_alloc(ctx, m, p, b); };
+    A((void **)&m->kcache, L * P * H * 2); A((void **)&m->vcache, L * P * H * 2);
+    A((void **)&m->x, H * 4); A((void **)&m->q, H * 4); A((void **)&m->k, H * 4); A((void **)&m->v, H * 4);
+    A((void **)&m->g, F * 4); A((void **)&m->u, F * 4); A((void **)&m->logits, V * 4);
+    A((void **)&m->xq_h, rt::xq_stride(H)); A((void **)&m->xq_a, rt::xq_stride(H)); A((void **)&m->xq_f, rt::xq_stride(F));
+    A((void **)&m->inv_freq, (size_t)(hd / 2) * 4); A((void **)&m->state, 4 * sizeof(int));
+    A((void **)&m->forced_dev, P * sizeof(int)); A((void **)&m->out_tokens_dev, P * sizeof(int));
+    if (rc != RT_HIP_OK) { free_all(m); delete m; return rc; }
+    std::vector<float> inv((size_t)hd / 2);
+    for (int i = 0; i < hd / 2; i++) inv[(size_t)i] = (float)std::pow((double)cfg->rope_theta, -2.0 * (double)i / (double)hd);
+    hipError_t e = hipMemcpyAsync(m->inv_freq, inv.data(), inv.size() * 4, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(m->state, 0, 4 * sizeof(int), ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) { free_all(m); delete m; return hip_fail(ctx, e, "llama_create init"); }
+    *out = m;
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_destroy(rt_hip_ctx *ctx, rt_hip_llama *m) {
+    if (!m) return RT_HIP_OK;
+    if (!ctx) return fail(nullptr, RT_HIP_ERR_INVALID_ARG, "ctx is NULL");
+    Guard g(ctx);
+    (void)hipStreamSynchronize(ctx->stream);
+    free_all(m);
+    delete m;
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_upload_tensor(rt_hip_ctx *ctx, rt_hip_llama *m, int slot, int layer, int ggml_type, size_t n_rows,
+                               size_t n_cols, const void *raw, size_t nbytes) {
+    if (!ctx || !m || !raw) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_upload_tensor: NULL argument");
+    const rt_hip_llama_config &c = m->cfg;
+    size_t H = (size_t)c.hidden, F = (size_t)c.ffn, V = (size_t)c.vocab;
+    bool per_layer = slot >= RT_LLAMA_ATTN_Q;
+    if (per_layer) RT_REQUIRE(ctx, layer >= 0 && layer < c.n_layers, RT_HIP_ERR_INVALID_ARG, "layer %d outside 0..%d", layer, c.n_layers - 1);
+    bool is_norm = slot == RT_LLAMA_OUTPUT_NORM || slot == RT_LLAMA_ATTN_NORM || slot == RT_LLAMA_FFN_NORM;
+    size_t er = 0, ec = 0;
+    switch (slot) {
+    case RT_LLAMA_TOK_EMBD: case RT_LLAMA_OUTPUT: er = V; ec = H; break;
+    case RT_LLAMA_ATTN_Q: case RT_LLAMA_ATTN_K: case RT_LLAMA_ATTN_V: case RT_LLAMA_ATTN_OUT: er = H; ec = H; break;
+    case RT_LLAMA_FFN_GATE: case RT_LLAMA_FFN_UP: er = F; ec = H; break;
+    case RT_LLAMA_FFN_DOWN: er = H; ec = F; break;
+    case RT_LLAMA_OUTPUT_NORM: case RT_LLAMA_ATTN_NORM: case RT_LLAMA_FFN_NORM: er = 1; ec = H; break;
+    default: return fail(ctx, RT_HIP_ERR_INVALID_ARG, "unknown tensor slot %d", slot);
+    }
+    if (is_norm) {
+        RT_REQUIRE(ctx, ggml_type == RT_GGML_F32, RT_HIP_ERR_UNSUPPORTED_TYPE, "norm weights must be F32 (got type id %d)", ggml_type);
+        RT_REQUIRE(ctx, n_rows * n_cols == H && nbytes == H * 4, RT_HIP_ERR_SHAPE, "norm weight has %zu x %zu elements / %zu bytes, expected %zu floats",
+                   n_rows, n_cols, nbytes, H);
+    } else {
+        RT_REQUIRE(ctx, n_rows == er && n_cols == ec, RT_HIP_ERR_SHAPE, "slot %d expects %zu x %zu, got %zu x %zu", slot, er, ec, n_rows, n_cols);
+        size_t be = rt::type_block_elems(ggml_type), bb = rt::type_block_bytes(ggml_type);
+        RT_REQUIRE(ctx, be != 0, RT_HIP_ERR_UNSUPPORTED_TYPE, "unsupported GGML type id %d", ggml_type);
+        if (slot != RT_LLAMA_TOK_EMBD)
+            RT_REQUIRE(ctx, gemv_type_ok(ggml_type), RT_HIP_ERR_UNSUPPORTED_TYPE, "GGML type id %d has no GEMV kernel", ggml_type);
+        RT_REQUIRE(ctx, n_cols % be == 0 && nbytes == n_rows * (n_cols / be) * bb, RT_HIP_ERR_SHAPE, "payload of %zu bytes does not match %zu x %zu of type %d",
+                   nbytes, n_rows, n_cols, ggml_type);
+    }
+    Guard g(ctx);
+    void *dev = nullptr;
+    int rc = dev_alloc(ctx, m, &dev, nbytes + 64);
+    if (rc) return rc;
+    RT_TRY_HIP(ctx, hipMemcpyAsync(dev, raw, nbytes, hipMemcpyHostToDevice, ctx->stream));
+    RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (is_norm) {
+        float *f = (float *)dev;
+        if (slot == RT_LLAMA_OUTPUT_NORM) m->out_norm = f;
+        else if (slot == RT_LLAMA_ATTN_NORM) m->attn_norm[(size_t)layer] = f;
+        else m->ffn_norm[(size_t)layer] = f;
+        return RT_HIP_OK;
+    }
+    rt_hip_llama::T t;
+    t.type = ggml_type; t.n_rows = n_rows; t.n_cols = n_cols; t.nbytes = nbytes;
+    t.row_bytes = n_cols / rt::type_block_elems(ggml_type) * rt::type_block_bytes(ggml_type);
+    t.dev = (uint8_t *)dev;
+    size_t l = (size_t)(layer < 0 ? 0 : layer);
+    switch (slot) {
+    case RT_LLAMA_TOK_EMBD: m->tok_embd = t; break;
+    case RT_LLAMA_OUTPUT: m->output = t; break;
+    case RT_LLAMA_ATTN_Q: m->wq[l] = t; break;
+    case RT_LLAMA_ATTN_K: m->wk[l] = t; break;
+    case RT_LLAMA_ATTN_V: m->wv[l] = t; break;
+    case RT_LLAMA_ATTN_OUT: m->wo[l] = t; break;
+    case RT_LLAMA_FFN_GATE: m->wgate[l] = t; break;
+    case RT_LLAMA_FFN_UP: m->wup[l] = t; break;
+    case RT_LLAMA_FFN_DOWN: m->wdown[l] = t; break;
+    }
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_reset(rt_hip_ctx *ctx, rt_hip_llama *m) {
+    if (!ctx || !m) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_reset: NULL argument");
+    Guard g(ctx);
+    m->n_fed = 0;
+    return RT_HIP_OK;
+}
+
+static int set_state(rt_hip_ctx *ctx, rt_hip_llama *m, int pos, int token) {
+    RT_TRY_HIP(ctx, rt::launch_set_int(ctx->stream, m->state + 0, pos));
+    RT_TRY_HIP(ctx, rt::launch_set_int(ctx->stream, m->state + 1, token));
+    RT_TRY_HIP(ctx, rt::launch_set_int(ctx->stream, m->state + 3, 0));
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_step(rt_hip_ctx *ctx, rt_hip_llama *m, int token, int pos, int *next_token) {
+    if (!ctx || !m) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_step: NULL argument");
+    RT_REQUIRE(ctx, token >= 0 && token < m->cfg.vocab, RT_HIP_ERR_INVALID_ARG, "token %d outside the vocabulary of %d", token, m->cfg.vocab);
+    RT_REQUIRE(ctx, pos == m->n_fed, RT_HIP_ERR_INVALID_ARG, "pos=%d but %d tokens have been fed", pos, m->n_fed);
+    RT_REQUIRE(ctx, pos < m->cfg.max_pos, RT_HIP_ERR_SHAPE, "pos=%d reaches max_pos=%d", pos, m->cfg.max_pos);
+    int rc = check_complete(ctx, m);
+    if (rc) return rc;
+    Guard g(ctx);
+    rc = set_state(ctx, m, pos, token);
+    if (rc) return rc;
+    rc = enqueue_step(ctx, m, true);
+    if (rc) return rc;
+    RT_TRY_HIP(ctx, rt::launch_argmax(ctx->stream, m->logits, (size_t)m->cfg.vocab, m->state + 2));
+    m->n_fed = pos + 1;
+    if (next_token) {
+        RT_TRY_HIP(ctx, hipMemcpyAsync(next_token, m->state + 2, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+        RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    }
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_prefill(rt_hip_ctx *ctx, rt_hip_llama *m, const int *tokens, int n_tok, int pos0) {
+    if (!ctx || !m || !tokens) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_prefill: NULL argument");
+    RT_REQUIRE(ctx, n_tok > 0, RT_HIP_ERR_SHAPE, "prefill of %d tokens", n_tok);
+    RT_REQUIRE(ctx, pos0 == m->n_fed, RT_HIP_ERR_INVALID_ARG, "pos0=%d but %d tokens have been fed", pos0, m->n_fed);
+    RT_REQUIRE(ctx, pos0 + n_tok <= m->cfg.max_pos, RT_HIP_ERR_SHAPE, "pos0+n_tok=%d exceeds max_pos=%d", pos0 + n_tok, m->cfg.max_pos);
+    for (int i = 0; i < n_tok; i++)
+        RT_REQUIRE(ctx, tokens[i] >= 0 && tokens[i] < m->cfg.vocab, RT_HIP_ERR_INVALID_ARG, "token %d (index %d) outside the vocabulary", tokens[i], i);
+    int rc = check_complete(ctx, m);
+    if (rc) return rc;
+    Guard g(ctx);
+    for (int i = 0; i < n_tok; i++) {
+        rc = set_state(ctx, m, pos0 + i, tokens[i]);
+        if (rc) return rc;
+        rc = enqueue_step(ctx, m, i == n_tok - 1);
+        if (rc) return rc;
+    }
+    m->n_fed = pos0 + n_tok;
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_logits(rt_hip_ctx *ctx, rt_hip_llama *m, float *logits_host) {
+    if (!ctx || !m || !logits_host) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_logits: NULL argument");
+    Guard g(ctx);
+    RT_TRY_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
+    RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_decode(rt_hip_ctx *ctx, rt_hip_llama *m, int first_token, int pos0, int n_steps, const int *forced,
+                        int *out_tokens) {
+    if (!ctx || !m || !out_tokens) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_decode: NULL argument");
+    RT_REQUIRE(ctx, n_steps > 0, RT_HIP_ERR_SHAPE, "decode of %d steps", n_steps);
+    RT_REQUIRE(ctx, first_token >= 0 && first_token < m->cfg.vocab, RT_HIP_ERR_INVALID_ARG, "token %d outside the vocabulary", first_token);
+    RT_REQUIRE(ctx, pos0 == m->n_fed, RT_HIP_ERR_INVALID_ARG, "pos0=%d but %d tokens have been fed", pos0, m->n_fed);
+    RT_REQUIRE(ctx, pos0 + n_steps <= m->cfg.max_pos, RT_HIP_ERR_SHAPE, "pos0+n_steps=%d exceeds max_pos=%d", pos0 + n_steps, m->cfg.max_pos);
+    if (forced)
+        for (int i = 0; i < n_steps; i++)
+            RT_REQUIRE(ctx, forced[i] >= 0 && forced[i] < m->cfg.vocab, RT_HIP_ERR_INVALID_ARG, "forced token %d (index %d) outside the vocabulary", forced[i], i);
+    int rc = check_complete(ctx, m);
+    if (rc) return rc;
+    Guard g(ctx);
+    if (forced) RT_TRY_HIP(ctx, hipMemcpyAsync(m->forced_dev, forced, (size_t)n_steps * sizeof(int), hipMemcpyHostToDevice, ctx->stream));
+    rc = set_state(ctx, m, pos0, first_token);
+    if (rc) return rc;
+    for (int i = 0; i < n_steps; i++) {
+        rc = enqueue_step(ctx, m, true);
+        if (rc) return rc;
+        RT_TRY_HIP(ctx, rt::launch_argmax(ctx->stream, m->logits, (size_t)m->cfg.vocab, m->state + 2));
+        RT_TRY_HIP(ctx, rt::launch_step_advance(ctx->stream, m->state + 0, m->state + 1, m->state + 2, forced ? m->forced_dev : nullptr,
+                                                m->out_tokens_dev, m->state + 3));
+    }
+    m->n_fed = pos0 + n_steps;
+    RT_TRY_HIP(ctx, hipMemcpyAsync(out_tokens, m->out_tokens_dev, (size_t)n_steps * sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+    RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return RT_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,145 @@
+"""Independent NumPy decoders / encoders of the four GGML block formats.
+
+Written from the element's point of view (which byte and which bits hold
+element e), not as the grouped loops the C oracle uses, so an indexing mistake
+in one is unlikely to be repeated in the other.  float16 -> float32 goes
+through numpy's own IEEE conversion.  All arithmetic is float32, one rounding
+per operation, in the order of the block definitions.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+F32 = np.float32
+
+
+def _f16(b: np.ndarray, off: int) -> np.float32:
+    return np.frombuffer(bytes(b[off:off + 2]), dtype="<f2")[0].astype(F32)
+
+
+# ------------------------------------------------------------------ decode
+
+def decode_q8_0(blk: np.ndarray) -> np.ndarray:
+    d = _f16(blk, 0)
+    q = blk[2:34].view(np.int8).astype(F32)
+    return (d * q).astype(F32)
+
+
+def decode_q4_0(blk: np.ndarray) -> np.ndarray:
+    d = _f16(blk, 0)
+    out = np.empty(32, dtype=F32)
+    for e in range(32):
+        byte = int(blk[2 + (e % 16)])
+        nib = (byte >> 4) if e >= 16 else (byte & 15)
+        out[e] = F32(nib - 8) * d
+    return out
+
+
+def q4k_scale_min(scales: np.ndarray, j: int):
+    s = [int(v) for v in scales]
+    if j < 4:
+        return s[j] & 63, s[j + 4] & 63
+    return (s[j + 4] & 15) | ((s[j - 4] >> 6) << 4), (s[j + 4] >> 4) | ((s[j] >> 6) << 4)
+
+
+def decode_q4_k(blk: np.ndarray) -> np.ndarray:
+    d, dmin = _f16(blk, 0), _f16(blk, 2)
+    out = np.empty(256, dtype=F32)
+    for e in range(256):
+        j = e // 32
+        sc, mn = q4k_scale_min(blk[4:16], j)
+        byte = int(blk[16 + 32 * (j // 2) + e % 32])
+        nib = (byte >> 4) if (j % 2) else (byte & 15)
+        dd = F32(d * F32(sc))
+        mm = F32(dmin * F32(mn))
+        out[e] = F32(F32(dd * F32(nib)) - mm)
+    return out
+
+
+def decode_q6_k(blk: np.ndarray) -> np.ndarray:
+    d = _f16(blk, 208)
+    sc = blk[192:208].view(np.int8)
+    out = np.empty(256, dtype=F32)
+    for e in range(256):
+        half, rem = divmod(e, 128)
+        run, l = divmod(rem, 32)          # run 0..3 of 32 elements inside the half
+        lo_byte = int(blk[64 * half + l + 32 * (run % 2)])
+        nib = (lo_byte >> 4) if run >= 2 else (lo_byte & 15)
+        hi2 = (int(blk[128 + 32 * half + l]) >> (2 * run)) & 3
+        q = (nib | (hi2 << 4)) - 32
+        s = int(sc[8 * half + 2 * run + l // 16])
+        out[e] = F32(F32(d * F32(s)) * F32(q))
+    return out
+
+
+DECODERS = {8: (34, 32, decode_q8_0), 2: (18, 32, decode_q4_0), 12: (144, 256, decode_q4_k), 14: (210, 256, decode_q6_k)}
+
+
+def decode(ggml_type: int, raw: np.ndarray) -> np.ndarray:
+    bb, be, fn = DECODERS[int(ggml_type)]
+    raw = np.ascontiguousarray(raw).view(np.uint8).reshape(-1, bb)
+    return np.concatenate([fn(b) for b in raw])
+
+
+# ------------------------------------------------------------------ encode
+
+def _put_f16(blk: np.ndarray, off: int, v) -> None:
+    blk[off:off + 2] = np.frombuffer(np.float16(v).tobytes(), dtype=np.uint8)
+
+
+def encode_q8_0(d, q) -> np.ndarray:
+    blk = np.zeros(34, dtype=np.uint8)
+    _put_f16(blk, 0, d)
+    blk[2:] = np.asarray(q, dtype=np.int8).view(np.uint8)
+    return blk
+
+
+def encode_q4_0(d, q) -> np.ndarray:
+    """q: 32 values in 0..15 (stored value; the decoded element is (q - 8) * d)."""
+    blk = np.zeros(18, dtype=np.uint8)
+    _put_f16(blk, 0, d)
+    q = np.asarray(q, dtype=np.uint8)
+    blk[2:] = q[:16] | (q[16:] << 4)
+    return blk
+
+
+def pack_q4k_scales(sc, mn) -> np.ndarray:
+    """8 six-bit scales and 8 six-bit mins into 12 bytes."""
+    out = np.zeros(12, dtype=np.uint8)
+    for j in range(8):
+        s, m = int(sc[j]), int(mn[j])
+        if j < 4:
+            out[j] |= s
+            out[j + 4] |= m
+        else:
+            out[j + 4] |= (s & 15) | ((m & 15) << 4)
+            out[j - 4] |= (s >> 4) << 6
+            out[j] |= (m >> 4) << 6
+    return out
+
+
+def encode_q4_k(d, dmin, sc, mn, q) -> np.ndarray:
+    """q: 256 values in 0..15."""
+    blk = np.zeros(144, dtype=np.uint8)
+    _put_f16(blk, 0, d)
+    _put_f16(blk, 2, dmin)
+    blk[4:16] = pack_q4k_scales(sc, mn)
+    q = np.asarray(q, dtype=np.uint8).reshape(4, 2, 32)
+    blk[16:] = (q[:, 0, :] | (q[:, 1, :] << 4)).reshape(-1)
+    return blk
+
+
+def encode_q6_k(d, sc, q) -> np.ndarray:
+    """q: 256 stored values in 0..63 (decoded element is d * sc * (q - 32)); sc: 16 int8."""
+    blk = np.zeros(210, dtype=np.uint8)
+    q = np.asarray(q, dtype=np.uint8)
+    for e in range(256):
+        half, rem = divmod(e, 128)
+        run, l = divmod(rem, 32)
+        v = int(q[e])
+        lo_i = 64 * half + l + 32 * (run % 2)
+        blk[lo_i] |= ((v & 15) << 4) if run >= 2 else (v & 15)
+        blk[128 + 32 * half + l] |= (v >> 4) << (2 * run)
+    blk[192:208] = np.asarray(sc, dtype=np.int8).view(np.uint8)
+    _put_f16(blk, 208, d)
+    return blk

@@ -1,0 +1,76 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/rustorch_hip.h declares."""
+import ctypes as C
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "rustorch_hip.h"
+
+
+def header_symbols():
+    text = HEADER.read_text()
+    return re.findall(r"RT_HIP_API\s+[\w\s\*]+?\b(rt_\w+)\s*\(", text)
+
+
+def test_header_symbols_are_exported_and_bound(lib):
+    from rustorch_amd import _lib
+    syms = header_symbols()
+    assert len(syms) >= 40 and len(set(syms)) == len(syms)
+    for s in syms:
+        assert hasattr(lib, s), "missing export %s" % s
+    assert sorted(syms) == sorted(_lib.SIGNATURES), "ctypes table and header disagree"
+
+
+def test_static_archive_holds_the_same_entry_points(lib):
+    import subprocess
+    a = ROOT / "rustorch_amd" / "librustorch_hip.a"
+    if not a.exists():
+        pytest.skip("static archive not built")
+    out = subprocess.run(["nm", "-g", "--defined-only", str(a)], stdout=subprocess.PIPE, text=True).stdout
+    defined = set(re.findall(r"\bT (rt_\w+)", out))
+    assert set(header_symbols()) <= defined
+
+
+def test_type_table_matches_reference_type_size(lib):
+    # example-cli/src/model/formats/gguf.rs:78-99,125-144
+    from rustorch_amd import GGMLType
+    for t, size, elems in ((0, 4, 1), (1, 2, 1), (2, 18, 32), (8, 34, 32), (12, 144, 256), (14, 210, 256)):
+        assert lib.rt_hip_type_block_bytes(t) == size and lib.rt_hip_type_block_elems(t) == elems
+        assert GGMLType(t).type_size() == size and GGMLType(t).block_elems() == elems
+    assert lib.rt_hip_type_block_bytes(3) == 0 and lib.rt_hip_type_block_bytes(99) == 0   # no kernel: reported, not guessed
+    # the reference's own unit tests: ids 0,1,2 and the unknown-id error (gguf.rs:414-426)
+    assert GGMLType.from_u32(0) is GGMLType.F32 and GGMLType.from_u32(1) is GGMLType.F16 and GGMLType.from_u32(2) is GGMLType.Q4_0
+    with pytest.raises(ValueError, match="Unknown GGML type"):
+        GGMLType.from_u32(999)
+    assert (GGMLType.F32.type_size(), GGMLType.F16.type_size(), GGMLType.I8.type_size()) == (4, 2, 1)
+    assert GGMLType.Q4_K.row_bytes(4096) == 2304 and GGMLType.Q6_K.row_bytes(11008) == 9030
+    with pytest.raises(ValueError):
+        GGMLType.Q4_K.row_bytes(1000)
+
+
+def test_null_and_missing_device_are_errors_not_crashes(lib):
+    from rustorch_amd import _lib, DeviceNotAvailable, InvalidParameters
+    from rustorch_amd.executor import HipKernelExecutor, device_count
+    assert lib.rt_hip_create(0, None) == 1
+    assert lib.rt_hip_synchronize(None) == 1
+    assert lib.rt_hip_destroy(None) == 0 and lib.rt_hip_qweight_free(None, None) == 0
+    ctx = C.c_void_p()
+    assert lib.rt_hip_create(4096, C.byref(ctx)) == 3 and not ctx.value
+    assert b"hip:4096" in lib.rt_hip_last_error(None)
+    with pytest.raises(DeviceNotAvailable):
+        HipKernelExecutor(4096)
+    with pytest.raises(InvalidParameters):
+        _lib.check(lib.rt_hip_malloc(None, 16, None))
+    if device_count() == 0:
+        with pytest.raises(DeviceNotAvailable):   # no silent CPU fallback
+            HipKernelExecutor(0)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from rustorch_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(ImportError, match="no CPU fallback"):
+        _lib.load()

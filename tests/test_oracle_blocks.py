@@ -1,0 +1,169 @@
+"""Pins the oracle's block decoders without the reference (which holds none):
+closed forms, exhaustive packer round trips, an independent NumPy decoder and
+committed golden vectors."""
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import np_blocks as nb
+
+GOLDEN = Path(__file__).resolve().parent / "golden" / "blocks_golden.npz"
+TYPES = [8, 2, 12, 14]
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def test_fp16_to_f32_exhaustive(orc):
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([orc.h2f(int(v)) for v in h], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(bits(got)[~nan], bits(want)[~nan])
+    assert np.all(np.isnan(got[nan]))
+
+
+def test_f32_to_fp16_rne(orc):
+    rng = np.random.default_rng(7)
+    vals = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-8, 5, 20000).astype(np.float32),
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e-8, 5.96e-8, 2.98e-8, 2.9802322e-8, 6.1e-5, 6.0975e-5, np.inf, -np.inf,
+                  1.0009765625, 1.00048828125, 1.00146484375], dtype=np.float32),
+        np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)[::7],
+    ]).astype(np.float32)
+    vals = vals[~np.isnan(vals)]
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([orc.f2h(float(v)) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    # halfway cases between consecutive fp16 values round to even
+    h = np.arange(0x3C00, 0x3C40, dtype=np.uint16)
+    lo, hi = h.view(np.float16).astype(np.float64), (h + 1).view(np.float16).astype(np.float64)
+    mid = ((lo + hi) / 2).astype(np.float32)
+    got = np.array([orc.f2h(float(v)) for v in mid], dtype=np.uint16)
+    assert np.array_equal(got, np.where(h % 2 == 0, h, h + 1))
+
+
+def test_block_geometry_matches_reference_type_size(orc):
+    # example-cli/src/model/formats/gguf.rs:125-144
+    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 8, 12, 14)] == [4, 2, 18, 34, 144, 210]
+    assert [orc.load().orc_block_elems(t) for t in (2, 8, 12, 14)] == [32, 32, 256, 256]
+    assert orc.load().orc_row_bytes(12, 4096) == 2304 and orc.load().orc_row_bytes(14, 11008) == 9030
+    assert orc.load().orc_row_bytes(12, 100) == 0
+
+
+def test_q8_0_closed_forms(orc):
+    q = np.arange(-16, 16)
+    y = orc.dequant(8, nb.encode_q8_0(1.0, q), 1, 32)[0]
+    assert np.array_equal(y, q.astype(np.float32))
+    y = orc.dequant(8, nb.encode_q8_0(2.0 ** -7, q), 1, 32)[0]
+    assert np.array_equal(y, q.astype(np.float32) / 128)
+    # all 256 byte values
+    allq = np.arange(256, dtype=np.uint8).view(np.int8)
+    for d in (0.5, 0.0123, 3.0):
+        raw = np.concatenate([nb.encode_q8_0(d, allq[i:i + 32]) for i in range(0, 256, 32)])
+        y = orc.dequant(8, raw, 1, 256)[0]
+        assert np.array_equal(bits(y), bits(np.float16(d).astype(np.float32) * allq.astype(np.float32)))
+
+
+def test_reference_affine_dequant_kat(orc):
+    # src/quantization/types.rs:431-443 / operations.rs:604-619: [10,20,30,40] * 0.1 = [1,2,3,4]
+    # one Q8_0 block is that affine map with zero_point 0; the scale is rounded to fp16 by the format
+    q = np.zeros(32, dtype=np.int8); q[:4] = [10, 20, 30, 40]
+    y = orc.dequant(8, nb.encode_q8_0(0.1, q), 1, 32)[0]
+    assert np.allclose(y[:4], [1, 2, 3, 4], rtol=2.5e-4) and np.all(y[4:] == 0)
+    y = orc.dequant(8, nb.encode_q8_0(0.125, q), 1, 32)[0]
+    assert np.array_equal(y[:4], np.array([1.25, 2.5, 3.75, 5.0], dtype=np.float32))
+
+
+def test_q4_0_nibble_order_and_offset(orc):
+    # element j < 16 is the LOW nibble of byte j, element 16 + j the HIGH nibble; stored value 8 decodes to 0
+    q = np.concatenate([np.arange(16), 15 - np.arange(16)]).astype(np.uint8)
+    y = orc.dequant(2, nb.encode_q4_0(1.0, q), 1, 32)[0]
+    assert np.array_equal(y, q.astype(np.float32) - 8)
+    blk = np.zeros(18, dtype=np.uint8); blk[0:2] = np.frombuffer(np.float16(2.0).tobytes(), np.uint8)
+    blk[2 + 3] = 0xA1   # low nibble 1 -> element 3, high nibble 10 -> element 19
+    y = orc.dequant(2, blk, 1, 32)[0]
+    want = np.full(32, -16.0, dtype=np.float32); want[3] = (1 - 8) * 2; want[19] = (10 - 8) * 2
+    assert np.array_equal(y, want)
+
+
+def test_q4_k_scale_packer_exhaustive(orc):
+    # every 6-bit (scale, min) pair at every sub-block position survives pack -> decode
+    d, dmin = np.float32(np.float16(0.5)), np.float32(np.float16(0.25))
+    ones = np.ones(256, dtype=np.uint8)
+    blocks, want = [], []
+    for j in range(8):
+        for s in range(64):
+            sc = np.zeros(8, dtype=np.uint8); mn = np.zeros(8, dtype=np.uint8)
+            sc[j] = s; mn[j] = 63 - s
+            # neighbours carry the complementary pattern so a bit leaking across fields is seen
+            sc[(j + 4) % 8] = 63 - s; mn[(j + 4) % 8] = s
+            blocks.append(nb.encode_q4_k(0.5, 0.25, sc, mn, ones))
+            w = np.zeros(256, dtype=np.float32)
+            for jj in range(8):
+                w[32 * jj:32 * jj + 32] = d * np.float32(sc[jj]) * 1 - dmin * np.float32(mn[jj])
+            want.append(w)
+    raw = np.concatenate(blocks)
+    y = orc.dequant(12, raw, len(blocks), 256)
+    assert np.array_equal(y, np.stack(want))
+    # and the full 64 x 64 grid at one low and one high sub-block
+    blocks, want = [], []
+    for j in (1, 6):
+        for s in range(64):
+            for m in range(0, 64, 1):
+                sc = np.zeros(8, dtype=np.uint8); mn = np.zeros(8, dtype=np.uint8)
+                sc[j] = s; mn[j] = m
+                blocks.append(nb.encode_q4_k(0.5, 0.25, sc, mn, ones))
+                want.append((j, s, m))
+    y = orc.dequant(12, np.concatenate(blocks), len(blocks), 256)
+    for row, (j, s, m) in zip(y, want):
+        assert row[32 * j] == d * s - dmin * m and row[(32 * j + 40) % 256] == 0
+
+
+def test_q4_k_nibbles_and_positions(orc):
+    # one-hot quants: value v at element e, everything else 0; scale 1 at e's sub-block only
+    for e in (0, 31, 32, 63, 64, 100, 127, 128, 191, 192, 255):
+        for v in range(16):
+            q = np.zeros(256, dtype=np.uint8); q[e] = v
+            sc = np.zeros(8, dtype=np.uint8); sc[e // 32] = 2
+            y = orc.dequant(12, nb.encode_q4_k(1.0, 1.0, sc, np.zeros(8, np.uint8), q), 1, 256)[0]
+            want = np.zeros(256, dtype=np.float32); want[e] = 2 * v
+            assert np.array_equal(y, want), (e, v)
+
+
+def test_q6_k_all_values_all_positions(orc):
+    for e in (0, 15, 16, 31, 32, 47, 64, 95, 96, 127, 128, 143, 160, 200, 224, 255):
+        for v in range(64):
+            q = np.full(256, 32, dtype=np.uint8); q[e] = v   # stored 32 decodes to 0
+            sc = np.zeros(16, dtype=np.int8); sc[e // 16] = -3
+            y = orc.dequant(14, nb.encode_q6_k(0.5, sc, q), 1, 256)[0]
+            want = np.zeros(256, dtype=np.float32); want[e] = 0.5 * -3 * (v - 32)
+            assert np.array_equal(y, want), (e, v)
+    # every scale slot addresses its own 16 elements, sign included
+    for s in range(16):
+        sc = np.zeros(16, dtype=np.int8); sc[s] = -128 if s % 2 else 127
+        y = orc.dequant(14, nb.encode_q6_k(1.0, sc, np.full(256, 33, np.uint8)), 1, 256)[0]
+        want = np.zeros(256, dtype=np.float32); want[16 * s:16 * s + 16] = sc[s]
+        assert np.array_equal(y, want)
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_golden_vectors(orc, t):
+    g = np.load(GOLDEN)
+    raw, val = g["raw_%d" % t], g["val_%d" % t]
+    got = orc.dequant(t, raw, raw.shape[0], val.shape[1])
+    assert np.array_equal(bits(got), bits(val))
+    # the fixture itself is reproducible from the independent decoder
+    assert np.array_equal(bits(nb.decode(t, raw).reshape(val.shape)), bits(val))
+
+
+@pytest.mark.parametrize("t", TYPES)
+def test_oracle_equals_numpy_decoder_on_synthetic_blocks(orc, lib, t):
+    from rustorch_amd import synth
+    be = 32 if t in (8, 2) else 256
+    raw = synth.blocks(t, 11, 3, 6, 2 * be)
+    got = orc.dequant(t, raw, 6, 2 * be)
+    assert np.array_equal(bits(got.reshape(-1)), bits(nb.decode(t, raw)))
