@@ -1,0 +1,188 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF quantized decode hot path on one MI355X.
+
+Headline workload (config.workload = "C3"): the seven projections of one Llama-7B decoder layer at
+batch 1 -- q, k, o (4096x4096), gate, up (11008x4096) in Q4_K and v (4096x4096), down (4096x11008) in
+Q6_K -- 129 785 856 weight bytes per layer.  One "step" is one pass over one layer: quantize the seven
+activation vectors, then the seven dequant-fused GEMVs in one grouped launch.  Steps rotate through 32
+distinct synthetic layers (4.15 GB), so weights come from HBM and not from the 256 MB Infinity Cache.
+`value` is weight GB/s = weight bytes per step / wall time per step (inputs resident in HBM).
+
+Also reported on the same JSON line:
+  roofline      the GEMV kernel alone: algorithmic bytes per launch / mean launch duration (HIP events
+                around back-to-back launches on the library's stream) against the 8 TB/s HBM peak
+  decode        the 32-layer, 7B-shaped greedy decode loop (config C5): tokens/s after a 128-token prompt
+  cpu_baseline  the oracle's restatement of the reference CPU path (dequantize the whole tensor to f32,
+                then naive row-dot with sequential k accumulation) timed on this host for one layer
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK = 8.0e12
+SEED = 20250127
+H, F, V, NH, NL = 4096, 11008, 32000, 32, 32
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def layer_bytes_algorithmic(specs):
+    """weights once + f32 x + f32 y per projection."""
+    w = sum(t.row_bytes(c) * r for _, t, r, c in specs)
+    io = sum(4 * c + 4 * r for _, _, r, c in specs)
+    return w, w + io
+
+
+def bench_layer_gemv(ex, steps, warmup, n_layers):
+    from rustorch_amd import synth
+    specs = synth.layer_tensor_specs(H, F)
+    wbytes, abytes = layer_bytes_algorithmic(specs)
+    layers = []
+    t0 = time.time()
+    for l in range(n_layers):
+        ws = [ex.upload_qweight(t, r, c, synth.blocks(t, SEED, synth.layer_tid(l, slot), r, c)) for slot, t, r, c in specs]
+        layers.append(ws)
+    log("[bench] %d layers (%.2f GB) generated and uploaded in %.1f s" % (n_layers, n_layers * wbytes / 1e9, time.time() - t0))
+    xs = [ex.to_device(synth.normal(SEED, 1000 + i, c)) for i, (_, _, _, c) in enumerate(specs)]
+    xqs = [ex.buffer(ex.xq_bytes(c)) for _, _, _, c in specs]
+    ys = [ex.buffer(4 * r) for _, _, r, _ in specs]
+    ncols = [c for _, _, _, c in specs]
+
+    def step(i):
+        ex.quantize_act_dev(xs, ncols, xqs)
+        ex.qgemv_xq_grouped_dev(layers[i % n_layers], xqs, ys)
+
+    for i in range(warmup):
+        step(i)
+    ex.synchronize()
+    e0, e1 = ex.event(), ex.event()
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        step(warmup + i)
+    e1.record()
+    ex.synchronize()
+    wall = time.perf_counter() - t0
+    ev_ms = e0.elapsed_ms(e1)
+    # kernel-only region: the grouped GEMV launch alone, back to back
+    ex.quantize_act_dev(xs, ncols, xqs)
+    ex.synchronize()
+    k0, k1 = ex.event(), ex.event()
+    k0.record()
+    for i in range(steps):
+        ex.qgemv_xq_grouped_dev(layers[(warmup + i) % n_layers], xqs, ys)
+    k1.record()
+    ex.synchronize()
+    kern_ms = k0.elapsed_ms(k1) / steps
+    for ws in layers:
+        for w in ws:
+            w.free()
+    return dict(wbytes=wbytes, abytes=abytes, wall_s=wall, event_ms=ev_ms, kernel_ms=kern_ms)
+
+
+def bench_decode(ex, n_prompt, n_gen):
+    from rustorch_amd import llama, synth
+    t0 = time.time()
+    gm = llama.HipLlama(ex, NL, H, NH, F, V, n_prompt + n_gen)
+    wbytes = llama.load_synthetic(gm, SEED)
+    log("[bench] 7B-shaped model (%.2f GB of blocks) generated and uploaded in %.1f s" % (wbytes / 1e9, time.time() - t0))
+    prompt = synth.tokens(SEED, synth.TID_PROMPT, n_prompt, V)
+    t0 = time.perf_counter()
+    gm.prefill(prompt[:-1], 0)
+    ex.synchronize()
+    t_prefill = time.perf_counter() - t0
+    # warm-up step, then rewind so the timed loop starts right after the prompt
+    t0 = time.perf_counter()
+    toks = gm.decode(int(prompt[-1]), n_prompt - 1, n_gen)
+    t_dec = time.perf_counter() - t0
+    gm.close()
+    per_layer = synth.layer_weight_bytes(H, F)
+    tok_bytes = NL * per_layer + 210 * (H // 256) * V       # weights streamed per token (output head is Q6_K)
+    kv_avg = 2 * NL * H * 2 * (n_prompt + n_gen / 2)           # fp16 K and V rows read per token, averaged over the run
+    return dict(tokens_per_s=n_gen / t_dec, ms_per_token=1e3 * t_dec / n_gen, prefill_tokens_per_s=(n_prompt - 1) / t_prefill,
+                bytes_per_token=int(tok_bytes + kv_avg), hbm_frac=(tok_bytes + kv_avg) * n_gen / t_dec / HBM_PEAK,
+                n_prompt=n_prompt, n_generated=n_gen, first_tokens=[int(t) for t in toks[:8]])
+
+
+def cpu_baseline(reps):
+    """Reference CPU path for one layer: dequantize each tensor to dense f32, then x . W^T with sequential k-sums."""
+    from oracle import oracle as orc
+    from rustorch_amd import synth
+    specs = synth.layer_tensor_specs(H, F)
+    wbytes, _ = layer_bytes_algorithmic(specs)
+    tensors = [(t, r, c, synth.blocks(t, SEED, synth.layer_tid(0, slot), r, c), synth.normal(SEED, 1000 + i, c))
+               for i, (slot, t, r, c) in enumerate(specs)]
+    ncores = orc.num_threads()
+    best = {}
+    for threads in (1, ncores):
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            for t, r, c, raw, x in tensors:
+                W = orc.dequant(t, raw, r, c, threads)
+                orc.matmul_xwt(x, W, threads)
+            ts.append(time.perf_counter() - t0)
+        best[threads] = min(ts)
+    return wbytes, best[1], best[ncores], ncores
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=320)
+    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--layers", type=int, default=32, help="distinct synthetic layers rotated through (32 = 4.15 GB)")
+    ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--decode-prompt", type=int, default=128)
+    ap.add_argument("--decode-gen", type=int, default=128)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (use --gpus 1)" % args.gpus)
+
+    from rustorch_amd.executor import HipKernelExecutor
+    ex = HipKernelExecutor(0)
+    info = ex.device_info()
+    log("[bench] device:", info)
+
+    g = bench_layer_gemv(ex, args.steps, args.warmup, args.layers)
+    ms_per_step = 1e3 * g["wall_s"] / args.steps
+    value = g["wbytes"] / (g["wall_s"] / args.steps) / 1e9
+    achieved = g["abytes"] / (g["kernel_ms"] * 1e-3) / 1e9
+    out = {
+        "metric": "Q4_K/Q6_K GEMV weight GB/s, one Llama-7B decoder layer at batch 1 (plus decode tokens/s), 1xMI355X",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "q4_K/q6_K blocks x int16 block-scaled activations (int8 dot4, f32 accumulate)", "data": "synthetic",
+        "config": {"workload": "C3: seven projections of one Llama-7B decoder layer, batch 1, q/k/o/gate/up Q4_K, v/down Q6_K",
+                   "weight_bytes_per_step": g["wbytes"], "layers_rotated": args.layers, "hbm_frac_of_value": round(value * 1e9 / HBM_PEAK, 4),
+                   "event_ms_per_step": round(g["event_ms"] / args.steps, 5)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": None, "kernel": "qgemv_kernel",
+                     "bytes_per_launch": g["abytes"], "avg_launch_ms": round(g["kernel_ms"], 5)},
+    }
+    if not args.no_decode:
+        out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen)
+    ex.close()
+    if not args.no_cpu:
+        wbytes, t1, tn, ncores = cpu_baseline(3)
+        out["cpu_baseline"] = {"value": round(wbytes / t1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": "one of the 32 layers (seven projections, batch 1): dequantize to dense f32, then naive x.W^T; best of 3",
+                               "all_cores_value": round(wbytes / tn / 1e9, 4), "all_cores": ncores}
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

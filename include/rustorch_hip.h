@@ -130,6 +130,15 @@ RT_HIP_API int rt_hip_qgemv_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const 
 /* n independent GEMVs (batch 1 each) in one launch: ws[i], xs_dev[i] (n_cols_i floats), ys_dev[i] (n_rows_i floats). */
 RT_HIP_API int rt_hip_qgemv_grouped_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const *ws,
                                         const float *const *xs_dev, float *const *ys_dev);
+/* The two halves of rt_hip_qgemv_grouped_dev, for callers that keep activations in the kernels' own
+ * quantized form (16-bit block-scaled integers split into two int8 planes, see rt_hip_xq_bytes):
+ * quantize n vectors of n_cols[i] floats (each a multiple of 32) into xqs_dev[i] (rt_hip_xq_bytes(n_cols[i]) bytes,
+ * 16-byte aligned), then run the n GEMVs on them in one launch. */
+RT_HIP_API size_t rt_hip_xq_bytes(size_t n_cols);
+RT_HIP_API int rt_hip_quantize_act_dev(rt_hip_ctx *ctx, int n, const float *const *xs_dev, const size_t *n_cols,
+                                       void *const *xqs_dev);
+RT_HIP_API int rt_hip_qgemv_xq_grouped_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const *ws,
+                                           const void *const *xqs_dev, float *const *ys_dev);
 /* Y[M, n_rows] = X[M, n_cols] . dequant(W)^T for prefill (any M >= 1; MFMA path for M >= 16). */
 RT_HIP_API int rt_hip_qgemm(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *X, size_t M, float *Y);
 RT_HIP_API int rt_hip_qgemm_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *X_dev, size_t M,

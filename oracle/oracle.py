@@ -35,6 +35,7 @@ def load() -> C.CDLL:
         "orc_f2h": (C.c_uint16, [C.c_float]),
         "orc_block_elems": (i, [i]), "orc_block_bytes": (i, [i]), "orc_row_bytes": (sz, [i, sz]),
         "orc_dequant": (i, [i, vp, sz, sz, vp]),
+        "orc_dequant_nt": (i, [i, vp, sz, sz, vp, i]),
         "orc_matmul_xwt": (None, [vp, vp, vp, sz, sz, sz, i]),
         "orc_qgemv": (i, [i, vp, sz, sz, vp, sz, vp, i]),
         "orc_qgemm": (i, [i, vp, sz, sz, vp, sz, vp, i]),
@@ -76,10 +77,14 @@ def f2h(x: float) -> int:
     return int(load().orc_f2h(float(x)))
 
 
-def dequant(ggml_type: int, raw, n_rows: int, n_cols: int) -> np.ndarray:
+def num_threads() -> int:
+    return int(load().orc_num_threads())
+
+
+def dequant(ggml_type: int, raw, n_rows: int, n_cols: int, nthreads: int = 0) -> np.ndarray:
     raw = _raw(raw)
     out = np.empty((n_rows, n_cols), dtype=np.float32)
-    if load().orc_dequant(int(ggml_type), _p(raw), n_rows, n_cols, _p(out)) != 0:
+    if load().orc_dequant_nt(int(ggml_type), _p(raw), n_rows, n_cols, _p(out), nthreads or num_threads()) != 0:
         raise ValueError("oracle: bad type/shape")
     return out
 
@@ -89,7 +94,7 @@ def matmul_xwt(x: np.ndarray, w: np.ndarray, nthreads: int = 0) -> np.ndarray:
     x = np.ascontiguousarray(x, dtype=np.float32); w = np.ascontiguousarray(w, dtype=np.float32)
     x2 = x.reshape(1, -1) if x.ndim == 1 else x
     y = np.empty((x2.shape[0], w.shape[0]), dtype=np.float32)
-    load().orc_matmul_xwt(_p(x2), _p(w), _p(y), x2.shape[0], w.shape[0], w.shape[1], nthreads)
+    load().orc_matmul_xwt(_p(x2), _p(w), _p(y), x2.shape[0], w.shape[0], w.shape[1], nthreads or num_threads())
     return y[0] if x.ndim == 1 else y
 
 
@@ -98,7 +103,7 @@ def qgemv(ggml_type: int, raw, n_rows: int, n_cols: int, x: np.ndarray, nthreads
     x = np.ascontiguousarray(x, dtype=np.float32)
     x2 = x.reshape(1, -1) if x.ndim == 1 else x
     y = np.empty((x2.shape[0], n_rows), dtype=np.float32)
-    if load().orc_qgemm(int(ggml_type), _p(raw), n_rows, n_cols, _p(x2), x2.shape[0], _p(y), nthreads) != 0:
+    if load().orc_qgemm(int(ggml_type), _p(raw), n_rows, n_cols, _p(x2), x2.shape[0], _p(y), nthreads or num_threads()) != 0:
         raise ValueError("oracle: bad type/shape")
     return y[0] if x.ndim == 1 else y
 
@@ -110,7 +115,7 @@ def qgemv_f64(ggml_type: int, raw, n_rows: int, n_cols: int, x: np.ndarray, nthr
     x2 = x.reshape(1, -1) if x.ndim == 1 else x
     y = np.empty((x2.shape[0], n_rows), dtype=np.float64)
     wn = np.empty(n_rows, dtype=np.float64)
-    if load().orc_qgemv_f64(int(ggml_type), _p(raw), n_rows, n_cols, _p(x2), x2.shape[0], _p(y), _p(wn), nthreads) != 0:
+    if load().orc_qgemv_f64(int(ggml_type), _p(raw), n_rows, n_cols, _p(x2), x2.shape[0], _p(y), _p(wn), nthreads or num_threads()) != 0:
         raise ValueError("oracle: bad type/shape")
     return (y[0] if x.ndim == 1 else y), wn
 
@@ -171,7 +176,7 @@ class OracleLlama:
     def __init__(self, n_layers, hidden, n_heads, ffn, vocab, max_pos, eps=1e-5, theta=10000.0, nthreads=0):
         self.vocab = vocab
         self.keep = []
-        self.h = C.c_void_p(load().orc_llama_create(n_layers, hidden, n_heads, ffn, vocab, max_pos, eps, theta, nthreads))
+        self.h = C.c_void_p(load().orc_llama_create(n_layers, hidden, n_heads, ffn, vocab, max_pos, eps, theta, nthreads or num_threads()))
 
     def set_tensor(self, slot, layer, ggml_type, n_rows, n_cols, raw):
         raw = np.ascontiguousarray(raw)

@@ -212,13 +212,20 @@ ORC_API size_t orc_row_bytes(int type, size_t n_cols) {
 }
 
 /* Whole tensor to dense f32 (tensor_loader.rs:41-67 with real block decode).  Returns 0, or -1 on a bad type / shape. */
-ORC_API int orc_dequant(int type, const void *raw, size_t n_rows, size_t n_cols, float *out) {
+ORC_API int orc_dequant_nt(int type, const void *raw, size_t n_rows, size_t n_cols, float *out, int nthreads) {
     size_t rb = orc_row_bytes(type, n_cols);
     if (rb == 0) return -1;
     const uint8_t *p = (const uint8_t *)raw;
+#ifdef _OPENMP
+    if (nthreads > 0) omp_set_num_threads(nthreads);
+#endif
 #pragma omp parallel for schedule(static)
     for (long r = 0; r < (long)n_rows; r++) deq_row(type, p + rb * (size_t)r, n_cols, out + n_cols * (size_t)r);
     return 0;
+}
+
+ORC_API int orc_dequant(int type, const void *raw, size_t n_rows, size_t n_cols, float *out) {
+    return orc_dequant_nt(type, raw, n_rows, n_cols, out, 0);
 }
 
 /* ------------------------------------------------------ dense x . W^T */
@@ -568,9 +575,10 @@ ORC_API int orc_llama_forward(orc_llama *m, const int *tokens, int n_tok, int po
     return 0;
 }
 
+/* Hardware threads OpenMP would use by default (not affected by earlier nthreads arguments). */
 ORC_API int orc_num_threads(void) {
 #ifdef _OPENMP
-    return omp_get_max_threads();
+    return omp_get_num_procs();
 #else
     return 1;
 #endif

@@ -397,16 +397,62 @@ int rt_hip_qgemv_grouped_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const
     int rc = ensure_scratch(ctx, need);
     if (rc) return rc;
     rt::GemvArgs a;
+    rt::QuantGroupArgs qa;
     memset(&a, 0, sizeof a);
+    memset(&qa, 0, sizeof qa);
     a.n = n;
+    qa.n = n;
     uint8_t *xq = (uint8_t *)ctx->scratch;
     for (int i = 0; i < n; i++) {
         const rt_hip_qweight *w = ws[i];
-        RT_TRY_HIP(ctx, rt::launch_quantize_x(ctx->stream, xs_dev[i], xq, w->n_cols, 1));
+        qa.x[i] = xs_dev[i]; qa.xq[i] = xq; qa.K[i] = (int)w->n_cols;
         a.p[i].w = w->dev; a.p[i].xq = xq; a.p[i].y = ys_dev[i]; a.p[i].res = nullptr; a.p[i].row_bytes = w->row_bytes;
         a.p[i].type = w->type; a.p[i].N = (int)w->n_rows; a.p[i].K = (int)w->n_cols;
         xq += rt::xq_stride(w->n_cols);
     }
+    RT_TRY_HIP(ctx, rt::launch_quantize_group(ctx->stream, qa));
+    RT_TRY_HIP(ctx, rt::launch_qgemv(ctx->stream, a, 1));
+    return RT_HIP_OK;
+}
+
+size_t rt_hip_xq_bytes(size_t n_cols) { return rt::xq_stride(n_cols); }
+
+int rt_hip_quantize_act_dev(rt_hip_ctx *ctx, int n, const float *const *xs_dev, const size_t *n_cols, void *const *xqs_dev) {
+    if (!ctx || !xs_dev || !n_cols || !xqs_dev) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_quantize_act_dev: NULL argument");
+    RT_REQUIRE(ctx, n >= 1 && n <= rt::kMaxGemvProbs, RT_HIP_ERR_INVALID_ARG, "quantize_act takes 1..%d vectors, got %d", rt::kMaxGemvProbs, n);
+    rt::QuantGroupArgs qa;
+    memset(&qa, 0, sizeof qa);
+    qa.n = n;
+    for (int i = 0; i < n; i++) {
+        RT_REQUIRE(ctx, xs_dev[i] && xqs_dev[i], RT_HIP_ERR_INVALID_ARG, "quantize_act: vector %d has a NULL pointer", i);
+        RT_REQUIRE(ctx, n_cols[i] > 0 && n_cols[i] % 32 == 0 && n_cols[i] < ((size_t)1 << 24), RT_HIP_ERR_SHAPE,
+                   "quantize_act: n_cols[%d]=%zu is not a positive multiple of 32", i, n_cols[i]);
+        RT_REQUIRE(ctx, ((uintptr_t)xqs_dev[i] & 15) == 0 && ((uintptr_t)xs_dev[i] & 15) == 0, RT_HIP_ERR_INVALID_ARG,
+                   "quantize_act: vector %d is not 16-byte aligned", i);
+        qa.x[i] = xs_dev[i]; qa.xq[i] = (uint8_t *)xqs_dev[i]; qa.K[i] = (int)n_cols[i];
+    }
+    Guard g(ctx);
+    RT_TRY_HIP(ctx, rt::launch_quantize_group(ctx->stream, qa));
+    return RT_HIP_OK;
+}
+
+int rt_hip_qgemv_xq_grouped_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const *ws, const void *const *xqs_dev,
+                                float *const *ys_dev) {
+    if (!ctx || !ws || !xqs_dev || !ys_dev) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_qgemv_xq_grouped_dev: NULL argument");
+    RT_REQUIRE(ctx, n >= 1 && n <= rt::kMaxGemvProbs, RT_HIP_ERR_INVALID_ARG, "grouped GEMV takes 1..%d problems, got %d", rt::kMaxGemvProbs, n);
+    rt::GemvArgs a;
+    memset(&a, 0, sizeof a);
+    a.n = n;
+    for (int i = 0; i < n; i++) {
+        if (!ws[i] || !xqs_dev[i] || !ys_dev[i]) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "grouped GEMV: problem %d has a NULL member", i);
+        int rc = qgemv_check(ctx, ws[i], 1);
+        if (rc) return rc;
+        RT_REQUIRE(ctx, ((uintptr_t)xqs_dev[i] & 15) == 0, RT_HIP_ERR_INVALID_ARG, "grouped GEMV: xq %d is not 16-byte aligned", i);
+        const rt_hip_qweight *w = ws[i];
+        a.p[i].w = w->dev; a.p[i].xq = (const uint8_t *)xqs_dev[i]; a.p[i].y = ys_dev[i]; a.p[i].res = nullptr;
+        a.p[i].row_bytes = w->row_bytes; a.p[i].type = w->type; a.p[i].N = (int)w->n_rows; a.p[i].K = (int)w->n_cols;
+    }
+    Guard g(ctx);
     RT_TRY_HIP(ctx, rt::launch_qgemv(ctx->stream, a, 1));
     return RT_HIP_OK;
 }

@@ -48,10 +48,16 @@ struct GemvArgs {
     int n;
 };
 
-struct Llama;  // defined in rt_llama.hip
+struct QuantGroupArgs {
+    const float *x[kMaxGemvProbs];
+    uint8_t *xq[kMaxGemvProbs];
+    int K[kMaxGemvProbs];
+    int n;
+};
 
 // ---- launchers (all enqueue on `s`, return hipError_t of the launch)
 hipError_t launch_quantize_x(hipStream_t s, const float *x, uint8_t *xq, size_t K, size_t batch);
+hipError_t launch_quantize_group(hipStream_t s, const QuantGroupArgs &a);
 hipError_t launch_qgemv(hipStream_t s, GemvArgs &args, int batch);  // fills tile0 / rows_per_tile
 hipError_t launch_dequant(hipStream_t s, int type, const uint8_t *w, size_t n_rows, size_t n_cols, float *out);
 hipError_t launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *y, uint8_t *xq, size_t rows,

@@ -174,6 +174,16 @@ __global__ __launch_bounds__(256) void quantize_x_kernel(const float *x, uint8_t
     quantize_store4(v, i4 * 4, xq + m * xq_stride(K), K);
 }
 
+// Several independent vectors in one launch (grid.y = vector index).
+__global__ __launch_bounds__(256) void quantize_group_kernel(QuantGroupArgs a) {
+    int p = blockIdx.y;
+    size_t K = (size_t)a.K[p];
+    size_t i4 = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i4 * 4 >= K) return;
+    float4 v = reinterpret_cast<const float4 *>(a.x[p])[i4];
+    quantize_store4(v, i4 * 4, a.xq[p], K);
+}
+
 // ------------------------------------------------------------ GEMV unit dots
 // A "unit" is the slice of one weight row a lane consumes in one go.  x lives in LDS in
 // xq form: xh / xl as dwords of 4 int8, xs per 32-block, xb per 16-run.
@@ -578,6 +588,15 @@ __global__ __launch_bounds__(1024) void matmul_f32_kernel(const float *a, const 
 hipError_t launch_quantize_x(hipStream_t s, const float *x, uint8_t *xq, size_t K, size_t batch) {
     dim3 grid((unsigned)((K / 4 + 255) / 256), (unsigned)batch);
     quantize_x_kernel<<<grid, 256, 0, s>>>(x, xq, K);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_group(hipStream_t s, const QuantGroupArgs &a) {
+    size_t maxK = 0;
+    for (int i = 0; i < a.n; i++) maxK = (size_t)a.K[i] > maxK ? (size_t)a.K[i] : maxK;
+    if (a.n == 0 || maxK == 0) return hipSuccess;
+    dim3 grid((unsigned)((maxK / 4 + 255) / 256), (unsigned)a.n);
+    quantize_group_kernel<<<grid, 256, 0, s>>>(a);
     return hipGetLastError();
 }
 

@@ -237,6 +237,21 @@ class HipKernelExecutor:
         wa = arr(*[w.handle for w in ws]); xa = arr(*[x.ptr for x in xs]); ya = arr(*[y.ptr for y in ys])
         _lib.check(self.lib.rt_hip_qgemv_grouped_dev(self.ctx, n, wa, xa, ya), self.ctx)
 
+    def xq_bytes(self, n_cols: int) -> int:
+        return int(self.lib.rt_hip_xq_bytes(n_cols))
+
+    def quantize_act_dev(self, xs: Sequence[DeviceBuffer], n_cols: Sequence[int], xqs: Sequence[DeviceBuffer]) -> None:
+        n = len(xs)
+        arr = C.c_void_p * n
+        xa = arr(*[x.ptr for x in xs]); qa = arr(*[q.ptr for q in xqs]); ka = (C.c_size_t * n)(*n_cols)
+        _lib.check(self.lib.rt_hip_quantize_act_dev(self.ctx, n, xa, ka, qa), self.ctx)
+
+    def qgemv_xq_grouped_dev(self, ws: Sequence[QWeight], xqs: Sequence[DeviceBuffer], ys: Sequence[DeviceBuffer]) -> None:
+        n = len(ws)
+        arr = C.c_void_p * n
+        wa = arr(*[w.handle for w in ws]); qa = arr(*[q.ptr for q in xqs]); ya = arr(*[y.ptr for y in ys])
+        _lib.check(self.lib.rt_hip_qgemv_xq_grouped_dev(self.ctx, n, wa, qa, ya), self.ctx)
+
     # -- decode-step operators (host arrays in, host arrays out; each call goes through device buffers)
     def rmsnorm(self, x, gamma, eps: float) -> np.ndarray:
         x = _f32(x, "x"); gamma = _f32(gamma, "gamma")
