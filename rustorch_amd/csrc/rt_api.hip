@@ -331,14 +331,12 @@ int rt_hip_dequant(rt_hip_ctx *ctx, const rt_hip_qweight *w, float *out_host) {
     return RT_HIP_OK;
 }
 
-// Enqueue quantize(x) + GEMV for one weight; xq lives at `xq` (device, batch * xq_stride(K) bytes).
-static int enqueue_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x_dev, float *y_dev, int batch,
-                         uint8_t *xq) {
-    RT_TRY_HIP(ctx, rt::launch_quantize_x(ctx->stream, x_dev, xq, w->n_cols, (size_t)batch));
+// Enqueue the GEMV for one weight; x is quantized by the kernel while it is staged into LDS.
+static int enqueue_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x_dev, float *y_dev, int batch) {
     rt::GemvArgs a;
     memset(&a, 0, sizeof a);
     a.n = 1;
-    a.p[0].w = w->dev; a.p[0].xq = xq; a.p[0].y = y_dev; a.p[0].res = nullptr; a.p[0].row_bytes = w->row_bytes;
+    a.p[0].w = w->dev; a.p[0].x = x_dev; a.p[0].stage = rt::kStageF32; a.p[0].y = y_dev; a.p[0].row_bytes = w->row_bytes;
     a.p[0].type = w->type; a.p[0].N = (int)w->n_rows; a.p[0].K = (int)w->n_cols;
     RT_TRY_HIP(ctx, rt::launch_qgemv(ctx->stream, a, batch));
     return RT_HIP_OK;
@@ -356,10 +354,9 @@ int rt_hip_qgemv_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x_de
     if (!ctx || !w || !x_dev || !y_dev) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_qgemv_dev: NULL argument");
     int rc = qgemv_check(ctx, w, batch);
     if (rc) return rc;
+    RT_REQUIRE(ctx, ((uintptr_t)x_dev & 15) == 0, RT_HIP_ERR_INVALID_ARG, "qgemv: x must be 16-byte aligned");
     Guard g(ctx);
-    rc = ensure_scratch(ctx, (size_t)batch * rt::xq_stride(w->n_cols));
-    if (rc) return rc;
-    return enqueue_qgemv(ctx, w, x_dev, y_dev, batch, (uint8_t *)ctx->scratch);
+    return enqueue_qgemv(ctx, w, x_dev, y_dev, batch);
 }
 
 int rt_hip_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x, float *y, int batch) {
@@ -368,13 +365,12 @@ int rt_hip_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x, float
     if (rc) return rc;
     Guard g(ctx);
     size_t xb = align_up((size_t)batch * w->n_cols * 4, 256), yb = align_up((size_t)batch * w->n_rows * 4, 256);
-    size_t qb = (size_t)batch * rt::xq_stride(w->n_cols);
-    rc = ensure_scratch(ctx, xb + yb + qb);
+    rc = ensure_scratch(ctx, xb + yb);
     if (rc) return rc;
     char *base = (char *)ctx->scratch;
     float *dx = (float *)base, *dy = (float *)(base + xb);
     RT_TRY_HIP(ctx, hipMemcpyAsync(dx, x, (size_t)batch * w->n_cols * 4, hipMemcpyHostToDevice, ctx->stream));
-    rc = enqueue_qgemv(ctx, w, dx, dy, batch, (uint8_t *)(base + xb + yb));
+    rc = enqueue_qgemv(ctx, w, dx, dy, batch);
     if (rc) return rc;
     RT_TRY_HIP(ctx, hipMemcpyAsync(y, dy, (size_t)batch * w->n_rows * 4, hipMemcpyDeviceToHost, ctx->stream));
     RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -386,31 +382,19 @@ int rt_hip_qgemv_grouped_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const
     if (!ctx || !ws || !xs_dev || !ys_dev) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_qgemv_grouped_dev: NULL argument");
     RT_REQUIRE(ctx, n >= 1 && n <= rt::kMaxGemvProbs, RT_HIP_ERR_INVALID_ARG, "grouped GEMV takes 1..%d problems, got %d",
                rt::kMaxGemvProbs, n);
-    size_t need = 0;
+    rt::GemvArgs a;
+    memset(&a, 0, sizeof a);
+    a.n = n;
     for (int i = 0; i < n; i++) {
         if (!ws[i] || !xs_dev[i] || !ys_dev[i]) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "grouped GEMV: problem %d has a NULL member", i);
         int rc = qgemv_check(ctx, ws[i], 1);
         if (rc) return rc;
-        need += rt::xq_stride(ws[i]->n_cols);
+        RT_REQUIRE(ctx, ((uintptr_t)xs_dev[i] & 15) == 0, RT_HIP_ERR_INVALID_ARG, "grouped GEMV: x %d is not 16-byte aligned", i);
+        const rt_hip_qweight *w = ws[i];
+        a.p[i].w = w->dev; a.p[i].x = xs_dev[i]; a.p[i].stage = rt::kStageF32; a.p[i].y = ys_dev[i]; a.p[i].row_bytes = w->row_bytes;
+        a.p[i].type = w->type; a.p[i].N = (int)w->n_rows; a.p[i].K = (int)w->n_cols;
     }
     Guard g(ctx);
-    int rc = ensure_scratch(ctx, need);
-    if (rc) return rc;
-    rt::GemvArgs a;
-    rt::QuantGroupArgs qa;
-    memset(&a, 0, sizeof a);
-    memset(&qa, 0, sizeof qa);
-    a.n = n;
-    qa.n = n;
-    uint8_t *xq = (uint8_t *)ctx->scratch;
-    for (int i = 0; i < n; i++) {
-        const rt_hip_qweight *w = ws[i];
-        qa.x[i] = xs_dev[i]; qa.xq[i] = xq; qa.K[i] = (int)w->n_cols;
-        a.p[i].w = w->dev; a.p[i].xq = xq; a.p[i].y = ys_dev[i]; a.p[i].res = nullptr; a.p[i].row_bytes = w->row_bytes;
-        a.p[i].type = w->type; a.p[i].N = (int)w->n_rows; a.p[i].K = (int)w->n_cols;
-        xq += rt::xq_stride(w->n_cols);
-    }
-    RT_TRY_HIP(ctx, rt::launch_quantize_group(ctx->stream, qa));
     RT_TRY_HIP(ctx, rt::launch_qgemv(ctx->stream, a, 1));
     return RT_HIP_OK;
 }
@@ -449,7 +433,7 @@ int rt_hip_qgemv_xq_grouped_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *co
         if (rc) return rc;
         RT_REQUIRE(ctx, ((uintptr_t)xqs_dev[i] & 15) == 0, RT_HIP_ERR_INVALID_ARG, "grouped GEMV: xq %d is not 16-byte aligned", i);
         const rt_hip_qweight *w = ws[i];
-        a.p[i].w = w->dev; a.p[i].xq = (const uint8_t *)xqs_dev[i]; a.p[i].y = ys_dev[i]; a.p[i].res = nullptr;
+        a.p[i].w = w->dev; a.p[i].x = xqs_dev[i]; a.p[i].y = ys_dev[i]; a.p[i].res = nullptr;
         a.p[i].row_bytes = w->row_bytes; a.p[i].type = w->type; a.p[i].N = (int)w->n_rows; a.p[i].K = (int)w->n_cols;
     }
     Guard g(ctx);
@@ -531,7 +515,8 @@ int rt_hip_attn_decode_dev(rt_hip_ctx *ctx, const float *q, const uint16_t *kcac
     RT_REQUIRE(ctx, head_dim == 64 || head_dim == 128, RT_HIP_ERR_SHAPE, "attn_decode: head_dim=%d (64 or 128 supported)", head_dim);
     RT_REQUIRE(ctx, n_heads > 0 && n_pos > 0 && n_pos <= 16000, RT_HIP_ERR_SHAPE, "attn_decode: n_heads=%d n_pos=%d", n_heads, n_pos);
     Guard g(ctx);
-    RT_TRY_HIP(ctx, rt::launch_attn_decode(ctx->stream, q, kcache, vcache, nullptr, n_pos, n_heads, head_dim, out, nullptr));
+    RT_TRY_HIP(ctx, rt::launch_attn_decode(ctx->stream, const_cast<float *>(q), nullptr, nullptr, const_cast<uint16_t *>(kcache),
+                                           const_cast<uint16_t *>(vcache), nullptr, n_pos, n_heads, head_dim, nullptr, out, nullptr, false));
     return RT_HIP_OK;
 }
 

@@ -1,0 +1,129 @@
+// Device-side helpers shared by the kernel translation units (gfx950, wave64).
+#pragma once
+
+#include "rt_internal.h"
+
+#include <hip/hip_fp16.h>
+
+namespace rt {
+
+
+__device__ __forceinline__ float h2f(uint32_t bits16) {
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)bits16);
+}
+__device__ __forceinline__ uint16_t f2h_rne(float f) {
+    return __builtin_bit_cast(unsigned short, (_Float16)f);
+}
+
+// Loads through a byte pointer with no alignment promise (Q6_K / Q8_0 / Q4_0 blocks are only 2-byte aligned).
+__device__ __forceinline__ uint4 ld16u(const uint8_t *p) { uint4 v; __builtin_memcpy(&v, p, 16); return v; }
+__device__ __forceinline__ uint2 ld8u(const uint8_t *p) { uint2 v; __builtin_memcpy(&v, p, 8); return v; }
+__device__ __forceinline__ uint32_t ld4u(const uint8_t *p) { uint32_t v; __builtin_memcpy(&v, p, 4); return v; }
+__device__ __forceinline__ uint32_t ld2u(const uint8_t *p) { unsigned short v; __builtin_memcpy(&v, p, 2); return v; }
+__device__ __forceinline__ uint4 ld16a(const uint8_t *p) { return *reinterpret_cast<const uint4 *>(p); }
+
+__device__ __forceinline__ int sdot4(uint32_t a, int b, int c) { return __builtin_amdgcn_sdot4((int)a, b, c, false); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Block-wide sum / max through LDS (red must hold blockDim/64 floats). All threads get the result.
+__device__ __forceinline__ float block_sum(float v, float *red) {
+    v = wave_sum(v);
+    int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; i++) t += red[i];
+    return t;
+}
+__device__ __forceinline__ float block_max(float v, float *red) {
+    v = wave_max(v);
+    int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float t = red[0];
+    for (int i = 1; i < nw; i++) t = fmaxf(t, red[i]);
+    return t;
+}
+
+
+// Activation accesses that must be coherent across XCDs inside one launch (COH) go out as device-scope
+// relaxed atomics, which bypass the per-XCD L2; otherwise they are plain cached accesses.
+template <bool COH> __device__ __forceinline__ float ld_f(const float *p) {
+    if (COH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return *p;
+}
+template <bool COH> __device__ __forceinline__ void st_f(float *p, float v) {
+    if (COH) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+template <bool COH> __device__ __forceinline__ float4 ld_f4(const float *p) {  // p is 16-byte aligned
+    if (COH) {
+        const unsigned long long *q = reinterpret_cast<const unsigned long long *>(p);
+        unsigned long long a = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned long long b = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return make_float4(__uint_as_float((unsigned)a), __uint_as_float((unsigned)(a >> 32)), __uint_as_float((unsigned)b),
+                           __uint_as_float((unsigned)(b >> 32)));
+    }
+    return *reinterpret_cast<const float4 *>(p);
+}
+
+// Sum over the 64 lanes of a wave with DPP row operations (no LDS traffic); every lane must be active.
+// The total is returned to all lanes.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+    int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, true);
+    return v + __int_as_float(r);
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v = dpp_add<0xB1, 0xF>(v);    // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xF>(v);    // quad_perm [2,3,0,1]
+    v = dpp_add<0x141, 0xF>(v);   // row_half_mirror
+    v = dpp_add<0x140, 0xF>(v);   // row_mirror: every lane of a 16-lane row holds the row sum
+    v = dpp_add<0x142, 0xA>(v);   // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xC>(v);   // row_bcast:31 into rows 2 and 3: lane 63 holds the total
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+// The 4-element quantization step shared by every producer of the xq form: returns the packed high / low
+// int8 planes, the block scale and the sum of the 16-element run the lane belongs to.
+struct Q4Pack {
+    uint32_t hi, lo;
+    float s;
+    int sum16, sum32;
+};
+__device__ __forceinline__ Q4Pack quantize4(float4 v) {
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    float inv = amax > 0.f ? 16383.0f / amax : 0.f;
+    Q4Pack r;
+    r.s = amax / 16383.0f;
+    int q0 = max(-16383, min(16383, __float2int_rn(v.x * inv)));
+    int q1 = max(-16383, min(16383, __float2int_rn(v.y * inv)));
+    int q2 = max(-16383, min(16383, __float2int_rn(v.z * inv)));
+    int q3 = max(-16383, min(16383, __float2int_rn(v.w * inv)));
+    r.hi = ((uint32_t)(q0 >> 7) & 0xFF) | (((uint32_t)(q1 >> 7) & 0xFF) << 8) | (((uint32_t)(q2 >> 7) & 0xFF) << 16) |
+           (((uint32_t)(q3 >> 7) & 0xFF) << 24);
+    r.lo = (uint32_t)(q0 & 127) | ((uint32_t)(q1 & 127) << 8) | ((uint32_t)(q2 & 127) << 16) | ((uint32_t)(q3 & 127) << 24);
+    int sum = q0 + q1 + q2 + q3;
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    r.sum16 = sum;
+    r.sum32 = sum + __shfl_xor(sum, 4, 64);
+    return r;
+}
+
+}  // namespace rt

@@ -1,0 +1,64 @@
+// Stand-alone dequant-fused GEMV launch (decode, batch 1..8): y = dequant(W) . x with W in raw GGUF blocks.
+// One workgroup of 1024 threads per CU; device code in rt_gemv_device.h.
+#include "rt_gemv_device.h"
+
+namespace rt {
+
+namespace {
+
+constexpr int kGemvThreads = 1024;
+constexpr int kGemvWaves = kGemvThreads / 64;
+
+__global__ __launch_bounds__(kGemvThreads) void qgemv_kernel(GemvArgs a, int r2) {
+    extern __shared__ uint4 lds4[];
+    __shared__ float red[kGemvWaves];
+    uint32_t *lds = reinterpret_cast<uint32_t *>(lds4);
+    const int wg = blockIdx.x;
+    int pi = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxGemvProbs; i++)
+        if (i < a.n && wg >= a.p[i].tile0) pi = i;
+    const GemvProb &P = a.p[pi];
+    gemv_dispatch<false>(P, wg - P.tile0, P.rows_per_tile, blockIdx.y, r2 != 0, lds, red);
+}
+
+}  // namespace
+
+// Gives every problem a share of the workgroups in proportion to its weight bytes (tile0 = first workgroup,
+// rows_per_tile = number of workgroups of the problem) and launches one grid over all of them
+// (grid.y = batch row).  Workgroups of a problem stage x once and deal its rows out round-robin.
+hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
+    if (a.n <= 0 || a.n > kMaxGemvProbs || batch <= 0) return hipErrorInvalidValue;
+    double total_bytes = 0;
+    size_t maxK = 0, total_rows = 0;
+    for (int i = 0; i < a.n; i++) {
+        total_bytes += (double)a.p[i].N * (double)a.p[i].row_bytes * (a.p[i].epi == kEpiSwiglu ? 2.0 : 1.0);
+        total_rows += (size_t)a.p[i].N;
+        if ((size_t)a.p[i].K > maxK) maxK = (size_t)a.p[i].K;
+    }
+    if (total_bytes <= 0) return hipErrorInvalidValue;
+    // one resident workgroup (16 waves) per CU over 256 CUs
+    int budget = 256 / batch;
+    if (budget < a.n) budget = a.n;
+    // two rows per wave step once every wave has at least three steps of work, else one
+    const int r2 = total_rows >= (size_t)3 * 2 * (size_t)budget * kGemvWaves ? 1 : 0;
+    int wgs = 0;
+    for (int i = 0; i < a.n; i++) {
+        const GemvProb &p = a.p[i];
+        double bytes = (double)p.N * (double)p.row_bytes * (p.epi == kEpiSwiglu ? 2.0 : 1.0);
+        int n = (int)(budget * (bytes / total_bytes) + 0.5);
+        int rows_per_group = (p.epi == kEpiSwiglu) ? 1 : (r2 ? 2 : 1);
+        int max_useful = ((p.N + rows_per_group - 1) / rows_per_group + kGemvWaves - 1) / kGemvWaves;
+        if (n > max_useful) n = max_useful;
+        if (n < 1) n = 1;
+        a.p[i].tile0 = wgs;
+        a.p[i].rows_per_tile = n;
+        wgs += n;
+    }
+    size_t lds = xq_stride(maxK);
+    dim3 grid((unsigned)wgs, (unsigned)batch);
+    qgemv_kernel<<<grid, kGemvThreads, lds, s>>>(a, r2);
+    return hipGetLastError();
+}
+
+}  // namespace rt

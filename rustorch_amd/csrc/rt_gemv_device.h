@@ -1,0 +1,411 @@
+// Device side of the dequant-fused GEMV (decode): shared by the stand-alone kernel and the persistent
+// decode-step kernel.
+//
+// The computation is HBM-bound: every weight byte is read once with 16-byte loads and consumed by integer
+// dot products (v_dot4_i32_i8) against the activation vector held in LDS as two int8 planes (16-bit
+// block-scaled integers, see rt_internal.h).
+//
+// Work split: the workgroups that share a problem deal its rows out round-robin, one "row group" (R rows)
+// per wave at a time; the 64 lanes of a wave stride the row's "units" (the slice of a row one lane eats:
+// 64 elements of Q4_K / Q6_K, one block of Q8_0 / Q4_0).  The loads of the next step are issued before the
+// current one is consumed, and the first step is requested before x is staged, so weight bytes are in
+// flight while the workgroup waits for its input.  Partial sums are reduced across the wave with DPP.
+//
+// x is staged once per workgroup into LDS, in an order permuted per weight type so that the 16-byte LDS
+// reads of consecutive lanes hit consecutive addresses.  The staging step can also produce x: quantize an
+// f32 vector, or RMS-normalise and quantize it (the norm that precedes q/k/v and gate/up in a decoder
+// layer).  The epilogue can add a residual or combine a gate row and an up row into up * silu(gate)
+// (src/nn/activation.rs:404-414).
+//
+// COH = true makes every access to activations (x, y, res) a device-coherent one, for the persistent kernel
+// where producer and consumer workgroups sit on different XCDs within one launch.
+#pragma once
+
+#include "rt_device.h"
+
+namespace rt {
+
+__device__ __forceinline__ int units_of(int type, int K) {
+    return (type == RT_GGML_Q4_K || type == RT_GGML_Q6_K) ? K / 64 : K / 32;
+}
+
+// dword index inside a plane (xh or xl) of the 4 elements starting at e (e % 4 == 0)
+__device__ __forceinline__ int x_slot_dword(int type, int e, int U) {
+    int j = e >> 4, w = (e >> 2) & 3;
+    int slot;
+    if (type == RT_GGML_Q4_K) slot = (j & 3) * U + (j >> 2);
+    else if (type == RT_GGML_Q6_K) slot = ((j >> 1) & 3) * U + (2 * (j >> 3) + (j & 1));
+    else slot = (j & 1) * U + (j >> 1);
+    return slot * 4 + w;
+}
+
+// Place 4 quantized elements and the block metadata they carry into the per-type LDS layout.
+//   planes: xh at dword 0, xl at dword K/4; floats S from dword K/2:
+//   Q4_K : S[4u + {0,1}] = scale of the unit's two 32-blocks, S[4u + {2,3}] = scale * sum of each block
+//   Q6_K : S[b] = scale of 32-block b (= 4 * half + run);  S[2U + 4u + r] = scale * sum of the unit's run r
+//   Q8_0 : S[u] = scale;   Q4_0 : S[2u] = scale, S[2u+1] = scale * sum of the block
+__device__ __forceinline__ void stage_store(int type, int K, int U, uint32_t *lds, int e, uint32_t hi, uint32_t lo,
+                                            float s, float bsum16, float bsum32) {
+    int d = x_slot_dword(type, e, U);
+    lds[d] = hi;
+    lds[K / 4 + d] = lo;
+    float *S = reinterpret_cast<float *>(lds + K / 2);
+    if (type == RT_GGML_Q4_K) {
+        if ((e & 31) == 0) {
+            int b = e >> 5, u = b >> 1, half = b & 1;
+            S[4 * u + half] = s;
+            S[4 * u + 2 + half] = bsum32;
+        }
+    } else if (type == RT_GGML_Q6_K) {
+        if ((e & 31) == 0) S[e >> 5] = s;
+        if ((e & 15) == 0) {
+            int i16 = e >> 4;
+            int u = 2 * (i16 >> 3) + (i16 & 1), r = (i16 >> 1) & 3;
+            S[2 * U + 4 * u + r] = bsum16;
+        }
+    } else if (type == RT_GGML_Q8_0) {
+        if ((e & 31) == 0) S[e >> 5] = s;
+    } else {
+        if ((e & 31) == 0) {
+            S[2 * (e >> 5)] = s;
+            S[2 * (e >> 5) + 1] = bsum32;
+        }
+    }
+}
+
+template <bool COH>
+__device__ __forceinline__ void stage_x(const GemvProb &P, int m, uint32_t *lds, float *red) {
+    const int K = P.K, U = units_of(P.type, K), type = P.type;
+    const int n4 = K / 4;
+    if (P.stage == kStageXq) {
+        const uint8_t *xq = reinterpret_cast<const uint8_t *>(P.x) + (size_t)m * xq_stride((size_t)K);
+        const uint32_t *qh = reinterpret_cast<const uint32_t *>(xq);
+        const uint32_t *ql = reinterpret_cast<const uint32_t *>(xq + K);
+        const float *xs = reinterpret_cast<const float *>(xq + 2 * (size_t)K);
+        const float *xb = xs + K / 32;
+        for (int i = threadIdx.x; i < n4; i += (int)blockDim.x) {
+            int e = 4 * i;
+            float s = 0.f, b16 = 0.f, b32 = 0.f;
+            if ((e & 15) == 0) {
+                s = xs[e >> 5];
+                b16 = xb[e >> 4];
+                if ((e & 31) == 0) b32 = b16 + xb[(e >> 4) + 1];
+            }
+            stage_store(type, K, U, lds, e, qh[i], ql[i], s, b16, b32);
+        }
+    } else {
+        const float *x = reinterpret_cast<const float *>(P.x) + (size_t)m * K;
+        float rms = 1.f;
+        if (P.stage == kStageRms) {
+            float ss = 0.f;
+            for (int i = threadIdx.x; i < n4; i += (int)blockDim.x) {
+                float4 v = ld_f4<COH>(x + 4 * i);
+                ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            }
+            ss = block_sum(ss, red);
+            rms = sqrtf(ss / (float)K + P.eps);
+        }
+        const float4 *g4 = reinterpret_cast<const float4 *>(P.gamma);
+        // K % 32 == 0 and blockDim.x % 8 == 0: the 8 lanes of a 32-block enter and leave this loop together
+        for (int i = threadIdx.x; i < n4; i += (int)blockDim.x) {
+            float4 v = ld_f4<COH>(x + 4 * i);
+            if (P.stage == kStageRms) {
+                float4 g = g4[i];
+                v = make_float4(g.x * (v.x / rms), g.y * (v.y / rms), g.z * (v.z / rms), g.w * (v.w / rms));
+            }
+            Q4Pack p = quantize4(v);
+            stage_store(type, K, U, lds, 4 * i, p.hi, p.lo, p.s, p.s * (float)p.sum16, p.s * (float)p.sum32);
+        }
+    }
+    __syncthreads();
+}
+
+// ---- per-type register images of one unit of one weight row, of the matching x slice, and their dot ----
+
+template <int TYPE> struct WRegs;
+template <int TYPE> struct XRegs;
+
+template <> struct WRegs<RT_GGML_Q4_K> { uint4 hdr, qa, qb; };
+template <> struct XRegs<RT_GGML_Q4_K> { uint4 h[4], l[4]; float4 sv; };
+template <> struct WRegs<RT_GGML_Q6_K> { uint4 A, B, H; uint2 sc; uint32_t d; };
+template <> struct XRegs<RT_GGML_Q6_K> { uint4 h[4], l[4]; float4 xs, xb; };
+template <> struct WRegs<RT_GGML_Q8_0> { uint4 a, b; uint32_t d; };
+template <> struct XRegs<RT_GGML_Q8_0> { uint4 h[2], l[2]; float s; };
+template <> struct WRegs<RT_GGML_Q4_0> { uint4 a; uint32_t d; };
+template <> struct XRegs<RT_GGML_Q4_0> { uint4 h[2], l[2]; float2 sv; };
+
+// row is wave-uniform; the lane part of the address is a 32-bit offset
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_K> &w, const uint8_t *row, int u) {
+    uint32_t off = (uint32_t)(u >> 2) * 144u, g = (uint32_t)(u & 3);
+    w.hdr = ld16a(row + off);
+    w.qa = ld16a(row + off + 16u + 32u * g);
+    w.qb = ld16a(row + off + 32u + 32u * g);
+}
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q6_K> &w, const uint8_t *row, int u) {
+    uint32_t off = (uint32_t)(u >> 2) * 210u, h = (uint32_t)((u >> 1) & 1), c = (uint32_t)(u & 1);
+    w.A = ld16u(row + off + 64u * h + 16u * c);
+    w.B = ld16u(row + off + 64u * h + 32u + 16u * c);
+    w.H = ld16u(row + off + 128u + 32u * h + 16u * c);
+    w.sc = ld8u(row + off + 192u + 8u * h);
+    w.d = ld2u(row + off + 208u);
+}
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q8_0> &w, const uint8_t *row, int u) {
+    uint32_t off = (uint32_t)u * 34u;
+    w.d = ld2u(row + off);
+    w.a = ld16u(row + off + 2u);
+    w.b = ld16u(row + off + 18u);
+}
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_0> &w, const uint8_t *row, int u) {
+    uint32_t off = (uint32_t)u * 18u;
+    w.d = ld2u(row + off);
+    w.a = ld16u(row + off + 2u);
+}
+
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_K> &x, const uint32_t *lds, int u, int U, int K) {
+    const uint4 *XH = reinterpret_cast<const uint4 *>(lds);
+    const uint4 *XL = XH + K / 16;
+#pragma unroll
+    for (int c = 0; c < 4; c++) { x.h[c] = XH[c * U + u]; x.l[c] = XL[c * U + u]; }
+    x.sv = reinterpret_cast<const float4 *>(lds + K / 2)[u];
+}
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q6_K> &x, const uint32_t *lds, int u, int U, int K) {
+    const uint4 *XH = reinterpret_cast<const uint4 *>(lds);
+    const uint4 *XL = XH + K / 16;
+#pragma unroll
+    for (int r = 0; r < 4; r++) { x.h[r] = XH[r * U + u]; x.l[r] = XL[r * U + u]; }
+    const float *S = reinterpret_cast<const float *>(lds + K / 2);
+    x.xs = reinterpret_cast<const float4 *>(S)[u >> 1];
+    x.xb = reinterpret_cast<const float4 *>(S + 2 * U)[u];
+}
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q8_0> &x, const uint32_t *lds, int u, int U, int K) {
+    const uint4 *XH = reinterpret_cast<const uint4 *>(lds);
+    const uint4 *XL = XH + K / 16;
+    x.h[0] = XH[u]; x.h[1] = XH[U + u]; x.l[0] = XL[u]; x.l[1] = XL[U + u];
+    x.s = reinterpret_cast<const float *>(lds + K / 2)[u];
+}
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_0> &x, const uint32_t *lds, int u, int U, int K) {
+    const uint4 *XH = reinterpret_cast<const uint4 *>(lds);
+    const uint4 *XL = XH + K / 16;
+    x.h[0] = XH[u]; x.h[1] = XH[U + u]; x.l[0] = XL[u]; x.l[1] = XL[U + u];
+    x.sv = reinterpret_cast<const float2 *>(lds + K / 2)[u];
+}
+
+#define RT_W4(v) { (v).x, (v).y, (v).z, (v).w }
+
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_K> &w, const XRegs<RT_GGML_Q4_K> &x, int u) {
+    const int g = u & 3;
+    uint32_t scw, mw;
+    if (g < 2) {
+        scw = w.hdr.y & 0x3f3f3f3fu;
+        mw = w.hdr.z & 0x3f3f3f3fu;
+    } else {
+        scw = (w.hdr.w & 0x0f0f0f0fu) | ((w.hdr.y >> 2) & 0x30303030u);
+        mw = ((w.hdr.w >> 4) & 0x0f0f0f0fu) | ((w.hdr.z >> 2) & 0x30303030u);
+    }
+    const int sh = (g & 1) * 16;
+    scw >>= sh;
+    mw >>= sh;
+    float sc0 = (float)(scw & 0xFF), sc1 = (float)((scw >> 8) & 0xFF);
+    float m0 = (float)(mw & 0xFF), m1 = (float)((mw >> 8) & 0xFF);
+    float d = h2f(w.hdr.x & 0xFFFF), dmin = h2f(w.hdr.x >> 16);
+    const uint32_t q[8] = { w.qa.x, w.qa.y, w.qa.z, w.qa.w, w.qb.x, w.qb.y, w.qb.z, w.qb.w };
+    const uint32_t hlo[8] = { x.h[0].x, x.h[0].y, x.h[0].z, x.h[0].w, x.h[1].x, x.h[1].y, x.h[1].z, x.h[1].w };
+    const uint32_t hhi[8] = { x.h[2].x, x.h[2].y, x.h[2].z, x.h[2].w, x.h[3].x, x.h[3].y, x.h[3].z, x.h[3].w };
+    const uint32_t llo[8] = { x.l[0].x, x.l[0].y, x.l[0].z, x.l[0].w, x.l[1].x, x.l[1].y, x.l[1].z, x.l[1].w };
+    const uint32_t lhi[8] = { x.l[2].x, x.l[2].y, x.l[2].z, x.l[2].w, x.l[3].x, x.l[3].y, x.l[3].z, x.l[3].w };
+    int dh0 = 0, dl0 = 0, dh1 = 0, dl1 = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        uint32_t lo = q[i] & 0x0f0f0f0fu, hi = (q[i] >> 4) & 0x0f0f0f0fu;
+        dh0 = sdot4(lo, (int)hlo[i], dh0);
+        dl0 = sdot4(lo, (int)llo[i], dl0);
+        dh1 = sdot4(hi, (int)hhi[i], dh1);
+        dl1 = sdot4(hi, (int)lhi[i], dl1);
+    }
+    float t0 = (float)((dh0 << 7) + dl0), t1 = (float)((dh1 << 7) + dl1);
+    return d * (sc0 * (x.sv.x * t0) + sc1 * (x.sv.y * t1)) - dmin * (m0 * x.sv.z + m1 * x.sv.w);
+}
+
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q6_K> &w, const XRegs<RT_GGML_Q6_K> &x, int u) {
+    const int s8 = (u & 1) * 8;
+    const uint32_t A[4] = RT_W4(w.A), B[4] = RT_W4(w.B), H[4] = RT_W4(w.H);
+    const uint32_t h0[4] = RT_W4(x.h[0]), h1[4] = RT_W4(x.h[1]), h2[4] = RT_W4(x.h[2]), h3[4] = RT_W4(x.h[3]);
+    const uint32_t l0[4] = RT_W4(x.l[0]), l1[4] = RT_W4(x.l[1]), l2[4] = RT_W4(x.l[2]), l3[4] = RT_W4(x.l[3]);
+    int dh[4] = { 0, 0, 0, 0 }, dl[4] = { 0, 0, 0, 0 };
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint32_t q1 = (A[i] & 0x0f0f0f0fu) | ((H[i] << 4) & 0x30303030u);
+        uint32_t q2 = (B[i] & 0x0f0f0f0fu) | ((H[i] << 2) & 0x30303030u);
+        uint32_t q3 = ((A[i] >> 4) & 0x0f0f0f0fu) | (H[i] & 0x30303030u);
+        uint32_t q4 = ((B[i] >> 4) & 0x0f0f0f0fu) | ((H[i] >> 2) & 0x30303030u);
+        dh[0] = sdot4(q1, (int)h0[i], dh[0]);  dl[0] = sdot4(q1, (int)l0[i], dl[0]);
+        dh[1] = sdot4(q2, (int)h1[i], dh[1]);  dl[1] = sdot4(q2, (int)l1[i], dl[1]);
+        dh[2] = sdot4(q3, (int)h2[i], dh[2]);  dl[2] = sdot4(q3, (int)l2[i], dl[2]);
+        dh[3] = sdot4(q4, (int)h3[i], dh[3]);  dl[3] = sdot4(q4, (int)l3[i], dl[3]);
+    }
+    uint32_t s01 = w.sc.x >> s8, s23 = w.sc.y >> s8;
+    float sc0 = (float)(int)(int8_t)(s01 & 0xFF), sc1 = (float)(int)(int8_t)((s01 >> 16) & 0xFF);
+    float sc2 = (float)(int)(int8_t)(s23 & 0xFF), sc3 = (float)(int)(int8_t)((s23 >> 16) & 0xFF);
+    float a = sc0 * (x.xs.x * (float)((dh[0] << 7) + dl[0]) - 32.f * x.xb.x);
+    a += sc1 * (x.xs.y * (float)((dh[1] << 7) + dl[1]) - 32.f * x.xb.y);
+    a += sc2 * (x.xs.z * (float)((dh[2] << 7) + dl[2]) - 32.f * x.xb.z);
+    a += sc3 * (x.xs.w * (float)((dh[3] << 7) + dl[3]) - 32.f * x.xb.w);
+    return h2f(w.d) * a;
+}
+
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q8_0> &w, const XRegs<RT_GGML_Q8_0> &x, int) {
+    const uint32_t q[8] = { w.a.x, w.a.y, w.a.z, w.a.w, w.b.x, w.b.y, w.b.z, w.b.w };
+    const uint32_t xh[8] = { x.h[0].x, x.h[0].y, x.h[0].z, x.h[0].w, x.h[1].x, x.h[1].y, x.h[1].z, x.h[1].w };
+    const uint32_t xl[8] = { x.l[0].x, x.l[0].y, x.l[0].z, x.l[0].w, x.l[1].x, x.l[1].y, x.l[1].z, x.l[1].w };
+    int dh = 0, dl = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        dh = sdot4(q[i], (int)xh[i], dh);
+        dl = sdot4(q[i], (int)xl[i], dl);
+    }
+    return h2f(w.d) * (x.s * ((float)dh * 128.f + (float)dl));
+}
+
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_0> &w, const XRegs<RT_GGML_Q4_0> &x, int) {
+    const uint32_t q[4] = RT_W4(w.a);
+    const uint32_t hlo[4] = RT_W4(x.h[0]), hhi[4] = RT_W4(x.h[1]), llo[4] = RT_W4(x.l[0]), lhi[4] = RT_W4(x.l[1]);
+    int dh = 0, dl = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint32_t lo = q[i] & 0x0f0f0f0fu, hi = (q[i] >> 4) & 0x0f0f0f0fu;
+        dh = sdot4(lo, (int)hlo[i], dh);
+        dl = sdot4(lo, (int)llo[i], dl);
+        dh = sdot4(hi, (int)hhi[i], dh);
+        dl = sdot4(hi, (int)lhi[i], dl);
+    }
+    return h2f(w.d) * (x.sv.x * (float)((dh << 7) + dl) - 8.f * x.sv.y);
+}
+
+// A wave walks "steps": step s = (row group s / n_iter, unit pass s % n_iter); a row group is R rows (with the
+// SwiGLU epilogue: R/2 gate rows and their up rows).  Row groups are dealt round-robin over all waves that work
+// on the problem.  The weight registers of step s+1 are requested before step s is consumed.
+template <int TYPE, int R, bool COH>
+struct Walker {
+    const GemvProb &P;
+    const uint32_t *lds;
+    int m, U, n_iter, lane, gw, n_gw, n_groups, rows_per_group;
+    bool dual;
+
+    __device__ __forceinline__ int group_of(int s) const { return gw + (s / n_iter) * n_gw; }
+    __device__ __forceinline__ int unit_of(int s) const { return lane + 64 * (s % n_iter); }
+
+    __device__ __forceinline__ void request(WRegs<TYPE> *w, int s) const {
+        const int g = group_of(s);
+        const int u = min(unit_of(s), U - 1);  // lanes past the end of the row reread the last unit; masked later
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int row = dual ? g * rows_per_group + (r >> 1) : g * rows_per_group + r;
+            row = min(row, P.N - 1);  // ragged tail: reread the last row, the store is skipped
+            const uint8_t *rp = ((dual && (r & 1)) ? P.w2 : P.w) + (size_t)row * P.row_bytes;
+            load_w(w[r], rp, u);
+        }
+    }
+
+    // x slice of the unit a lane works on in step s (rows of <= 64 units: the same slice in every step)
+    __device__ __forceinline__ void fetch_x(XRegs<TYPE> &x, int s) const { load_x(x, lds, min(unit_of(s), U - 1), U, P.K); }
+
+    __device__ __forceinline__ void consume(const WRegs<TYPE> *w, const XRegs<TYPE> &x, int s, float *acc) const {
+        const int u = unit_of(s);
+        const int uc = min(u, U - 1);
+        const float live = u < U ? 1.f : 0.f;
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += live * dot_unit(w[r], x, uc);
+        if (s % n_iter != n_iter - 1) return;
+        const int g = group_of(s);
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = wave_sum_dpp(acc[r]);
+        if (dual) {
+#pragma unroll
+            for (int r = 0; r < R / 2; r++) {
+                int row = g * rows_per_group + r;
+                if (lane == r && row < P.N) {
+                    float gate = acc[2 * r], up = acc[2 * r + 1];
+                    st_f<COH>(&P.y[(size_t)m * P.N + row], up * (gate * (1.0f / (1.0f + expf(-gate)))));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                int row = g * rows_per_group + r;
+                if (lane == r && row < P.N) {
+                    size_t o = (size_t)m * P.N + row;
+                    st_f<COH>(&P.y[o], P.res ? ld_f<COH>(&P.res[o]) + acc[r] : acc[r]);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = 0.f;
+    }
+};
+
+
+// All rows of problem P that fall to workgroup `wg` of the `n_wg` workgroups sharing it.
+template <int TYPE, int R, bool COH>
+__device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg, int m, uint32_t *lds, float *red) {
+    const int waves = (int)(blockDim.x >> 6);
+    Walker<TYPE, R, COH> W{ P, lds, m, units_of(TYPE, P.K), 0, (int)(threadIdx.x & 63), 0, 0, 0, 0, P.epi == kEpiSwiglu };
+    W.n_iter = (W.U + 63) / 64;
+    W.rows_per_group = W.dual ? R / 2 : R;
+    W.n_groups = (P.N + W.rows_per_group - 1) / W.rows_per_group;
+    W.gw = wg * waves + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // wave-uniform: row addresses stay scalar
+    W.n_gw = n_wg * waves;
+    const int my_groups = W.gw < W.n_groups ? (W.n_groups - W.gw + W.n_gw - 1) / W.n_gw : 0;
+    const int steps = my_groups * W.n_iter;
+    WRegs<TYPE> a[R], b[R];
+    if (steps > 0) W.request(a, 0);      // in flight while x is being staged
+    stage_x<COH>(P, m, lds, red);
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+    XRegs<TYPE> x;
+    if (W.n_iter == 1) {
+        // every step of this lane meets the same x slice: keep it in registers, LDS is read once
+        W.fetch_x(x, 0);
+        for (int s = 0; s < steps; s += 2) {
+            if (s + 1 < steps) W.request(b, s + 1);
+            W.consume(a, x, s, acc);
+            if (s + 1 < steps) {
+                if (s + 2 < steps) W.request(a, s + 2);
+                W.consume(b, x, s + 1, acc);
+            }
+        }
+    } else {
+        for (int s = 0; s < steps; s += 2) {
+            if (s + 1 < steps) W.request(b, s + 1);
+            W.fetch_x(x, s);
+            W.consume(a, x, s, acc);
+            if (s + 1 < steps) {
+                if (s + 2 < steps) W.request(a, s + 2);
+                W.fetch_x(x, s + 1);
+                W.consume(b, x, s + 1, acc);
+            }
+        }
+    }
+}
+
+// Dispatch on the block format.  R2 picks two rows per wave step (always used by the SwiGLU epilogue).
+template <bool COH>
+__device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_wg, int m, bool r2, uint32_t *lds, float *red) {
+    if (r2 || P.epi == kEpiSwiglu) {
+        switch (P.type) {
+        case RT_GGML_Q4_K: gemv_problem<RT_GGML_Q4_K, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q6_K: gemv_problem<RT_GGML_Q6_K, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        }
+    } else {
+        switch (P.type) {
+        case RT_GGML_Q4_K: gemv_problem<RT_GGML_Q4_K, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q6_K: gemv_problem<RT_GGML_Q6_K, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        }
+    }
+}
+
+}  // namespace rt

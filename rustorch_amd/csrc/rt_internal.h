@@ -32,13 +32,28 @@ constexpr int kWave = 64;
 // padded to a multiple of 16 bytes.
 __host__ __device__ inline size_t xq_stride(size_t K) { return (2 * K + K / 8 + K / 4 + 15) & ~(size_t)15; }
 
+// How a GEMV workgroup obtains the activation vector it stages into LDS.
+enum : int {
+    kStageXq = 0,   // x points at a ready xq vector (batch stride xq_stride(K))
+    kStageF32 = 1,  // x points at f32 (batch stride K); quantized while staging
+    kStageRms = 2,  // x points at f32; RMS-normalised with gamma / eps, then quantized
+};
+enum : int {
+    kEpiStore = 0,   // y = W x (+ res when res != nullptr)
+    kEpiSwiglu = 1,  // y = (W2 x) * silu(W x): W = gate rows, W2 = up rows of the same shape and type
+};
+
 struct GemvProb {
     const uint8_t *w;    // raw GGUF blocks, row r at w + r * row_bytes
-    const uint8_t *xq;   // quantized activations, vector m at xq + m * xq_stride(K)
+    const uint8_t *w2;   // second matrix for kEpiSwiglu
+    const void *x;       // activations, see kStage*
+    const float *gamma;  // kStageRms
     float *y;            // [batch, N]
     const float *res;    // optional residual added to y (same shape), may alias y
     size_t row_bytes;
+    float eps;           // kStageRms
     int type, N, K;
+    int stage, epi;
     int tile0;           // index of this problem's first tile in the launch
     int rows_per_tile;
 };
@@ -70,8 +85,10 @@ hipError_t launch_kv_append(hipStream_t s, uint16_t *cache, const float *v, cons
 hipError_t launch_rope_kv(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache,
                           uint16_t *vcache, const int *pos_dev, int n_heads, int head_dim,
                           const float *inv_freq_dev);
-hipError_t launch_attn_decode(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc,
-                              const int *pos_dev, int n_pos, int n_heads, int head_dim, float *out, uint8_t *xq);
+// fused = rotate q / k of the step, append k / v at *pos_dev, then attend over [0, *pos_dev]; otherwise attend over [0, n_pos)
+hipError_t launch_attn_decode(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
+                              const int *pos_dev, int n_pos, int n_heads, int head_dim, const float *inv_freq_dev,
+                              float *out, uint8_t *xq, bool fused);
 hipError_t launch_add(hipStream_t s, float *x, const float *y, size_t n);
 hipError_t launch_argmax(hipStream_t s, const float *v, size_t n, int *out_dev);
 hipError_t launch_embed_row(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,

@@ -8,62 +8,9 @@
 //   Q4_0 18 B / 32 el : f16 d; u8 qs[16]        (low nibbles = el 0..15, high = 16..31)
 //   Q4_K 144 B / 256  : f16 d; f16 dmin; u8 scales[12]; u8 qs[128]
 //   Q6_K 210 B / 256  : u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d
-#include "rt_internal.h"
-
-#include <hip/hip_fp16.h>
+#include "rt_device.h"
 
 namespace rt {
-
-// ------------------------------------------------------------------ helpers
-
-__device__ __forceinline__ float h2f(uint32_t bits16) {
-    return (float)__builtin_bit_cast(_Float16, (unsigned short)bits16);
-}
-__device__ __forceinline__ uint16_t f2h_rne(float f) {
-    return __builtin_bit_cast(unsigned short, (_Float16)f);
-}
-
-// Loads through a byte pointer with no alignment promise (Q6_K / Q8_0 / Q4_0 blocks are only 2-byte aligned).
-__device__ __forceinline__ uint4 ld16u(const uint8_t *p) { uint4 v; __builtin_memcpy(&v, p, 16); return v; }
-__device__ __forceinline__ uint2 ld8u(const uint8_t *p) { uint2 v; __builtin_memcpy(&v, p, 8); return v; }
-__device__ __forceinline__ uint32_t ld4u(const uint8_t *p) { uint32_t v; __builtin_memcpy(&v, p, 4); return v; }
-__device__ __forceinline__ uint32_t ld2u(const uint8_t *p) { unsigned short v; __builtin_memcpy(&v, p, 2); return v; }
-__device__ __forceinline__ uint4 ld16a(const uint8_t *p) { return *reinterpret_cast<const uint4 *>(p); }
-
-__device__ __forceinline__ int sdot4(uint32_t a, int b, int c) { return __builtin_amdgcn_sdot4((int)a, b, c, false); }
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
-}
-
-// Block-wide sum / max through LDS (red must hold blockDim/64 floats). All threads get the result.
-__device__ __forceinline__ float block_sum(float v, float *red) {
-    v = wave_sum(v);
-    int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) red[w] = v;
-    __syncthreads();
-    float t = 0.f;
-    for (int i = 0; i < nw; i++) t += red[i];
-    return t;
-}
-__device__ __forceinline__ float block_max(float v, float *red) {
-    v = wave_max(v);
-    int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) red[w] = v;
-    __syncthreads();
-    float t = red[0];
-    for (int i = 1; i < nw; i++) t = fmaxf(t, red[i]);
-    return t;
-}
 
 // --------------------------------------------------------- exact block decode
 // One element of a tensor row, evaluated exactly as the block definition is written
@@ -141,29 +88,13 @@ __global__ void embed_row_kernel(int type, const uint8_t *w, size_t row_bytes, s
 // Quantize 4 consecutive elements (e % 4 == 0) of a K-vector into xq.  The 8 lanes that
 // hold one 32-element block must be consecutive lanes of one wave and all active.
 __device__ __forceinline__ void quantize_store4(float4 v, size_t e, uint8_t *xq, size_t K) {
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
-    float inv = amax > 0.f ? 16383.0f / amax : 0.f;
-    float s = amax / 16383.0f;
-    int q0 = max(-16383, min(16383, __float2int_rn(v.x * inv)));
-    int q1 = max(-16383, min(16383, __float2int_rn(v.y * inv)));
-    int q2 = max(-16383, min(16383, __float2int_rn(v.z * inv)));
-    int q3 = max(-16383, min(16383, __float2int_rn(v.w * inv)));
-    uint32_t hi = ((uint32_t)(q0 >> 7) & 0xFF) | (((uint32_t)(q1 >> 7) & 0xFF) << 8) |
-                  (((uint32_t)(q2 >> 7) & 0xFF) << 16) | (((uint32_t)(q3 >> 7) & 0xFF) << 24);
-    uint32_t lo = (uint32_t)(q0 & 127) | ((uint32_t)(q1 & 127) << 8) | ((uint32_t)(q2 & 127) << 16) |
-                  ((uint32_t)(q3 & 127) << 24);
-    int sum = q0 + q1 + q2 + q3;
-    sum += __shfl_xor(sum, 1, 64);
-    sum += __shfl_xor(sum, 2, 64);
-    *reinterpret_cast<uint32_t *>(xq + e) = hi;
-    *reinterpret_cast<uint32_t *>(xq + K + e) = lo;
+    Q4Pack p = quantize4(v);
+    *reinterpret_cast<uint32_t *>(xq + e) = p.hi;
+    *reinterpret_cast<uint32_t *>(xq + K + e) = p.lo;
     float *sp = reinterpret_cast<float *>(xq + 2 * K);
     float *bp = sp + K / 32;
-    if ((e & 15) == 0) bp[e >> 4] = s * (float)sum;
-    if ((e & 31) == 0) sp[e >> 5] = s;
+    if ((e & 15) == 0) bp[e >> 4] = p.s * (float)p.sum16;
+    if ((e & 31) == 0) sp[e >> 5] = p.s;
 }
 
 __global__ __launch_bounds__(256) void quantize_x_kernel(const float *x, uint8_t *xq, size_t K) {
@@ -182,177 +113,6 @@ __global__ __launch_bounds__(256) void quantize_group_kernel(QuantGroupArgs a) {
     if (i4 * 4 >= K) return;
     float4 v = reinterpret_cast<const float4 *>(a.x[p])[i4];
     quantize_store4(v, i4 * 4, a.xq[p], K);
-}
-
-// ------------------------------------------------------------ GEMV unit dots
-// A "unit" is the slice of one weight row a lane consumes in one go.  x lives in LDS in
-// xq form: xh / xl as dwords of 4 int8, xs per 32-block, xb per 16-run.
-
-struct XLds {
-    const int *xh, *xl;
-    const float *xs, *xb;
-};
-
-// Q4_K unit u: super-block u/4, 64-element group g = u%4 (32 qs bytes; low nibbles = sub-block 2g, high = 2g+1).
-__device__ __forceinline__ float unit_q4k(const uint8_t *row, int u, const XLds &X) {
-    int sb = u >> 2, g = u & 3;
-    const uint8_t *blk = row + (size_t)sb * 144;
-    uint4 hdr = ld16a(blk);
-    uint4 qa = ld16a(blk + 16 + 32 * g);
-    uint4 qb = ld16a(blk + 32 + 32 * g);
-    uint32_t scw, mw;
-    if (g < 2) {
-        scw = hdr.y & 0x3f3f3f3fu;
-        mw = hdr.z & 0x3f3f3f3fu;
-    } else {
-        scw = (hdr.w & 0x0f0f0f0fu) | ((hdr.y >> 2) & 0x30303030u);
-        mw = ((hdr.w >> 4) & 0x0f0f0f0fu) | ((hdr.z >> 2) & 0x30303030u);
-    }
-    int sh = (g & 1) * 16;
-    float sc0 = (float)((scw >> sh) & 0xFF), sc1 = (float)((scw >> (sh + 8)) & 0xFF);
-    float m0 = (float)((mw >> sh) & 0xFF), m1 = (float)((mw >> (sh + 8)) & 0xFF);
-    float d = h2f(hdr.x & 0xFFFF), dmin = h2f(hdr.x >> 16);
-    uint32_t q[8] = { qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w };
-    int e4 = u * 16;
-    int dh0 = 0, dl0 = 0, dh1 = 0, dl1 = 0;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        uint32_t lo = q[i] & 0x0f0f0f0fu, hi = (q[i] >> 4) & 0x0f0f0f0fu;
-        dh0 = sdot4(lo, X.xh[e4 + i], dh0);
-        dl0 = sdot4(lo, X.xl[e4 + i], dl0);
-        dh1 = sdot4(hi, X.xh[e4 + 8 + i], dh1);
-        dl1 = sdot4(hi, X.xl[e4 + 8 + i], dl1);
-    }
-    float t0 = (float)((dh0 << 7) + dl0), t1 = (float)((dh1 << 7) + dl1);
-    int b = u * 2;
-    float s0 = X.xs[b], s1 = X.xs[b + 1];
-    float bs0 = X.xb[2 * b] + X.xb[2 * b + 1], bs1 = X.xb[2 * b + 2] + X.xb[2 * b + 3];
-    return d * (sc0 * (s0 * t0) + sc1 * (s1 * t1)) - dmin * (m0 * bs0 + m1 * bs1);
-}
-
-// Q6_K unit u: super-block u/4, half h = (u/2)%2, l-range c = u%2 (l in [16c, 16c+16)); four 16-element runs.
-__device__ __forceinline__ float unit_q6k(const uint8_t *row, int u, const XLds &X) {
-    int sb = u >> 2, h = (u >> 1) & 1, c = u & 1;
-    const uint8_t *blk = row + (size_t)sb * 210;
-    uint4 A4 = ld16u(blk + 64 * h + 16 * c);
-    uint4 B4 = ld16u(blk + 64 * h + 32 + 16 * c);
-    uint4 H4 = ld16u(blk + 128 + 32 * h + 16 * c);
-    uint2 scw = ld8u(blk + 192 + 8 * h);
-    float d = h2f(ld2u(blk + 208));
-    uint32_t A[4] = { A4.x, A4.y, A4.z, A4.w }, B[4] = { B4.x, B4.y, B4.z, B4.w }, H[4] = { H4.x, H4.y, H4.z, H4.w };
-    int dh[4] = { 0, 0, 0, 0 }, dl[4] = { 0, 0, 0, 0 };
-    int xd = 64 * sb + 32 * h + 4 * c;  // dword index of run 0
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        uint32_t q1 = (A[i] & 0x0f0f0f0fu) | ((H[i] << 4) & 0x30303030u);
-        uint32_t q2 = (B[i] & 0x0f0f0f0fu) | ((H[i] << 2) & 0x30303030u);
-        uint32_t q3 = ((A[i] >> 4) & 0x0f0f0f0fu) | (H[i] & 0x30303030u);
-        uint32_t q4 = ((B[i] >> 4) & 0x0f0f0f0fu) | ((H[i] >> 2) & 0x30303030u);
-        dh[0] = sdot4(q1, X.xh[xd + i], dh[0]);       dl[0] = sdot4(q1, X.xl[xd + i], dl[0]);
-        dh[1] = sdot4(q2, X.xh[xd + 8 + i], dh[1]);   dl[1] = sdot4(q2, X.xl[xd + 8 + i], dl[1]);
-        dh[2] = sdot4(q3, X.xh[xd + 16 + i], dh[2]);  dl[2] = sdot4(q3, X.xl[xd + 16 + i], dl[2]);
-        dh[3] = sdot4(q4, X.xh[xd + 24 + i], dh[3]);  dl[3] = sdot4(q4, X.xl[xd + 24 + i], dl[3]);
-    }
-    // scales sc[c + 2r], r = 0..3: bytes c, c+2 of scw.x and of scw.y
-    int s8 = c * 8;
-    float sc0 = (float)(int)(int8_t)((scw.x >> s8) & 0xFF), sc1 = (float)(int)(int8_t)((scw.x >> (s8 + 16)) & 0xFF);
-    float sc2 = (float)(int)(int8_t)((scw.y >> s8) & 0xFF), sc3 = (float)(int)(int8_t)((scw.y >> (s8 + 16)) & 0xFF);
-    int sbk = 8 * sb + 4 * h;            // x 32-block of run 0
-    int bbk = 16 * sb + 8 * h + c;       // x 16-run of run 0
-    float acc = sc0 * (X.xs[sbk] * (float)((dh[0] << 7) + dl[0]) - 32.f * X.xb[bbk]);
-    acc += sc1 * (X.xs[sbk + 1] * (float)((dh[1] << 7) + dl[1]) - 32.f * X.xb[bbk + 2]);
-    acc += sc2 * (X.xs[sbk + 2] * (float)((dh[2] << 7) + dl[2]) - 32.f * X.xb[bbk + 4]);
-    acc += sc3 * (X.xs[sbk + 3] * (float)((dh[3] << 7) + dl[3]) - 32.f * X.xb[bbk + 6]);
-    return d * acc;
-}
-
-// Q8_0 unit u = block u.
-__device__ __forceinline__ float unit_q80(const uint8_t *row, int u, const XLds &X) {
-    const uint8_t *blk = row + (size_t)u * 34;
-    float d = h2f(ld2u(blk));
-    uint4 a = ld16u(blk + 2), b = ld16u(blk + 18);
-    uint32_t q[8] = { a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w };
-    int dh = 0, dl = 0;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        dh = sdot4(q[i], X.xh[8 * u + i], dh);
-        dl = sdot4(q[i], X.xl[8 * u + i], dl);
-    }
-    return d * (X.xs[u] * ((float)dh * 128.f + (float)dl));
-}
-
-// Q4_0 unit u = block u.
-__device__ __forceinline__ float unit_q40(const uint8_t *row, int u, const XLds &X) {
-    const uint8_t *blk = row + (size_t)u * 18;
-    float d = h2f(ld2u(blk));
-    uint4 a = ld16u(blk + 2);
-    uint32_t q[4] = { a.x, a.y, a.z, a.w };
-    int dh = 0, dl = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        uint32_t lo = q[i] & 0x0f0f0f0fu, hi = (q[i] >> 4) & 0x0f0f0f0fu;
-        dh = sdot4(lo, X.xh[8 * u + i], dh);
-        dl = sdot4(lo, X.xl[8 * u + i], dl);
-        dh = sdot4(hi, X.xh[8 * u + 4 + i], dh);
-        dl = sdot4(hi, X.xl[8 * u + 4 + i], dl);
-    }
-    return d * (X.xs[u] * (float)((dh << 7) + dl) - 8.f * (X.xb[2 * u] + X.xb[2 * u + 1]));
-}
-
-template <int TYPE> __device__ __forceinline__ float unit_dot(const uint8_t *row, int u, const XLds &X) {
-    if (TYPE == RT_GGML_Q4_K) return unit_q4k(row, u, X);
-    if (TYPE == RT_GGML_Q6_K) return unit_q6k(row, u, X);
-    if (TYPE == RT_GGML_Q8_0) return unit_q80(row, u, X);
-    return unit_q40(row, u, X);
-}
-
-template <int TYPE>
-__device__ __forceinline__ void gemv_rows(const GemvProb &P, int row0, int row1, int m, const XLds &X) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int nwaves = blockDim.x >> 6;
-    const int unit_elems = (TYPE == RT_GGML_Q4_K || TYPE == RT_GGML_Q6_K) ? 64 : 32;
-    const int n_units = P.K / unit_elems;
-    for (int row = row0 + wave; row < row1; row += nwaves) {
-        const uint8_t *rp = P.w + (size_t)row * P.row_bytes;
-        float acc = 0.f;
-        for (int u = lane; u < n_units; u += 64) acc += unit_dot<TYPE>(rp, u, X);
-        acc = wave_sum(acc);
-        if (lane == 0) {
-            size_t o = (size_t)m * P.N + row;
-            P.y[o] = P.res ? P.res[o] + acc : acc;
-        }
-    }
-}
-
-__global__ __launch_bounds__(256) void qgemv_kernel(GemvArgs a) {
-    extern __shared__ uint4 lds[];
-    int tile = blockIdx.x;
-    int pi = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxGemvProbs; i++)
-        if (i < a.n && tile >= a.p[i].tile0) pi = i;
-    const GemvProb &P = a.p[pi];
-    int t = tile - P.tile0;
-    int row0 = t * P.rows_per_tile;
-    int row1 = min(P.N, row0 + P.rows_per_tile);
-    int m = blockIdx.y;
-    size_t K = (size_t)P.K;
-    size_t stride = xq_stride(K);
-    const uint4 *src = reinterpret_cast<const uint4 *>(P.xq + (size_t)m * stride);
-    for (int i = threadIdx.x; i < (int)(stride / 16); i += blockDim.x) lds[i] = src[i];
-    __syncthreads();
-    const char *base = reinterpret_cast<const char *>(lds);
-    XLds X;
-    X.xh = reinterpret_cast<const int *>(base);
-    X.xl = reinterpret_cast<const int *>(base + K);
-    X.xs = reinterpret_cast<const float *>(base + 2 * K);
-    X.xb = X.xs + K / 32;
-    switch (P.type) {
-    case RT_GGML_Q4_K: gemv_rows<RT_GGML_Q4_K>(P, row0, row1, m, X); break;
-    case RT_GGML_Q6_K: gemv_rows<RT_GGML_Q6_K>(P, row0, row1, m, X); break;
-    case RT_GGML_Q8_0: gemv_rows<RT_GGML_Q8_0>(P, row0, row1, m, X); break;
-    case RT_GGML_Q4_0: gemv_rows<RT_GGML_Q4_0>(P, row0, row1, m, X); break;
-    }
 }
 
 // ------------------------------------------------------------------ RMSNorm
@@ -460,61 +220,132 @@ __global__ void rope_kv_kernel(float *q, const float *k, const float *v, uint16_
 
 // -------------------------------------------------------- decode attention
 // One block (256 threads) per head; cache layout [pos][head][dim], fp16.
-// scores = (q . k_j) / sqrt(dim); p = softmax(scores) with max subtraction; out = sum_j p_j v_j
+//   scores_j = (q . k_j) / sqrt(dim);  p = softmax(scores) with max subtraction;  out = sum_j p_j v_j
 // (example-cli/src/model/architectures/attention.rs:233-338 for one query row).
-// EPL = head_dim / 64 (1 or 2).  Dynamic LDS: n_pos floats of scores.
-template <int EPL>
-__global__ __launch_bounds__(256) void attn_decode_kernel(const float *q, const uint16_t *kc, const uint16_t *vc,
-                                                          const int *pos_dev, int n_pos_arg, int n_heads, float *out,
-                                                          uint8_t *xq) {
+// FUSED: the block first rotates its head's q and k (interleaved pairs, angle pos * inv_freq[i]), stores
+// fp16(k), fp16(v) as cache row pos and attends over [0, pos]; the fresh row is taken from LDS, not re-read.
+// Scores: one thread per position, the whole head_dim dot in that thread (16-byte loads of 8 halves).
+// Values: 16-byte column chunks x position groups, combined through LDS.
+// Dynamic LDS: n_pos floats.
+__device__ __forceinline__ void unpack8(uint4 v, float *f) {
+    const uint32_t w[4] = { v.x, v.y, v.z, v.w };
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        f[2 * i] = h2f(w[i] & 0xFFFF);
+        f[2 * i + 1] = h2f(w[i] >> 16);
+    }
+}
+
+template <int HD, bool FUSED>
+__global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float *k, const float *v, uint16_t *kc,
+                                                          uint16_t *vc, const int *pos_dev, int n_pos_arg, int n_heads,
+                                                          const float *inv_freq, float *out, uint8_t *xq) {
     extern __shared__ float sc[];
     __shared__ float red[4];
-    __shared__ __align__(16) float part[256];
-    constexpr int HD = 64 * EPL;
-    const int n_pos = pos_dev ? *pos_dev + 1 : n_pos_arg;
-    const int h = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    __shared__ __align__(16) float qs[HD];
+    __shared__ __align__(16) float kcur[HD];
+    __shared__ __align__(16) float vcur[HD];
+    __shared__ __align__(16) float part[2048];
+    constexpr int CH = HD / 8;          // 16-byte chunks per cache row of this head
+    constexpr int NG = 256 / CH;        // position groups in the value phase
+    const int h = blockIdx.x, tid = threadIdx.x;
     const size_t row = (size_t)n_heads * HD;
+    const int cur = FUSED ? *pos_dev : -1;
+    const int n_pos = FUSED ? cur + 1 : n_pos_arg;
     const float scale = 1.0f / sqrtf((float)HD);
-    float qv[EPL];
-#pragma unroll
-    for (int e = 0; e < EPL; e++) qv[e] = q[(size_t)h * HD + lane * EPL + e];
-    for (int j = wave; j < n_pos; j += 4) {
-        const uint16_t *kr = kc + (size_t)j * row + (size_t)h * HD + lane * EPL;
-        float s = 0.f;
-#pragma unroll
-        for (int e = 0; e < EPL; e++) s += qv[e] * h2f(kr[e]);
-        s = wave_sum(s);
-        if (lane == 0) sc[j] = s * scale;
+    if (FUSED) {
+        if (tid < HD / 2) {
+            int i = tid;
+            float sn, cs;
+            sincosf((float)cur * inv_freq[i], &sn, &cs);
+            float2 qv = reinterpret_cast<const float2 *>(q + (size_t)h * HD)[i];
+            float2 kv = reinterpret_cast<const float2 *>(k + (size_t)h * HD)[i];
+            float q0 = qv.x * cs - qv.y * sn, q1 = qv.x * sn + qv.y * cs;
+            float k0 = kv.x * cs - kv.y * sn, k1 = kv.x * sn + kv.y * cs;
+            qs[2 * i] = q0;
+            qs[2 * i + 1] = q1;
+            reinterpret_cast<float2 *>(q + (size_t)h * HD)[i] = make_float2(q0, q1);
+            uint16_t a = f2h_rne(k0), b = f2h_rne(k1);
+            kcur[2 * i] = h2f(a);
+            kcur[2 * i + 1] = h2f(b);
+            reinterpret_cast<uint32_t *>(kc + (size_t)cur * row + (size_t)h * HD)[i] = (uint32_t)a | ((uint32_t)b << 16);
+        } else if (tid < HD) {
+            int i = tid - HD / 2;
+            float2 vv = reinterpret_cast<const float2 *>(v + (size_t)h * HD)[i];
+            uint16_t a = f2h_rne(vv.x), b = f2h_rne(vv.y);
+            vcur[2 * i] = h2f(a);
+            vcur[2 * i + 1] = h2f(b);
+            reinterpret_cast<uint32_t *>(vc + (size_t)cur * row + (size_t)h * HD)[i] = (uint32_t)a | ((uint32_t)b << 16);
+        }
+    } else if (tid < HD) {
+        qs[tid] = q[(size_t)h * HD + tid];
     }
     __syncthreads();
+    // ---- scores
     float mx = -INFINITY;
-    for (int j = threadIdx.x; j < n_pos; j += 256) mx = fmaxf(mx, sc[j]);
+    for (int j = tid; j < n_pos; j += 256) {
+        float s = 0.f;
+        if (j == cur) {
+#pragma unroll 8
+            for (int d = 0; d < HD; d++) s += qs[d] * kcur[d];
+        } else {
+            const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)j * row + (size_t)h * HD);
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                float f[8];
+                unpack8(kr[c], f);
+#pragma unroll
+                for (int e = 0; e < 8; e++) s += qs[8 * c + e] * f[e];
+            }
+        }
+        s *= scale;
+        sc[j] = s;
+        mx = fmaxf(mx, s);
+    }
     mx = block_max(mx, red);
     float sum = 0.f;
-    for (int j = threadIdx.x; j < n_pos; j += 256) {
+    for (int j = tid; j < n_pos; j += 256) {
         float e = expf(sc[j] - mx);
         sc[j] = e;
         sum += e;
     }
     sum = block_sum(sum, red);
-    for (int j = threadIdx.x; j < n_pos; j += 256) sc[j] = sc[j] / sum;
+    for (int j = tid; j < n_pos; j += 256) sc[j] = sc[j] / sum;
     __syncthreads();
-    const int d = threadIdx.x % HD, grp = threadIdx.x / HD, ngrp = 256 / HD;
-    float acc = 0.f;
-    for (int j = grp; j < n_pos; j += ngrp) acc += sc[j] * h2f(vc[(size_t)j * row + (size_t)h * HD + d]);
-    part[threadIdx.x] = acc;
+    // ---- values
+    const int c = tid % CH, g = tid / CH;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] = 0.f;
+    for (int j = g; j < n_pos; j += NG) {
+        float f[8];
+        if (j == cur) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) f[e] = vcur[8 * c + e];
+        } else {
+            unpack8(reinterpret_cast<const uint4 *>(vc + (size_t)j * row + (size_t)h * HD)[c], f);
+        }
+        float p = sc[j];
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += p * f[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) part[g * HD + 8 * c + e] = acc[e];
     __syncthreads();
-    if (threadIdx.x < HD) {
-        float o = 0.f;
-        for (int g = 0; g < ngrp; g++) o += part[g * HD + threadIdx.x];
-        part[threadIdx.x] = o;
-        if (out) out[(size_t)h * HD + threadIdx.x] = o;
+    float o = 0.f;
+    if (tid < HD) {
+        for (int gg = 0; gg < NG; gg++) o += part[gg * HD + tid];
+    }
+    __syncthreads();
+    if (tid < HD) {
+        part[tid] = o;
+        if (out) out[(size_t)h * HD + tid] = o;
     }
     if (xq) {
         __syncthreads();
-        if (threadIdx.x < HD / 4) {
-            float4 v = reinterpret_cast<const float4 *>(part)[threadIdx.x];
-            quantize_store4(v, (size_t)h * HD + threadIdx.x * 4, xq, row);
+        if (tid < HD / 4) {
+            float4 vq = reinterpret_cast<const float4 *>(part)[tid];
+            quantize_store4(vq, (size_t)h * HD + tid * 4, xq, row);
         }
     }
 }
@@ -600,28 +431,6 @@ hipError_t launch_quantize_group(hipStream_t s, const QuantGroupArgs &a) {
     return hipGetLastError();
 }
 
-hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
-    size_t total_rows = 0, maxK = 0;
-    for (int i = 0; i < a.n; i++) {
-        total_rows += (size_t)a.p[i].N;
-        if ((size_t)a.p[i].K > maxK) maxK = (size_t)a.p[i].K;
-    }
-    // aim for ~4 workgroups per CU across the launch; each workgroup re-stages x, so do not go below 8 rows
-    int rpt = (int)((total_rows + 1023) / 1024);
-    rpt = (rpt + 3) & ~3;
-    if (rpt < 8) rpt = 8;
-    int tiles = 0;
-    for (int i = 0; i < a.n; i++) {
-        a.p[i].tile0 = tiles;
-        a.p[i].rows_per_tile = rpt;
-        tiles += (a.p[i].N + rpt - 1) / rpt;
-    }
-    size_t lds = xq_stride(maxK);
-    dim3 grid((unsigned)tiles, (unsigned)batch);
-    qgemv_kernel<<<grid, 256, lds, s>>>(a);
-    return hipGetLastError();
-}
-
 hipError_t launch_dequant(hipStream_t s, int type, const uint8_t *w, size_t n_rows, size_t n_cols, float *out) {
     size_t total = n_rows * n_cols;
     size_t rb = n_cols / type_block_elems(type) * type_block_bytes(type);
@@ -671,13 +480,19 @@ hipError_t launch_rope_kv(hipStream_t s, float *q, const float *k, const float *
     return hipGetLastError();
 }
 
-hipError_t launch_attn_decode(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc,
-                              const int *pos_dev, int n_pos, int n_heads, int head_dim, float *out, uint8_t *xq) {
-    size_t lds = (size_t)n_pos * sizeof(float);  // with pos_dev set, n_pos is the upper bound (max_pos)
-    if (head_dim == 128)
-        attn_decode_kernel<2><<<dim3((unsigned)n_heads), 256, lds, s>>>(q, kc, vc, pos_dev, n_pos, n_heads, out, xq);
+hipError_t launch_attn_decode(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
+                              const int *pos_dev, int n_pos, int n_heads, int head_dim, const float *inv_freq_dev,
+                              float *out, uint8_t *xq, bool fused) {
+    size_t lds = (size_t)n_pos * sizeof(float);  // fused: n_pos is the upper bound (max_pos)
+    dim3 grid((unsigned)n_heads);
+    if (head_dim == 128 && fused)
+        attn_decode_kernel<128, true><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, inv_freq_dev, out, xq);
+    else if (head_dim == 128)
+        attn_decode_kernel<128, false><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, inv_freq_dev, out, xq);
+    else if (head_dim == 64 && fused)
+        attn_decode_kernel<64, true><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, inv_freq_dev, out, xq);
     else if (head_dim == 64)
-        attn_decode_kernel<1><<<dim3((unsigned)n_heads), 256, lds, s>>>(q, kc, vc, pos_dev, n_pos, n_heads, out, xq);
+        attn_decode_kernel<64, false><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, inv_freq_dev, out, xq);
     else
         return hipErrorInvalidValue;
     return hipGetLastError();

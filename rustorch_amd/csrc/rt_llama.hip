@@ -56,9 +56,12 @@ void free_all(rt_hip_llama *m) {
     m->allocs.clear();
 }
 
-void fill_prob(rt::GemvProb &p, const rt_hip_llama::T &t, const uint8_t *xq, float *y, const float *res) {
-    p.w = t.dev; p.xq = xq; p.y = y; p.res = res; p.row_bytes = t.row_bytes;
+rt::GemvProb make_prob(const rt_hip_llama::T &t, const void *x, int stage, float *y, const float *res) {
+    rt::GemvProb p;
+    memset(&p, 0, sizeof p);
+    p.w = t.dev; p.x = x; p.stage = stage; p.y = y; p.res = res; p.row_bytes = t.row_bytes;
     p.type = t.type; p.N = (int)t.n_rows; p.K = (int)t.n_cols;
+    return p;
 }
 
 int check_complete(rt_hip_ctx *ctx, const rt_hip_llama *m) {
@@ -72,48 +75,51 @@ int check_complete(rt_hip_ctx *ctx, const rt_hip_llama *m) {
     return RT_HIP_OK;
 }
 
-// One decode step driven by state[0] (pos) and state[1] (token). Enqueue only.
+// One decode step driven by state[0] (pos) and state[1] (token). Enqueue only.  Five launches per layer:
+//   q,k,v = W . rmsnorm(x)         (norm + quantization fused into the GEMV's staging)
+//   rope + cache append + attention (output in the GEMV's quantized form)
+//   x += Wo . a
+//   f = up(h) * silu(gate(h)), h = rmsnorm(x)   (norm in the staging, SwiGLU in the epilogue)
+//   x += Wdown . f                  (quantization of f in the staging)
 int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
     hipStream_t s = ctx->stream;
     const rt_hip_llama_config &c = m->cfg;
-    const size_t H = (size_t)c.hidden, F = (size_t)c.ffn;
+    const size_t H = (size_t)c.hidden;
     int *pos_dev = m->state, *tok_dev = m->state + 1;
     RT_TRY_HIP(ctx, rt::launch_embed_row(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, tok_dev, c.vocab, m->x));
     for (int l = 0; l < c.n_layers; l++) {
         uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * H;
         uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * H;
-        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, m->x, m->attn_norm[l], nullptr, m->xq_h, 1, H, c.rms_eps));
         rt::GemvArgs a;
         memset(&a, 0, sizeof a);
         a.n = 3;
-        fill_prob(a.p[0], m->wq[l], m->xq_h, m->q, nullptr);
-        fill_prob(a.p[1], m->wk[l], m->xq_h, m->k, nullptr);
-        fill_prob(a.p[2], m->wv[l], m->xq_h, m->v, nullptr);
+        a.p[0] = make_prob(m->wq[l], m->x, rt::kStageRms, m->q, nullptr);
+        a.p[1] = make_prob(m->wk[l], m->x, rt::kStageRms, m->k, nullptr);
+        a.p[2] = make_prob(m->wv[l], m->x, rt::kStageRms, m->v, nullptr);
+        for (int i = 0; i < 3; i++) { a.p[i].gamma = m->attn_norm[l]; a.p[i].eps = c.rms_eps; }
         RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
-        RT_TRY_HIP(ctx, rt::launch_rope_kv(s, m->q, m->k, m->v, kc, vc, pos_dev, c.n_heads, m->head_dim, m->inv_freq));
-        RT_TRY_HIP(ctx, rt::launch_attn_decode(s, m->q, kc, vc, pos_dev, c.max_pos, c.n_heads, m->head_dim, nullptr, m->xq_a));
+        RT_TRY_HIP(ctx, rt::launch_attn_decode(s, m->q, m->k, m->v, kc, vc, pos_dev, c.max_pos, c.n_heads, m->head_dim, m->inv_freq,
+                                               nullptr, m->xq_a, true));
         memset(&a, 0, sizeof a);
         a.n = 1;
-        fill_prob(a.p[0], m->wo[l], m->xq_a, m->x, m->x);
+        a.p[0] = make_prob(m->wo[l], m->xq_a, rt::kStageXq, m->x, m->x);
         RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
-        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, m->x, m->ffn_norm[l], nullptr, m->xq_h, 1, H, c.rms_eps));
-        memset(&a, 0, sizeof a);
-        a.n = 2;
-        fill_prob(a.p[0], m->wgate[l], m->xq_h, m->g, nullptr);
-        fill_prob(a.p[1], m->wup[l], m->xq_h, m->u, nullptr);
-        RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
-        RT_TRY_HIP(ctx, rt::launch_swiglu(s, m->g, m->u, nullptr, m->xq_f, F));
         memset(&a, 0, sizeof a);
         a.n = 1;
-        fill_prob(a.p[0], m->wdown[l], m->xq_f, m->x, m->x);
+        a.p[0] = make_prob(m->wgate[l], m->x, rt::kStageRms, m->g, nullptr);
+        a.p[0].w2 = m->wup[l].dev; a.p[0].epi = rt::kEpiSwiglu; a.p[0].gamma = m->ffn_norm[l]; a.p[0].eps = c.rms_eps;
+        RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
+        memset(&a, 0, sizeof a);
+        a.n = 1;
+        a.p[0] = make_prob(m->wdown[l], m->g, rt::kStageF32, m->x, m->x);
         RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
     }
     if (want_logits) {
-        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, m->x, m->out_norm, nullptr, m->xq_h, 1, H, c.rms_eps));
         rt::GemvArgs a;
         memset(&a, 0, sizeof a);
         a.n = 1;
-        fill_prob(a.p[0], m->output, m->xq_h, m->logits, nullptr);
+        a.p[0] = make_prob(m->output, m->x, rt::kStageRms, m->logits, nullptr);
+        a.p[0].gamma = m->out_norm; a.p[0].eps = c.rms_eps;
         RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
     }
     return RT_HIP_OK;
