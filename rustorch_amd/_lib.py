@@ -68,6 +68,7 @@ SIGNATURES = {
     "rt_hip_llama_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
     "rt_hip_llama_upload_tensor": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t]),
     "rt_hip_llama_reset": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "rt_hip_llama_set_mode": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "rt_hip_llama_step": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, c_int_p]),
     "rt_hip_llama_prefill": (C.c_int, [C.c_void_p, C.c_void_p, c_int_p, C.c_int, C.c_int]),
     "rt_hip_llama_logits": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),

@@ -58,6 +58,61 @@ __device__ __forceinline__ float block_max(float v, float *red) {
 }
 
 
+// --------------------------------------------------------- exact block decode
+// One element of a tensor row, evaluated exactly as the block definition is written
+// (f32, no contraction), so a dump of these values can be memcmp'd against the CPU decode.
+#pragma clang fp contract(off)
+__device__ inline float deq_elem(int type, const uint8_t *row, size_t col) {
+    switch (type) {
+    case RT_GGML_F32: { float f; __builtin_memcpy(&f, row + 4 * col, 4); return f; }
+    case RT_GGML_F16: return h2f(ld2u(row + 2 * col));
+    case RT_GGML_Q8_0: {
+        const uint8_t *b = row + 34 * (col >> 5);
+        float d = h2f(ld2u(b));
+        return d * (float)(int)(int8_t)b[2 + (col & 31)];
+    }
+    case RT_GGML_Q4_0: {
+        const uint8_t *b = row + 18 * (col >> 5);
+        float d = h2f(ld2u(b));
+        int j = (int)(col & 31);
+        int q = j < 16 ? (b[2 + j] & 0x0F) : (b[2 + j - 16] >> 4);
+        return (float)(q - 8) * d;
+    }
+    case RT_GGML_Q4_K: {
+        const uint8_t *b = row + 144 * (col >> 8);
+        int e = (int)(col & 255);
+        int j = e >> 5;             // sub-block 0..7
+        int l = e & 31;
+        const uint8_t *s = b + 4;
+        int sc, m;
+        if (j < 4) { sc = s[j] & 63; m = s[j + 4] & 63; }
+        else { sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4); m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4); }
+        float d = h2f(ld2u(b)) * (float)sc;
+        float mn = h2f(ld2u(b + 2)) * (float)m;
+        uint8_t qb = b[16 + 32 * (j >> 1) + l];
+        int q = (j & 1) ? (qb >> 4) : (qb & 0x0F);
+        return d * (float)q - mn;
+    }
+    case RT_GGML_Q6_K: {
+        const uint8_t *b = row + 210 * (col >> 8);
+        int e = (int)(col & 255);
+        int h = e >> 7;             // half 0..1
+        int r = (e >> 5) & 3;       // 32-run within the half
+        int l = e & 31;
+        const uint8_t *ql = b + 64 * h, *qh = b + 128 + 32 * h;
+        const int8_t *sc = (const int8_t *)(b + 192 + 8 * h);
+        uint8_t lo = ql[l + 32 * (r & 1)];
+        int nib = (r & 2) ? (lo >> 4) : (lo & 0x0F);
+        int q = (nib | (((qh[l] >> (2 * r)) & 3) << 4)) - 32;
+        float d = h2f(ld2u(b + 208));
+        return d * (float)(int)sc[(l >> 4) + 2 * r] * (float)q;
+    }
+    }
+    return 0.f;
+}
+
+#pragma clang fp contract(fast)
+
 // Activation accesses that must be coherent across XCDs inside one launch (COH) go out as device-scope
 // relaxed atomics, which bypass the per-XCD L2; otherwise they are plain cached accesses.
 template <bool COH> __device__ __forceinline__ float ld_f(const float *p) {

@@ -19,7 +19,7 @@ __global__ __launch_bounds__(kGemvThreads) void qgemv_kernel(GemvArgs a, int r2)
     for (int i = 1; i < kMaxGemvProbs; i++)
         if (i < a.n && wg >= a.p[i].tile0) pi = i;
     const GemvProb &P = a.p[pi];
-    gemv_dispatch<false>(P, wg - P.tile0, P.rows_per_tile, blockIdx.y, r2 != 0, lds, red);
+    gemv_dispatch<false, true>(P, wg - P.tile0, P.rows_per_tile, blockIdx.y, r2 != 0, lds, red);
 }
 
 }  // namespace

@@ -363,7 +363,7 @@ __device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
     XRegs<TYPE> x;
-    if (W.n_iter == 1) {
+    if (R == 1 && W.n_iter == 1) {
         // every step of this lane meets the same x slice: keep it in registers, LDS is read once
         W.fetch_x(x, 0);
         for (int s = 0; s < steps; s += 2) {
@@ -389,9 +389,9 @@ __device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg
 }
 
 // Dispatch on the block format.  R2 picks two rows per wave step (always used by the SwiGLU epilogue).
-template <bool COH>
+template <bool COH, bool ALLOW_R2>
 __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_wg, int m, bool r2, uint32_t *lds, float *red) {
-    if (r2 || P.epi == kEpiSwiglu) {
+    if ((ALLOW_R2 && r2) || P.epi == kEpiSwiglu) {
         switch (P.type) {
         case RT_GGML_Q4_K: gemv_problem<RT_GGML_Q4_K, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q6_K: gemv_problem<RT_GGML_Q6_K, 2, COH>(P, wg, n_wg, m, lds, red); break;

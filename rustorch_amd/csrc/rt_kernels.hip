@@ -12,59 +12,7 @@
 
 namespace rt {
 
-// --------------------------------------------------------- exact block decode
-// One element of a tensor row, evaluated exactly as the block definition is written
-// (f32, no contraction), so a dump of these values can be memcmp'd against the CPU decode.
 #pragma clang fp contract(off)
-__device__ float deq_elem(int type, const uint8_t *row, size_t col) {
-    switch (type) {
-    case RT_GGML_F32: { float f; __builtin_memcpy(&f, row + 4 * col, 4); return f; }
-    case RT_GGML_F16: return h2f(ld2u(row + 2 * col));
-    case RT_GGML_Q8_0: {
-        const uint8_t *b = row + 34 * (col >> 5);
-        float d = h2f(ld2u(b));
-        return d * (float)(int)(int8_t)b[2 + (col & 31)];
-    }
-    case RT_GGML_Q4_0: {
-        const uint8_t *b = row + 18 * (col >> 5);
-        float d = h2f(ld2u(b));
-        int j = (int)(col & 31);
-        int q = j < 16 ? (b[2 + j] & 0x0F) : (b[2 + j - 16] >> 4);
-        return (float)(q - 8) * d;
-    }
-    case RT_GGML_Q4_K: {
-        const uint8_t *b = row + 144 * (col >> 8);
-        int e = (int)(col & 255);
-        int j = e >> 5;             // sub-block 0..7
-        int l = e & 31;
-        const uint8_t *s = b + 4;
-        int sc, m;
-        if (j < 4) { sc = s[j] & 63; m = s[j + 4] & 63; }
-        else { sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4); m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4); }
-        float d = h2f(ld2u(b)) * (float)sc;
-        float mn = h2f(ld2u(b + 2)) * (float)m;
-        uint8_t qb = b[16 + 32 * (j >> 1) + l];
-        int q = (j & 1) ? (qb >> 4) : (qb & 0x0F);
-        return d * (float)q - mn;
-    }
-    case RT_GGML_Q6_K: {
-        const uint8_t *b = row + 210 * (col >> 8);
-        int e = (int)(col & 255);
-        int h = e >> 7;             // half 0..1
-        int r = (e >> 5) & 3;       // 32-run within the half
-        int l = e & 31;
-        const uint8_t *ql = b + 64 * h, *qh = b + 128 + 32 * h;
-        const int8_t *sc = (const int8_t *)(b + 192 + 8 * h);
-        uint8_t lo = ql[l + 32 * (r & 1)];
-        int nib = (r & 2) ? (lo >> 4) : (lo & 0x0F);
-        int q = (nib | (((qh[l] >> (2 * r)) & 3) << 4)) - 32;
-        float d = h2f(ld2u(b + 208));
-        return d * (float)(int)sc[(l >> 4) + 2 * r] * (float)q;
-    }
-    }
-    return 0.f;
-}
-
 __global__ void dequant_kernel(int type, const uint8_t *w, size_t row_bytes, size_t n_rows, size_t n_cols, float *out) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     size_t total = n_rows * n_cols;
@@ -384,6 +332,11 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *v, size_t n, 
 }
 
 __global__ void set_int_kernel(int *dst, int value) { *dst = value; }
+__global__ void set_state_kernel(int *state, int pos, int token, int step) {
+    state[0] = pos;
+    state[1] = token;
+    state[3] = step;
+}
 
 // End of a decode step: record the pick, choose the next input token, advance the position.
 __global__ void step_advance_kernel(int *pos_dev, int *token_dev, const int *pick_dev, const int *forced_dev,
@@ -520,6 +473,11 @@ hipError_t launch_matmul_f32(hipStream_t s, const float *a, const float *b, floa
     if (m == 0 || n == 0) return hipSuccess;
     dim3 grid((unsigned)((n + 31) / 32), (unsigned)((m + 31) / 32));
     matmul_f32_kernel<<<grid, dim3(32, 32), 0, s>>>(a, b, c, m, n, k);
+    return hipGetLastError();
+}
+
+hipError_t launch_set_state(hipStream_t s, int *state, int pos, int token, int step) {
+    set_state_kernel<<<1, 1, 0, s>>>(state, pos, token, step);
     return hipGetLastError();
 }
 

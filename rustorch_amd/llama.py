@@ -29,6 +29,10 @@ class HipLlama:
         _lib.check(self.ex.lib.rt_hip_llama_upload_tensor(self.ex.ctx, self.h, SLOT[slot], layer, int(ggml_type), n_rows,
                                                           n_cols, C.c_void_p(raw.ctypes.data), raw.nbytes), self.ex.ctx)
 
+    def set_mode(self, mode: int) -> None:
+        """1 = one launch per operator group (default); 0 = one persistent launch per token (switched off in this build)."""
+        _lib.check(self.ex.lib.rt_hip_llama_set_mode(self.ex.ctx, self.h, mode), self.ex.ctx)
+
     def reset(self) -> None:
         _lib.check(self.ex.lib.rt_hip_llama_reset(self.ex.ctx, self.h), self.ex.ctx)
 

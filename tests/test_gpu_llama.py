@@ -27,11 +27,15 @@ def logit_tol(wn, hidden):
     return 1e-3 * wn * np.sqrt(hidden)
 
 
-def test_small_model_teacher_forced(ex, orc):
+@pytest.mark.parametrize("mode", [
+    pytest.param(0, marks=pytest.mark.skip(reason="persistent step kernel switched off: GPU memory fault on first run, cause not found")),
+    1])
+def test_small_model_teacher_forced(ex, orc, mode):
     from rustorch_amd import synth
     cfg = dict(n_layers=3, hidden=512, n_heads=4, ffn=1024, vocab=1000, max_pos=48)
-    print("llama small", cfg, flush=True)
+    print("llama small", cfg, "mode", mode, flush=True)
     gm, om, wn = build_pair(ex, orc, 17, **cfg)
+    gm.set_mode(mode)
     toks = synth.tokens(17, synth.TID_PROMPT, 40, cfg["vocab"])
     want = om.forward(toks, 0)                                  # [40, vocab]
     tol = logit_tol(wn, cfg["hidden"])
@@ -55,11 +59,15 @@ def test_small_model_teacher_forced(ex, orc):
     assert np.all(np.abs(gm.logits() - want[25]) <= tol)
 
 
-def test_decode_loop_without_host_round_trips(ex, orc):
+@pytest.mark.parametrize("mode", [
+    pytest.param(0, marks=pytest.mark.skip(reason="persistent step kernel switched off: GPU memory fault on first run, cause not found")),
+    1])
+def test_decode_loop_without_host_round_trips(ex, orc, mode):
     from rustorch_amd import synth, InvalidParameters, ShapeMismatch
     cfg = dict(n_layers=2, hidden=256, n_heads=2, ffn=512, vocab=300, max_pos=32)
-    print("llama decode loop", cfg, flush=True)
+    print("llama decode loop", cfg, "mode", mode, flush=True)
     gm, om, wn = build_pair(ex, orc, 23, **cfg)
+    gm.set_mode(mode)
     prompt = synth.tokens(23, synth.TID_PROMPT, 8, cfg["vocab"])
     # greedy, stepping from the host
     picks = []
@@ -100,3 +108,11 @@ def test_incomplete_model_is_an_error(ex):
         gm.step(0, 0)
     with pytest.raises(ShapeMismatch):
         gm.upload("attn_q", 0, 12, 256, 512, synth.blocks(12, 1, 1, 256, 512))
+
+
+def test_persistent_mode_is_refused_not_silently_replaced(ex):
+    from rustorch_amd import llama, UnsupportedOperation
+    gm = llama.HipLlama(ex, 1, 256, 2, 256, 64, 8)
+    gm.set_mode(1)
+    with pytest.raises(UnsupportedOperation):
+        gm.set_mode(0)
