@@ -5,6 +5,12 @@
 
 #include <hip/hip_fp16.h>
 
+// The launch-sized LDS region of a kernel.  A CPU build of the device code (bounds / race checking) predefines
+// this macro to hand out its own per-workgroup buffer.
+#ifndef RT_DYN_LDS
+#define RT_DYN_LDS(T, name) extern __shared__ T name[]
+#endif
+
 namespace rt {
 
 

@@ -10,7 +10,7 @@ constexpr int kGemvThreads = 1024;
 constexpr int kGemvWaves = kGemvThreads / 64;
 
 __global__ __launch_bounds__(kGemvThreads) void qgemv_kernel(GemvArgs a, int r2) {
-    extern __shared__ uint4 lds4[];
+    RT_DYN_LDS(uint4, lds4);
     __shared__ float red[kGemvWaves];
     uint32_t *lds = reinterpret_cast<uint32_t *>(lds4);
     const int wg = blockIdx.x;

@@ -96,7 +96,16 @@ struct MegaArgs {
 };
 constexpr size_t kMegaBarBytes = 4096;
 constexpr size_t kMegaErrWord = 32 * 24;  // index of the time-out flag inside the barrier words
-size_t mega_lds_bytes(int hidden, int ffn, int head_dim, int max_pos);
+constexpr int kMegaThreads = 1024;
+// Launch-sized LDS of the step kernel: the larger of the GEMV staging area, the attention phase
+// (q / k / v of the step, per-group partial outputs, scores) and the greedy-pick scratch.
+inline size_t mega_lds_bytes(int hidden, int ffn, int head_dim, int max_pos) {
+    size_t g = xq_stride((size_t)(hidden > ffn ? hidden : ffn));
+    size_t a = ((size_t)3 * head_dim + (size_t)(kMegaThreads / (head_dim / 8)) * head_dim + (size_t)max_pos) * sizeof(float);
+    size_t m = g > a ? g : a;
+    size_t am = (size_t)2 * kMegaThreads * sizeof(float);
+    return m > am ? m : am;
+}
 int mega_grid(int device, size_t lds_bytes);
 hipError_t launch_llama_step(hipStream_t s, MegaArgs &a, int grid, size_t lds_bytes);
 hipError_t launch_set_state(hipStream_t s, int *state, int pos, int token, int step);

@@ -188,7 +188,7 @@ template <int HD, bool FUSED>
 __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float *k, const float *v, uint16_t *kc,
                                                           uint16_t *vc, const int *pos_dev, int n_pos_arg, int n_heads,
                                                           const float *inv_freq, float *out, uint8_t *xq) {
-    extern __shared__ float sc[];
+    RT_DYN_LDS(float, sc);
     __shared__ float red[4];
     __shared__ __align__(16) float qs[HD];
     __shared__ __align__(16) float kcur[HD];
