@@ -116,6 +116,35 @@ def bench_decode(ex, n_prompt, n_gen):
                 n_prompt=n_prompt, n_generated=n_gen, first_tokens=[int(t) for t in toks[:8]])
 
 
+def bench_prefill(ex, reps=20):
+    """Config C4: Y = X . dequant(W)^T on the matrix cores, X resident in HBM; 2MNK flops against the fp16 MFMA peak."""
+    from rustorch_amd import synth, GGMLType
+    MFMA_PEAK = 2.5e15
+    out = []
+    for name, t, rows, cols in (("q4k_4096x4096", GGMLType.Q4_K, 4096, 4096), ("q4k_11008x4096", GGMLType.Q4_K, 11008, 4096),
+                                ("q6k_4096x11008", GGMLType.Q6_K, 4096, 11008)):
+        w = ex.upload_qweight(t, rows, cols, synth.blocks(t, SEED, 7000 + rows + cols, rows, cols))
+        for M in (64, 512, 2048):
+            x = ex.to_device(synth.normal(SEED, 7100 + M, M * cols))
+            y = ex.buffer(4 * M * rows)
+            for _ in range(3):
+                ex.qgemm_dev(w, x, M, y)
+            ex.synchronize()
+            e0, e1 = ex.event(), ex.event()
+            e0.record()
+            for _ in range(reps):
+                ex.qgemm_dev(w, x, M, y)
+            e1.record()
+            ex.synchronize()
+            ms = e0.elapsed_ms(e1) / reps
+            flops = 2.0 * M * rows * cols
+            out.append({"shape": name, "M": M, "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                        "mfma_frac": round(flops / (ms * 1e-3) / MFMA_PEAK, 4)})
+            x.free(); y.free()
+        w.free()
+    return out
+
+
 def cpu_baseline(reps):
     """Reference CPU path for one layer: dequantize each tensor to dense f32, then x . W^T with sequential k-sums."""
     from oracle import oracle as orc
@@ -146,6 +175,7 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="distinct synthetic layers rotated through (32 = 4.15 GB)")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--decode-prompt", type=int, default=128)
     ap.add_argument("--decode-gen", type=int, default=128)
     args = ap.parse_args()
@@ -173,6 +203,8 @@ def main():
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": None, "kernel": "qgemv_kernel",
                      "bytes_per_launch": g["abytes"], "avg_launch_ms": round(g["kernel_ms"], 5)},
     }
+    if not args.no_prefill:
+        out["prefill"] = bench_prefill(ex)
     if not args.no_decode:
         out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen)
     ex.close()

@@ -28,6 +28,7 @@ SOURCES = ["rt_api.hip", "rt_kernels.hip", "rt_gemv.hip", "rt_mega.hip", "rt_gem
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-munsafe-fp-atomics",  # f32 atomic adds of the split-k GEMM epilogue as hardware atomics (device memory only)
     "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]
 

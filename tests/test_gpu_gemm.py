@@ -1,0 +1,88 @@
+"""Prefill contraction (MFMA path) against the oracle.
+
+Bound stated by the benchmark: max |delta| <= 1e-3 * ||w_row||_2 * ||x_row||_2 per element.  The fp16 operands
+of the matrix cores keep the kernel about 20x inside it; the test holds it to 1e-4 at K = 4096 (scaled by sqrt(4096/K))."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-3
+HELD = 1e-4
+
+
+def check(Y, rows, toks, raw, t, n_rows, n_cols, X, orc, what):
+    """Compare Y[toks][:, rows] with the f64 yardstick on the sampled weight rows / tokens."""
+    rb = len(raw) // n_rows
+    worst = 0.0
+    for r0, r1 in rows:
+        sub = raw[r0 * rb:r1 * rb]
+        y64, wn = orc.qgemv_f64(t, sub, r1 - r0, n_cols, X[toks])
+        xn = np.linalg.norm(X[toks].astype(np.float64), axis=1)[:, None]
+        ratio = np.abs(Y[toks][:, r0:r1] - y64) / (wn[None, :] * xn)
+        worst = max(worst, float(ratio.max()))
+    print("%s: max |delta| / (||w|| ||x||) = %.3e (bound %.0e, held to %.0e)" % (what, worst, REL_TOL, HELD), flush=True)
+    assert np.isfinite(Y).all()
+    assert worst <= HELD
+
+
+CASES = [
+    ("q4k_4096x4096", 12, 4096, 4096),
+    ("q4k_11008x4096", 12, 11008, 4096),
+    ("q6k_4096x11008", 14, 4096, 11008),
+]
+
+
+@pytest.mark.parametrize("name,t,rows,cols", CASES)
+@pytest.mark.parametrize("M", [64, 512, 2048])
+def test_prefill_shapes(ex, orc, name, t, rows, cols, M):
+    from rustorch_amd import synth
+    print("gemm", name, "M", M, flush=True)
+    raw = synth.blocks(t, 31, 7, rows, cols)
+    w = ex.upload_qweight(t, rows, cols, raw)
+    X = synth.normal(31, 100 + M, M * cols).reshape(M, cols)
+    Y = ex.qgemm(w, X)
+    assert Y.shape == (M, rows)
+    rng = np.random.default_rng(M)
+    toks = np.sort(rng.choice(M, size=min(M, 48), replace=False))
+    starts = sorted(set([0, rows - 64] + [int(v) for v in rng.integers(0, rows - 64, 4)]))
+    check(Y, [(s, s + 64) for s in starts], toks, raw, t, rows, cols, X, orc, "%s M=%d" % (name, M))
+
+
+@pytest.mark.parametrize("t", [12, 14])
+def test_ragged_and_scaled_inputs(ex, orc, t):
+    from rustorch_amd import synth
+    rows, cols = 1000, 1024                         # N not a multiple of the tile, several k splits
+    raw = synth.blocks(t, 32, 1, rows, cols)
+    w = ex.upload_qweight(t, rows, cols, raw)
+    for M in (16, 17, 100, 300):
+        print("gemm ragged type", t, "M", M, flush=True)
+        X = synth.normal(32, M, M * cols).reshape(M, cols).copy()
+        X[0] *= 3e5                                 # beyond the fp16 range before row scaling
+        X[1] *= 1e-20
+        X[2] = 0
+        X[3, 5:] = 0                                # one non-zero element
+        Y = ex.qgemm(w, X)
+        y64, wn = orc.qgemv_f64(t, raw, rows, cols, X)
+        xn = np.linalg.norm(X.astype(np.float64), axis=1)[:, None]
+        xn[xn == 0] = 1
+        ratio = np.abs(Y - y64) / (wn[None, :] * xn)
+        held = HELD * np.sqrt(4096 / cols)          # the rounding noise of the fp16 operands averages as 1/sqrt(K)
+        assert np.isfinite(Y).all() and ratio.max() <= held, (M, ratio.max())
+        assert not Y[2].any()
+        # a GEMM row is the GEMV of that token, to rounding of the two paths
+        for m in (0, 4, M - 1):
+            yv = ex.qgemv(w, X[m])
+            assert np.all(np.abs(Y[m] - yv) <= 2 * held * wn * xn[m])
+
+
+def test_other_formats_and_small_m_use_the_row_form(ex, orc):
+    from rustorch_amd import synth
+    for t, cols in ((8, 512), (2, 512), (12, 512)):
+        raw = synth.blocks(t, 33, t, 96, cols)
+        w = ex.upload_qweight(t, 96, cols, raw)
+        for M in (1, 9, 40):
+            X = synth.normal(33, M, M * cols).reshape(M, cols)
+            y64, wn = orc.qgemv_f64(t, raw, 96, cols, X)
+            xn = np.linalg.norm(X.astype(np.float64), axis=1)[:, None]
+            assert (np.abs(ex.qgemm(w, X) - y64) / (wn[None, :] * xn)).max() <= HELD * np.sqrt(4096 / cols)
