@@ -178,6 +178,9 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--decode-prompt", type=int, default=128)
     ap.add_argument("--decode-gen", type=int, default=128)
+    ap.add_argument("--calibrate", action="store_true",
+                    help="run only a plain x += y kernel over 2 x 128 MiB (reads 256 MiB, writes 128 MiB per launch): "
+                         "the known-size launch that hardware traffic counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (use --gpus 1)" % args.gpus)
@@ -186,6 +189,17 @@ def main():
     ex = HipKernelExecutor(0)
     info = ex.device_info()
     log("[bench] device:", info)
+
+    if args.calibrate:
+        n = 32 << 20
+        a, b = ex.buffer(4 * n), ex.buffer(4 * n)
+        a.zero(); b.zero()
+        for _ in range(8):
+            ex.add_dev(a, b, n)
+        ex.synchronize()
+        print(json.dumps({"calibrate": "add_kernel", "launches": 8, "read_bytes_per_launch": 8 * n, "write_bytes_per_launch": 4 * n}), flush=True)
+        ex.close()
+        return
 
     g = bench_layer_gemv(ex, args.steps, args.warmup, args.layers)
     ms_per_step = 1e3 * g["wall_s"] / args.steps

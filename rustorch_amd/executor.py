@@ -306,6 +306,10 @@ class HipKernelExecutor:
         _lib.check(self.lib.rt_hip_add_dev(self.ctx, dx.ptr, dy.ptr, x.size), self.ctx)
         return dx.download(np.float32).reshape(x.shape)
 
+    def add_dev(self, x: DeviceBuffer, y: DeviceBuffer, n: int) -> None:
+        """x[i] += y[i] for n f32 values, both resident on the device."""
+        _lib.check(self.lib.rt_hip_add_dev(self.ctx, x.ptr, y.ptr, n), self.ctx)
+
     def argmax(self, v) -> int:
         v = _f32(v, "v")
         dv = self.to_device(v)

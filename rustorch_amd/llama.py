@@ -97,3 +97,91 @@ def load_synthetic(model: HipLlama, seed: int, sink: Callable | None = None) -> 
         if t != GGMLType.F32:
             total += raw.nbytes
     return total
+
+
+# ---- GGUF model files: llama tensor names and metadata keys -> the upload slots above
+
+_GLOBAL_NAMES = {"token_embd.weight": "token_embd", "output.weight": "output", "output_norm.weight": "output_norm"}
+_LAYER_NAMES = {"attn_q": "attn_q", "attn_k": "attn_k", "attn_v": "attn_v", "attn_output": "attn_output", "ffn_gate": "ffn_gate",
+                "ffn_up": "ffn_up", "ffn_down": "ffn_down", "attn_norm": "attn_norm", "ffn_norm": "ffn_norm"}
+
+
+def gguf_tensor_name(slot: str, layer: int) -> str:
+    return "%s.weight" % slot if layer < 0 else "blk.%d.%s.weight" % (layer, slot)
+
+
+def write_synthetic_gguf(path, seed: int, n_layers: int, hidden: int, n_heads: int, ffn: int, vocab: int, context: int,
+                         rms_eps: float = 1e-5, rope_theta: float = 10000.0) -> None:
+    """A random-init Llama as a GGUF v3 file (same tensors as `synthetic_tensors`), so the file path can be
+    exercised without a downloaded model."""
+    from . import gguf
+    w = gguf.GGUFWriter()
+    w.add_kv("general.architecture", gguf.VT_STRING, "llama")
+    w.add_kv("general.name", gguf.VT_STRING, "synthetic-llama-seed-%d" % seed)
+    w.add_kv("llama.block_count", gguf.VT_UINT32, n_layers)
+    w.add_kv("llama.context_length", gguf.VT_UINT32, context)
+    w.add_kv("llama.embedding_length", gguf.VT_UINT32, hidden)
+    w.add_kv("llama.feed_forward_length", gguf.VT_UINT32, ffn)
+    w.add_kv("llama.attention.head_count", gguf.VT_UINT32, n_heads)
+    w.add_kv("llama.attention.head_count_kv", gguf.VT_UINT32, n_heads)
+    w.add_kv("llama.attention.layer_norm_rms_epsilon", gguf.VT_FLOAT32, rms_eps)
+    w.add_kv("llama.rope.freq_base", gguf.VT_FLOAT32, rope_theta)
+    for slot, layer, t, r, c, raw in synthetic_tensors(seed, n_layers, hidden, ffn, vocab):
+        dims = (c,) if t == GGMLType.F32 else (c, r)
+        w.add_tensor(gguf_tensor_name(slot, layer), t, dims, raw)
+    w.write(path)
+
+
+def load_gguf(ex: HipKernelExecutor, path, max_pos: int | None = None) -> HipLlama:
+    """Build a device model from a llama-architecture GGUF file: hyper-parameters from the metadata keys,
+    every tensor's raw bytes uploaded as stored (what the reference's `load_gguf` stub,
+    example-cli/src/model/loader.rs:55-59, leaves open)."""
+    from . import gguf
+    from .errors import InvalidParameters, UnsupportedOperation
+    with gguf.GGUFLoader(path) as g:
+        arch = g.get_metadata("general.architecture")
+        if arch is None or arch.as_str() != "llama":
+            raise UnsupportedOperation("load_gguf: architecture %r is not llama" % (arch.as_str() if arch else None))
+
+        def need_u32(key):
+            v = g.get_metadata(key)
+            if v is None or v.as_u32() is None:
+                raise InvalidParameters("load_gguf: metadata key %s missing or not an unsigned integer" % key)
+            return v.as_u32()
+
+        def opt_f32(key, default):
+            v = g.get_metadata(key)
+            return default if v is None or v.as_f32() is None else float(v.as_f32())
+
+        n_layers, hidden = need_u32("llama.block_count"), need_u32("llama.embedding_length")
+        ffn, n_heads = need_u32("llama.feed_forward_length"), need_u32("llama.attention.head_count")
+        kv = g.get_metadata("llama.attention.head_count_kv")
+        if kv is not None and kv.as_u32() not in (None, n_heads):
+            raise UnsupportedOperation("load_gguf: grouped-query attention (head_count_kv=%d) is not supported" % kv.as_u32())
+        emb = g.find_tensor("token_embd.weight")
+        if emb is None or emb.n_dims != 2:
+            raise InvalidParameters("load_gguf: token_embd.weight missing or not 2-D")
+        vocab = emb.dims[1]
+        ctx = g.get_metadata("llama.context_length")
+        if max_pos is None:
+            max_pos = ctx.as_u32() if ctx is not None and ctx.as_u32() else 2048
+        model = HipLlama(ex, n_layers, hidden, n_heads, ffn, vocab, max_pos, opt_f32("llama.attention.layer_norm_rms_epsilon", 1e-5),
+                         opt_f32("llama.rope.freq_base", 10000.0))
+        try:
+            wanted = [(s, -1) for s in ("token_embd", "output", "output_norm")] + [(s, l) for l in range(n_layers) for s in _LAYER_NAMES]
+            for slot, layer in wanted:
+                name = gguf_tensor_name(slot, layer)
+                t = g.find_tensor(name)
+                if t is None and slot == "output":
+                    t, name = emb, "token_embd.weight"          # tied embeddings: the head reuses the embedding matrix
+                if t is None:
+                    raise InvalidParameters("load_gguf: tensor %s missing" % name)
+                raw = g.load_tensor_data(name)
+                if slot.endswith("norm"):
+                    model.upload(slot, layer, GGMLType.F32, 1, t.n_cols, g.load_f32(name))
+                else:
+                    model.upload(slot, layer, t.ggml_type, t.n_rows, t.n_cols, raw)
+        except Exception:
+            model.close()
+            raise
+        return model

@@ -116,3 +116,31 @@ def test_persistent_mode_is_refused_not_silently_replaced(ex):
     gm.set_mode(1)
     with pytest.raises(UnsupportedOperation):
         gm.set_mode(0)
+
+
+def test_model_from_gguf_file_equals_direct_upload(ex, orc, tmp_path):
+    """write a synthetic llama GGUF, load it through the container parser, compare with the oracle and with
+    the model whose tensors were uploaded directly: same bytes on the device, so identical logits."""
+    from rustorch_amd import llama, synth, InvalidParameters
+    cfg = dict(n_layers=2, hidden=256, n_heads=2, ffn=512, vocab=128)
+    print("llama from gguf", cfg, flush=True)
+    p = tmp_path / "tiny.gguf"
+    llama.write_synthetic_gguf(p, 31, context=24, **cfg)
+    gf = llama.load_gguf(ex, p)
+    assert (gf.cfg.n_layers, gf.cfg.hidden, gf.cfg.n_heads, gf.cfg.ffn, gf.cfg.vocab, gf.cfg.max_pos) == (2, 256, 2, 512, 128, 24)
+    gm, om, wn = build_pair(ex, orc, 31, max_pos=24, **cfg)
+    toks = synth.tokens(31, synth.TID_PROMPT, 10, cfg["vocab"])
+    want = om.forward(toks, 0)
+    tol = logit_tol(wn, cfg["hidden"])
+    for pos, t in enumerate(toks):
+        a, b = gf.step(int(t), pos), gm.step(int(t), pos)
+        la, lb = gf.logits(), gm.logits()
+        assert a == b and np.array_equal(la, lb)
+        assert np.all(np.abs(la - want[pos]) <= tol)
+    # a file without the block count is an error, not a guess
+    from rustorch_amd import gguf
+    w = gguf.GGUFWriter()
+    w.add_kv("general.architecture", gguf.VT_STRING, "llama")
+    w.write(tmp_path / "empty.gguf")
+    with pytest.raises(InvalidParameters):
+        llama.load_gguf(ex, tmp_path / "empty.gguf")
