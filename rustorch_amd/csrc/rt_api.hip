@@ -447,7 +447,7 @@ int rt_hip_qgemm_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *X_de
     RT_REQUIRE(ctx, M >= 1 && M <= 65535, RT_HIP_ERR_SHAPE, "qgemm: M=%zu outside 1..65535", M);
     RT_REQUIRE(ctx, rt::xq_stride(w->n_cols) <= 64 * 1024, RT_HIP_ERR_SHAPE, "qgemm: n_cols=%zu too large", w->n_cols);
     Guard g(ctx);
-    size_t sb = rt::qgemm_scratch_bytes(M, w->n_cols);
+    size_t sb = rt::qgemm_scratch_bytes(w->type, M, w->n_rows, w->n_cols);
     int rc = ensure_scratch(ctx, sb);
     if (rc) return rc;
     RT_TRY_HIP(ctx, rt::launch_qgemm(ctx->stream, w->type, w->dev, w->n_rows, w->n_cols, w->row_bytes, X_dev, M, Y_dev,
@@ -462,7 +462,7 @@ int rt_hip_qgemm(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *X, size_
     RT_REQUIRE(ctx, rt::xq_stride(w->n_cols) <= 64 * 1024, RT_HIP_ERR_SHAPE, "qgemm: n_cols=%zu too large", w->n_cols);
     Guard g(ctx);
     size_t xb = align_up(M * w->n_cols * 4, 256), yb = align_up(M * w->n_rows * 4, 256);
-    size_t sb = rt::qgemm_scratch_bytes(M, w->n_cols);
+    size_t sb = rt::qgemm_scratch_bytes(w->type, M, w->n_rows, w->n_cols);
     int rc = ensure_scratch(ctx, xb + yb + sb);
     if (rc) return rc;
     char *base = (char *)ctx->scratch;
