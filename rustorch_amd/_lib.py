@@ -2,12 +2,14 @@
 from __future__ import annotations
 
 import ctypes as C
+import os
 from pathlib import Path
 
 from . import errors
 
 _PKG = Path(__file__).resolve().parent
-LIB_PATH = _PKG / "librustorch_hip.so"
+# RUSTORCH_HIP_LIBRARY names another build of the same library (a differently tuned or instrumented one)
+LIB_PATH = Path(os.environ["RUSTORCH_HIP_LIBRARY"]) if os.environ.get("RUSTORCH_HIP_LIBRARY") else _PKG / "librustorch_hip.so"
 
 c_void_pp = C.POINTER(C.c_void_p)
 c_float_p = C.POINTER(C.c_float)

@@ -29,6 +29,7 @@
 #include "rt_device.h"
 
 #include <algorithm>
+#include <type_traits>
 #include <cstring>
 
 namespace rt {
@@ -41,21 +42,43 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ u32x4 ldg16(const uint8_t *p) { u32x4 v; __builtin_memcpy(&v, p, 16); return v; }
-__device__ __forceinline__ u32x4 ldg16a(const uint8_t *p) { return *reinterpret_cast<const u32x4 *>(p); }
 
 constexpr int kBK = 64;          // k per tile
 constexpr int kMaxSplit = 8;     // most k splits of one launch
 
-// ---- pre-pass: X f32 [M,K] -> fp16, row-scaled, k-permuted; inv_scale[m] undoes the row scale
+// ---- pre-pass: X f32 [M,K] -> fp16, row-scaled, k-permuted; inv_scale[m] undoes the row scale.
+// One workgroup per row; output chunk g (8 halves) is the aligned group of 8 floats at
+// 64*(g>>3) + 32*(s>>1) + 16*h + 8*(s&1) with s = (g&7)>>1, h = g&1, its elements in the order 0,2,1,3,4,6,5,7.
+// A thread keeps its (up to kXprepChunks) groups in registers between the maximum and the conversion, so the
+// row is read once; longer rows take the groups beyond that from memory again.
+constexpr int kXprepChunks = 6;
 __global__ __launch_bounds__(256) void xprep_kernel(const float *X, size_t K, _Float16 *Xp, float *inv_scale) {
     __shared__ float red[4];
     const size_t m = blockIdx.x;
     const float *x = X + m * K;
+    const size_t n_chunks = K / 8;
+    auto src_of = [](size_t g) {
+        const int sh = (int)(g & 7), s = sh >> 1, h = sh & 1;
+        return 64 * (g >> 3) + 32 * (size_t)(s >> 1) + 16 * (size_t)h + 8 * (size_t)(s & 1);
+    };
+    float4 lo[kXprepChunks], hi[kXprepChunks];
     float amax = 0.f;
-    for (size_t i = threadIdx.x; i < K / 4; i += blockDim.x) {
-        float4 v = reinterpret_cast<const float4 *>(x)[i];
-        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+#pragma unroll
+    for (int j = 0; j < kXprepChunks; j++) {
+        const size_t g = threadIdx.x + 256 * (size_t)j;
+        if (g < n_chunks) {
+            const float4 *p = reinterpret_cast<const float4 *>(x + src_of(g));
+            lo[j] = p[0];
+            hi[j] = p[1];
+            amax = fmaxf(amax, fmaxf(fmaxf(fmaxf(fabsf(lo[j].x), fabsf(lo[j].y)), fmaxf(fabsf(lo[j].z), fabsf(lo[j].w))),
+                                     fmaxf(fmaxf(fabsf(hi[j].x), fabsf(hi[j].y)), fmaxf(fabsf(hi[j].z), fabsf(hi[j].w)))));
+        }
+    }
+    for (size_t g = threadIdx.x + 256 * (size_t)kXprepChunks; g < n_chunks; g += 256) {
+        const float4 *p = reinterpret_cast<const float4 *>(x + src_of(g));
+        const float4 a = p[0], b = p[1];
+        amax = fmaxf(amax, fmaxf(fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))),
+                                 fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w)))));
     }
     amax = block_max(amax, red);
     int e = 0;
@@ -68,44 +91,146 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float *X, size_t K, _F
         inv = ldexpf(1.f, -se);
     }
     if (threadIdx.x == 0) inv_scale[m] = inv;
-    const int perm[8] = { 0, 2, 1, 3, 4, 6, 5, 7 };
-    for (size_t g = threadIdx.x; g < K / 8; g += blockDim.x) {
-        size_t kt = g >> 3;
-        int sh = (int)(g & 7), s = sh >> 1, h = sh & 1;
-        size_t src = 64 * kt + 32 * (size_t)(s >> 1) + 16 * (size_t)h + 8 * (size_t)(s & 1);
-        float4 a = reinterpret_cast<const float4 *>(x + src)[0], b = reinterpret_cast<const float4 *>(x + src)[1];
-        const float v[8] = { a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w };
-        half8v o;
-#pragma unroll
-        for (int i = 0; i < 8; i++) o[i] = (_Float16)(v[perm[i]] * scale);
+    auto emit = [&](size_t g, const float4 &a, const float4 &b) {
+        half8v o = { (_Float16)(a.x * scale), (_Float16)(a.z * scale), (_Float16)(a.y * scale), (_Float16)(a.w * scale),
+                     (_Float16)(b.x * scale), (_Float16)(b.z * scale), (_Float16)(b.y * scale), (_Float16)(b.w * scale) };
         *reinterpret_cast<half8v *>(Xp + m * K + 8 * g) = o;
+    };
+#pragma unroll
+    for (int j = 0; j < kXprepChunks; j++) {
+        const size_t g = threadIdx.x + 256 * (size_t)j;
+        if (g < n_chunks) emit(g, lo[j], hi[j]);
+    }
+    for (size_t g = threadIdx.x + 256 * (size_t)kXprepChunks; g < n_chunks; g += 256) {
+        const float4 *p = reinterpret_cast<const float4 *>(x + src_of(g));
+        emit(g, p[0], p[1]);
     }
 }
 
-// ---- raw weight bytes of one lane (weight row nl, k half h) for one super-block of 256 k
+// ---- weights of one super-block (256 k) on their way to the lanes that expand them
+//
+// MFMA lane (nl, h) needs bytes of weight row nl only, and rows lie row_bytes apart: loading them lane by
+// lane touches 32 cache lines per instruction and the address path becomes the bottleneck.  So a wave fetches
+// its 32 row-blocks as consecutive 16-byte chunks (chunk c = 64 i + lane of instruction i; the chunks of one
+// row-block are adjacent in memory), parks them in a wave-private LDS area at 16 c, and every lane reads its
+// row's pieces back.  LDS operations of one wave execute in order, so no barrier is involved.
+template <int TYPE> struct WGeo;
+template <> struct WGeo<RT_GGML_Q4_K> {
+    static constexpr int blk = 144, chunks = 9, loads = 5, tail = 0, reads = 5, stage_bytes = 32 * 144;
+};
+template <> struct WGeo<RT_GGML_Q6_K> {   // 13 whole chunks (208 bytes) + the 2-byte d, parked behind the rows
+    static constexpr int blk = 210, chunks = 13, loads = 7, tail = 1, reads = 8, stage_bytes = 32 * 208 + 32 * 4;
+};
+
+template <int TYPE> struct WTmp { u32x4 c[WGeo<TYPE>::loads]; uint32_t tail; };
+
+// per-lane byte offsets (from the weight row of the wave's first row) of the chunk each load instruction fetches
+template <int TYPE> struct WOff { uint32_t c[WGeo<TYPE>::loads]; uint32_t tail; };
+
+template <int TYPE>
+__device__ __forceinline__ void make_woff(WOff<TYPE> &o, int lane, int rows_left, size_t row_bytes) {
+    using G = WGeo<TYPE>;
+#pragma unroll
+    for (int i = 0; i < G::loads; i++) {
+        const int c = 64 * i + lane, row = c / G::chunks, part = c - row * G::chunks;
+        o.c[i] = (uint32_t)(min(row, rows_left - 1) * row_bytes) + 16u * part;     // rows past the matrix repeat its last row
+    }
+    o.tail = (uint32_t)(min(lane & 31, rows_left - 1) * row_bytes) + 208u;
+}
+
+// global load OP of WGeo::loads + WGeo::tail of the chunks of super-block sb
+template <int TYPE, int OP>
+__device__ __forceinline__ void load_op(WTmp<TYPE> &r, const WOff<TYPE> &o, const uint8_t *base, int lane) {
+    using G = WGeo<TYPE>;
+    // Written as assembly so that the compiler keeps no book on them: with LDS-DMA loads in flight its own
+    // wait before the first use would be "all vector memory operations", i.e. the X tile requested last.
+    // The waits that cover these loads are the vmcnt waits of superblock().
+    if constexpr (OP < G::loads) {
+        if (64 * OP + lane < 32 * G::chunks)
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.c[OP]) : "v"(base + o.c[OP]) : "memory");
+    } else {
+        if (lane < 32) asm volatile("global_load_ushort %0, %1, off" : "=v"(r.tail) : "v"(base + o.tail) : "memory");
+    }
+}
+
+// LDS accesses and their waits are written by hand: with LDS-DMA loads in the same loop the compiler's own
+// wait insertion falls back to "wait for everything" before each use, which exposes the full LDS latency
+// every other step.  LDS operations return in order, so "at most n outstanding" pins which have completed.
+template <int OFF> __device__ __forceinline__ half8v lds_read16(uint32_t addr) {
+    half8v r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+    return r;
+}
+template <int OFF> __device__ __forceinline__ u32x4 lds_read16u(uint32_t addr) {
+    u32x4 r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+    return r;
+}
+template <int OFF> __device__ __forceinline__ uint32_t lds_read4(uint32_t addr) {
+    uint32_t r;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
+    return r;
+}
+template <int OFF> __device__ __forceinline__ void lds_write16(uint32_t addr, u32x4 v) {
+    asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(addr), "v"(v), "n"(OFF) : "memory");
+}
+template <int OFF> __device__ __forceinline__ void lds_write4(uint32_t addr, uint32_t v) {
+    asm volatile("ds_write_b32 %0, %1 offset:%2" : : "v"(addr), "v"(v), "n"(OFF) : "memory");
+}
+template <int N> __device__ __forceinline__ void wait_lgkmcnt_c() {
+    static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit counter");
+    __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
+}
+// s_waitcnt that only constrains the vector-memory counter (gfx9 encoding: vmcnt in bits 3:0 and 15:14;
+// lgkmcnt = 15 and expcnt = 7 mean no constraint).
+template <int N> __device__ __forceinline__ void wait_vmcnt_c() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// compile-time loop: f(std::integral_constant<int, I>) for I = B .. E-1 (indices stay constants, so the
+// register-resident structs below are never addressed dynamically)
+template <int B, int E, class F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
+// park the fetched chunks: lane's chunk of instruction i goes to 16 * (64 i + lane); operation OP of
+// WGeo::loads + WGeo::tail (every lane of the wave issues each of them, partly masked)
+template <int TYPE, int OP>
+__device__ __forceinline__ void park_op(const WTmp<TYPE> &r, uint32_t wpark, int lane) {
+    using G = WGeo<TYPE>;
+    if constexpr (OP < G::loads) {
+        if (64 * OP + lane < 32 * G::chunks) lds_write16<1024 * OP>(wpark, r.c[OP]);
+    } else {
+        if (lane < 32) lds_write4<32 * 208>(wpark - 12u * (uint32_t)lane, r.tail);     // 16 lane - 12 lane = 4 lane
+    }
+}
+template <int TYPE> struct WParkOps { static constexpr int n = WGeo<TYPE>::loads + WGeo<TYPE>::tail; };
+
+// ---- raw weight bytes of one lane (weight row nl, k half h) for one super-block
 template <int TYPE> struct WSb;
 template <> struct WSb<RT_GGML_Q4_K> { u32x4 hdr; u32x4 qs[4]; };                 // d|dmin, 12 scale bytes; 16 bytes per 64-k tile
 template <> struct WSb<RT_GGML_Q6_K> { u32x4 A[2], B[2], H[2], sc; uint32_t d; };  // per 128-k half: ql[l], ql[l+32], qh[l]
-template <int TYPE> struct WLoads;
-template <> struct WLoads<RT_GGML_Q4_K> { static constexpr int n = 5; };
-template <> struct WLoads<RT_GGML_Q6_K> { static constexpr int n = 8; };
 
-__device__ __forceinline__ void load_sb(WSb<RT_GGML_Q4_K> &w, const uint8_t *row, int sb, int h) {
-    const uint8_t *blk = row + (size_t)sb * 144;
-    w.hdr = ldg16a(blk);
-#pragma unroll
-    for (int t = 0; t < 4; t++) w.qs[t] = ldg16a(blk + 16 + 32 * t + 16 * h);
+// Read-back operation OP of WGeo::reads; la.wrow is the LDS address of this lane's row-block in the wave's
+// area, wrow_h the same + 16 h for the half-dependent pieces.  The order is the order of first use: what the
+// constants need (OP 0 / 0..1), then tile 0, then the rest.
+template <int OP> __device__ __forceinline__ void fetch_op(WSb<RT_GGML_Q4_K> &w, uint32_t wrow, uint32_t wrow_h, uint32_t) {
+    if constexpr (OP == 0) w.hdr = lds_read16u<0>(wrow);
+    else w.qs[OP - 1] = lds_read16u<16 + 32 * (OP - 1)>(wrow_h);
 }
-__device__ __forceinline__ void load_sb(WSb<RT_GGML_Q6_K> &w, const uint8_t *row, int sb, int h) {
-    const uint8_t *blk = row + (size_t)sb * 210;
-#pragma unroll
-    for (int hf = 0; hf < 2; hf++) {
-        w.A[hf] = ldg16(blk + 64 * hf + 16 * h);
-        w.B[hf] = ldg16(blk + 64 * hf + 32 + 16 * h);
-        w.H[hf] = ldg16(blk + 128 + 32 * hf + 16 * h);
-    }
-    w.sc = ldg16(blk + 192);
-    w.d = ld2u(blk + 208);
+template <int OP> __device__ __forceinline__ void fetch_op(WSb<RT_GGML_Q6_K> &w, uint32_t wrow, uint32_t wrow_h, uint32_t wtail) {
+    if constexpr (OP == 0) w.d = lds_read4<0>(wtail);
+    else if constexpr (OP == 1) w.sc = lds_read16u<192>(wrow);
+    else if constexpr (OP == 2) w.A[0] = lds_read16u<0>(wrow_h);
+    else if constexpr (OP == 3) w.H[0] = lds_read16u<128>(wrow_h);
+    else if constexpr (OP == 4) w.B[0] = lds_read16u<32>(wrow_h);
+    else if constexpr (OP == 5) w.A[1] = lds_read16u<64>(wrow_h);
+    else if constexpr (OP == 6) w.B[1] = lds_read16u<96>(wrow_h);
+    else w.H[1] = lds_read16u<160>(wrow_h);
 }
 
 __device__ __forceinline__ half2v splat(float f) {
@@ -121,61 +246,91 @@ __device__ __forceinline__ uint32_t and_or(uint32_t v, uint32_t m, uint32_t g) {
     asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(m), "v"(g));
     return r;
 }
+// Keeps the computation of v where it is written: without it the optimizer sinks work whose result is only
+// needed after the loop branch into the next iteration, i.e. out from behind the matrix instructions.
+template <class T> __device__ __forceinline__ void pin(T &v) { asm volatile("" : "+v"(v)); }
+
+// Exponent patterns of the in-place integer -> fp16 conversion, kept in vector registers (operands of
+// v_and_or_b32).  A field of an fp16 mantissa under the exponent 2^E reads as 2^E + field * 2^(E-10):
+//   Q4_K: nibble n at bits 3:0 under 2^6 is 64 + n/16, at bits 7:4 under 2^2 it is 4 + n/16;
+//   Q6_K: 6-bit v at bits 5:0 under 2^4 is 16 + v/64.
+struct ExpPat { uint32_t lo, hi; };
 
 // Per-super-block constants of one lane's weight row: everything of the expansion that does not depend on the
-// MFMA step.  One register holds the pair the two halves of a tile need; the fma picks the half.
+// MFMA step.  One register holds the pair the two halves of a tile need; the fma picks the half.  They are
+// computed in kPrepPieces small pieces so that the work can be placed behind matrix instructions of the
+// previous super-block; the trailing fields are intermediates shared by the pieces.
 template <int TYPE> struct SbK;
-template <> struct SbK<RT_GGML_Q4_K> { half2v a[4], c[4]; };   // tile t: (16*d*sc, -dmin*m) of sub-blocks 2t (low nibbles) and 2t+1
-template <> struct SbK<RT_GGML_Q6_K> { half2v a[4]; };         // tile t: 64*d*sc of the tile's two 16-element runs of this lane
+template <> struct SbK<RT_GGML_Q4_K> {
+    half2v a[4], c[4];   // tile t: (16*d*sc, -dmin*m) of sub-blocks 2t (low nibbles) and 2t+1 (high nibbles)
+    uint32_t sc_lo, sc_hi, m_lo, m_hi;
+    half2v d16, nmin;
+};
+template <> struct SbK<RT_GGML_Q6_K> {
+    half2v a[4];         // tile t: 64*d*sc of the tile's two 16-element runs of this lane
+    half2v d64;
+};
+constexpr int kPrepPieces = 9;
 
-// bytes 0 and 1 of v as two exact fp16 numbers: 0x6400 | b is 1024 + b
-__device__ __forceinline__ half2v byte_pair(uint32_t v) {
-    return as_h2((v & 0xFFu) | ((v & 0xFF00u) << 8) | 0x64006400u) - splat(1024.f);
+// bytes i and i+1 (i = 0 or 2) of v as two exact fp16 numbers: one byte permute builds 0x6400 | b = 1024 + b
+__device__ __forceinline__ half2v byte_pair(uint32_t v, int i) {
+    return as_h2(__builtin_amdgcn_perm(0x64646464u, v, i ? 0x04030402u : 0x04010400u)) - splat(1024.f);
 }
 
-__device__ __forceinline__ void prep(SbK<RT_GGML_Q4_K> &k, const WSb<RT_GGML_Q4_K> &w, int) {
-    const uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w;
-    const uint32_t sc_lo = y & 0x3f3f3f3fu, m_lo = z & 0x3f3f3f3fu;
-    const uint32_t sc_hi = (x & 0x0f0f0f0fu) | ((y >> 2) & 0x30303030u);
-    const uint32_t m_hi = ((x >> 4) & 0x0f0f0f0fu) | ((z >> 2) & 0x30303030u);
-    // fp16 products of an 11-bit and a 6-bit number round once: the same value as the f32 product rounded to fp16
-    const half2v d16 = splat_h(h_bits(w.hdr.x & 0xFFFF)) * splat(16.f);
-    const half2v nmin = -splat_h(h_bits(w.hdr.x >> 16));
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        const uint32_t scw = t < 2 ? sc_lo : sc_hi, mw = t < 2 ? m_lo : m_hi;
-        k.a[t] = byte_pair(scw >> (16 * (t & 1))) * d16;
-        k.c[t] = byte_pair(mw >> (16 * (t & 1))) * nmin;
+__device__ __forceinline__ void prep_piece(SbK<RT_GGML_Q4_K> &k, const WSb<RT_GGML_Q4_K> &w, int, int piece) {
+    if (piece == 0) {
+        const uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w;
+        k.sc_lo = y & 0x3f3f3f3fu;
+        k.m_lo = z & 0x3f3f3f3fu;
+        k.sc_hi = (x & 0x0f0f0f0fu) | ((y >> 2) & 0x30303030u);
+        k.m_hi = ((x >> 4) & 0x0f0f0f0fu) | ((z >> 2) & 0x30303030u);
+        // fp16 products of an 11-bit and a 6-bit number round once: the same value as the f32 product rounded to fp16
+        k.d16 = splat_h(h_bits(w.hdr.x & 0xFFFF)) * splat(16.f);
+        k.nmin = -splat_h(h_bits(w.hdr.x >> 16));
+        pin(k.sc_lo); pin(k.m_lo); pin(k.sc_hi); pin(k.m_hi); pin(k.d16); pin(k.nmin);
+    } else {
+        const int i = piece - 1, t = i >> 1;
+        if (i & 1) {
+            k.c[t] = byte_pair(t < 2 ? k.m_lo : k.m_hi, 2 * (t & 1)) * k.nmin;
+            pin(k.c[t]);
+        } else {
+            k.a[t] = byte_pair(t < 2 ? k.sc_lo : k.sc_hi, 2 * (t & 1)) * k.d16;
+            pin(k.a[t]);
+        }
     }
 }
 
 // Packed pair u (k slots 2u, 2u+1 of this lane's row) of the fp16 A operand for MFMA step s of tile t.
 // A step's operand is four such pairs; they are produced one at a time so that each can be issued behind
-// one matrix instruction.
-__device__ __forceinline__ half2v expand_unit(const WSb<RT_GGML_Q4_K> &w, const SbK<RT_GGML_Q4_K> &k, int t, int s, int u, uint32_t G) {
+// one matrix instruction.  w = (n/16) * (16*d*sc) - dmin*m: the subtraction of the exponent's 2^E is exact, so
+// the only roundings are those of the scale, of the offset and of the final fma.
+__device__ __forceinline__ half2v expand_unit(const WSb<RT_GGML_Q4_K> &w, const SbK<RT_GGML_Q4_K> &k, int t, int s, int u, ExpPat G) {
     const int hi = s >> 1;
     const u32x4 qs = w.qs[t];
     const uint32_t q = (s & 1) ? ((u & 2) ? qs.w : qs.z) : ((u & 2) ? qs.y : qs.x);
-    // low nibbles of bytes (0,2) / (1,3) sit at bits 3:0 / 11:8 (and +16); high nibbles 4 bits further up
-    const int sh = (u & 1) * 8 + hi * 4;    // nibble position to bring to bit 6
-    const uint32_t p = (sh <= 6 ? (q << (6 - sh)) : (q >> (sh - 6)));
+    // pair u & 1 = 0 takes bytes 0 and 2 of the word, pair 1 bytes 1 and 3 (one shift brings them down)
+    const uint32_t src = (u & 1) ? (q >> 8) : q;
     const half2v a = splat_h(k.a[t][hi]), c = splat_h(k.c[t][hi]);
-    return (as_h2(and_or(p, 0x03C003C0u, G)) - splat(1.f)) * a + c;
+    if (hi) return (as_h2(and_or(src, 0x00F000F0u, G.hi)) - splat(4.f)) * a + c;
+    return (as_h2(and_or(src, 0x000F000Fu, G.lo)) - splat(64.f)) * a + c;
 }
 
-__device__ __forceinline__ void prep(SbK<RT_GGML_Q6_K> &k, const WSb<RT_GGML_Q6_K> &w, int h) {
+__device__ __forceinline__ void prep_piece(SbK<RT_GGML_Q6_K> &k, const WSb<RT_GGML_Q6_K> &w, int h, int piece) {
     // tile t = 2*hf + p: half hf of the super-block, runs 2p and 2p+1 of that half; of a run's 32 elements this
     // lane holds 16 with scale index 2*run + h among the half's 8 scales, i.e. bytes h and h+2 of word 2*hf + p
-    const half2v d64 = splat_h(h_bits(w.d)) * splat(64.f);
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        const uint32_t v = w.sc[t] >> (8 * h);
+    if (piece == 0) {
+        k.d64 = splat_h(h_bits(w.d)) * splat(64.f);
+        pin(k.d64);
+    } else if (piece <= 4) {
+        const int t = piece - 1;
         // int8 b -> fp16: 0x6400 | (b ^ 0x80) is 1024 + b + 128
-        k.a[t] = (as_h2((((v & 0xFFu) | (v & 0x00FF0000u)) ^ 0x00800080u) | 0x64006400u) - splat(1152.f)) * d64;
+        const uint32_t v = __builtin_amdgcn_perm(0x64646464u, w.sc[t] >> (8 * h), 0x04020400u) ^ 0x00800080u;
+        k.a[t] = (as_h2(v) - splat(1152.f)) * k.d64;
+        pin(k.a[t]);
     }
 }
 
-__device__ __forceinline__ half2v expand_unit(const WSb<RT_GGML_Q6_K> &w, const SbK<RT_GGML_Q6_K> &k, int t, int s, int u, uint32_t G) {
+__device__ __forceinline__ half2v expand_unit(const WSb<RT_GGML_Q6_K> &w, const SbK<RT_GGML_Q6_K> &k, int t, int s, int u, ExpPat G) {
     const int hf = t >> 1, p = t & 1, j = s >> 1, tt = s & 1;
     const u32x4 L = j ? w.B[hf] : w.A[hf];    // run parity = j: even runs read ql[l], odd runs ql[l + 32]
     const u32x4 H = w.H[hf];
@@ -186,87 +341,118 @@ __device__ __forceinline__ half2v expand_unit(const WSb<RT_GGML_Q6_K> &w, const 
     const int shh = 2 * (2 * p + j);
     const uint32_t hb = shh <= 4 ? (hq << (4 - shh)) : (hq >> (shh - 4));
     const uint32_t v = (hb & 0x30303030u) | lo;
-    // fp16 value 1 + v/64 is the bit pattern 0x3C00 | v << 4;  (1 + v/64) - 1.5 = (v - 32)/64 exactly,
-    // so w = 64*dsc * ((1 + v/64) - 1.5) carries only the rounding of the scale and of the product
-    const uint32_t pp = (u & 1) ? (v >> 4) : (v << 4);
-    return (as_h2(and_or(pp, 0x03F003F0u, G)) - splat(1.5f)) * splat_h(k.a[t][j]);
+    // 16 + v/64 minus 16.5 is (v - 32)/64 exactly, so w = 64*d*sc * (v - 32)/64 carries only the rounding of the
+    // scale and of the product
+    const uint32_t src = (u & 1) ? (v >> 8) : v;
+    return (as_h2(and_or(src, 0x003F003Fu, G.lo)) - splat(16.5f)) * splat_h(k.a[t][j]);
 }
 
-// s_waitcnt that only constrains the vector-memory counter (gfx9 encoding: vmcnt in bits 3:0 and 15:14;
-// lgkmcnt = 15 and expcnt = 7 mean no constraint).
-template <int N> __device__ __forceinline__ void wait_vmcnt_c() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+template <int TYPE>
+__device__ __forceinline__ half8v expand_step(const WSb<TYPE> &w, const SbK<TYPE> &k, int t, int s, ExpPat G) {
+    half2v r0 = expand_unit(w, k, t, s, 0, G), r1 = expand_unit(w, k, t, s, 1, G), r2 = expand_unit(w, k, t, s, 2, G),
+           r3 = expand_unit(w, k, t, s, 3, G);
+    return half8v{ r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1] };
 }
 
-// One super-block (256 k = 4 tiles x 4 MFMA steps) of a wave's 32 rows x 32*MF tokens.
+// LDS addresses a lane works with
+struct LaneLds {
+    uint32_t b[4];       // B fragment of step s (stage and fragment go into the instruction's offset field)
+    uint32_t wpark;      // where this lane parks chunk 0 (wave area + 16 lane)
+    uint32_t wrow, wrow_h, wtail;   // its row-block in the wave area, the same + 16 h, its Q6_K d
+};
+
+// One super-block (256 k = 4 tiles x 4 MFMA steps) of a wave's 32 rows x 32*MF tokens, as one software
+// pipeline: every step issues, in this pinned order, the LDS reads of the next step's B fragments, then MF
+// times { matrix instruction; one slice of the next step's A expansion; one slice of other work }.
+// "Next step" crosses tile and super-block borders, so the matrix pipe never waits for an operand:
+//   - the last step of the super-block expands from the next super-block's bytes (wn) with its constants (kn);
+//   - those bytes were requested from global memory at the top of this super-block (tmp), are parked in LDS
+//     and read back by their lanes in the last step of tile 2, and the constants are prepared, a piece per
+//     slot, during tile 3;
+//   - the barrier that publishes X tile t+1 sits in the middle of tile t (before step 2), so the LDS reads
+//     of its first fragments are covered by steps 2 and 3.
 //
 // X tiles (BM rows x 64 k, fp16) go from global memory straight into a ring of 4 LDS stages with 16-byte
-// LDS-DMA loads, issued 3 tiles ahead; since a split starts on a super-block boundary, tile t of every
-// super-block lives in stage t.  One barrier per tile.  LDS stage: row m holds 8 chunks of 16 bytes, chunk c
-// at position c ^ ((m >> 1) & 7), so that the 16 lanes that read the same chunk index of 16 consecutive
-// rows fall on distinct banks.
+// LDS-DMA loads; since a split starts on a super-block boundary, tile t of every super-block lives in stage
+// t.  The load of tile kt+3 is issued right after the barrier in tile kt: by then every wave has left tile
+// kt-1, whose stage it overwrites.  LDS stage: row m holds 8 chunks of 16 bytes, chunk c at position
+// c ^ ((m >> 1) & 7), so that the 16 lanes that read the same chunk index of 16 consecutive rows fall on
+// distinct banks.
 //
 // Vector-memory operations complete in order, so "at most n outstanding" pins which have landed.  Issue order
-// per super-block: weights of the next super-block (WL loads), then one X tile (XI loads) after each barrier.
-// Before tile t the operations younger than its own X tile are two more X tiles and, for t < 3, the weight
-// prefetch.  LAST: no prefetch, and only tile 0 still has an X tile to request.
-template <int TYPE, int MF, int XI, bool LAST, class IssueX>
-__device__ __forceinline__ void superblock(float16v (&acc)[MF], const WSb<TYPE> &w, const _Float16 *xs, int stage_halves,
-                                           const int (&brow)[MF], const int (&bsw)[MF], int h, uint32_t G, int kt, IssueX issue_x) {
-    constexpr int WL = WLoads<TYPE>::n;
-    constexpr int UPM = (4 + MF - 1) / MF;    // expansion pairs issued behind each matrix instruction
-    SbK<TYPE> k;
-    prep(k, w, h);
-    half8v a;
-    {
-        half2v r0 = expand_unit(w, k, 0, 0, 0, G), r1 = expand_unit(w, k, 0, 0, 1, G), r2 = expand_unit(w, k, 0, 0, 2, G),
-               r3 = expand_unit(w, k, 0, 0, 3, G);
-        a = half8v{ r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1] };
-    }
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        if (!LAST) {
-            if (t < 3) wait_vmcnt_c<2 * XI + WL>(); else wait_vmcnt_c<2 * XI>();
-        } else {
-            if (t < 2) wait_vmcnt_c<2 * XI>(); else if (t == 2) wait_vmcnt_c<XI>(); else wait_vmcnt_c<0>();
-        }
-        __builtin_amdgcn_s_barrier();
-        if (!LAST || t == 0) issue_x(kt + t + 3, (t + 3) & 3);
-        const _Float16 *stage = xs + (size_t)t * stage_halves;
-        half8v b[MF];
-#pragma unroll
-        for (int i = 0; i < MF; i++) b[i] = *reinterpret_cast<const half8v *>(stage + (size_t)brow[i] * kBK + 8 * (h ^ bsw[i]));
-#pragma unroll
-        for (int s = 0; s < 4; s++) {
-            // Operands of the next step are fetched (LDS) at the top of this step and expanded (VALU) one packed
-            // pair behind each matrix instruction of this step; the order below is pinned for the scheduler.
-            const bool more_b = s < 3, more_a = s < 3 || t < 3;
-            const int tn = s < 3 ? t : t + 1, sn = (s + 1) & 3;
-            half8v bn[MF];
-            half2v an[4];
-            if (more_b) {
-#pragma unroll
-                for (int i = 0; i < MF; i++)
-                    bn[i] = *reinterpret_cast<const half8v *>(stage + (size_t)brow[i] * kBK + 8 * ((2 * (s + 1) + h) ^ bsw[i]));
+// per super-block: weights of the next super-block (WL loads) at the top, one X tile (XI loads) after each
+// barrier.  At the barrier of tile t the operations younger than X tile kt+1 are X tile kt+2 and, for
+// t < 2, the weight prefetch.  Past the end of the k range the same loads are issued for the last tile /
+// super-block again (the data is not used), which keeps the counts -- and the code -- uniform.
+// Slices of work that ride along with the steps of a super-block (t = tile, s = step), all compile-time:
+//   global loads of the next super-block's chunks: tile 0, steps 0 and 1 (before that tile's barrier)
+//   parking them in LDS:                            tile 2, steps 2 and 3 (after the wait that proves they landed)
+//   reading them back per lane:                     from tile 2 step 3 on, two per step, in order of first use
+template <int TYPE> struct Ride {
+    using G = WGeo<TYPE>;
+    static constexpr int n_load = G::loads + G::tail, n_park = n_load, n_fetch = G::reads;
+    static constexpr int half_load = (n_load + 1) / 2, half_park = (n_park + 1) / 2;
+    static constexpr int load_lo(int t, int s) { return t == 0 && s == 0 ? 0 : (t == 0 && s == 1 ? half_load : n_load); }
+    static constexpr int load_hi(int t, int s) { return t == 0 && s == 0 ? half_load : n_load; }
+    static constexpr int park_lo(int t, int s) { return t == 2 && s == 2 ? 0 : (t == 2 && s == 3 ? half_park : n_park); }
+    static constexpr int park_hi(int t, int s) { return t == 2 && s == 2 ? half_park : n_park; }
+    // first read-back slot is (2,3); slot index = 4*(t-2) + s - 3
+    static constexpr int fetch_lo(int t, int s) { int k = 4 * (t - 2) + s - 3; return k < 0 ? n_fetch : (2 * k < n_fetch ? 2 * k : n_fetch); }
+    static constexpr int fetch_hi(int t, int s) { int k = 4 * (t - 2) + s - 3; return k < 0 ? n_fetch : (2 * k + 2 < n_fetch ? 2 * k + 2 : n_fetch); }
+};
+
+template <int TYPE, int MF, int XI, class IssueX>
+__device__ __forceinline__ void superblock(float16v (&acc)[MF], const WSb<TYPE> &w, const SbK<TYPE> &k, WTmp<TYPE> &tmp,
+                                           const WOff<TYPE> &woff, const uint8_t *wnext, WSb<TYPE> &wn, SbK<TYPE> &kn, half8v &a,
+                                           half8v (&bb)[2][MF], const LaneLds &la, int lane, int h, ExpPat G, int kt, int kt_last,
+                                           IssueX issue_x) {
+    using Geo = WGeo<TYPE>;
+    using R = Ride<TYPE>;
+    constexpr int WL = Geo::loads + Geo::tail;
+    constexpr int UPM = (4 + MF - 1) / MF;                        // expansion pairs issued behind each matrix instruction
+    constexpr int PPS = (kPrepPieces + 2 * MF - 1) / (2 * MF);   // preparation pieces per slot of tile 3, steps 1 and 2
+    constexpr int kStageBytes = 32 * MF * kBK * 2;
+    static_for<0, 4>([&](auto T) {
+        constexpr int t = decltype(T)::value;
+        static_for<0, 4>([&](auto S) {
+            constexpr int s = decltype(S)::value;
+            constexpr int cur = s & 1, nxt = cur ^ 1;             // 16 steps per super-block: the parity carries over
+            if constexpr (s == 2) {
+                wait_vmcnt_c<(t < 2 ? XI + WL : XI)>();
+                __builtin_amdgcn_s_barrier();
             }
+            // the X tile three ahead, one load instruction per step from the barrier on (spreads the burst of
+            // the eight waves over the address path)
+            if constexpr (s >= 2 && s - 2 < XI) issue_x(min(kt + t + 3, kt_last), (t + 3) & 3, s - 2);
+            static_for<R::load_lo(t, s), R::load_hi(t, s)>([&](auto O) { load_op<TYPE, decltype(O)::value>(tmp, woff, wnext, lane); });
+            constexpr int tn = s < 3 ? t : t + 1, sn = (s + 1) & 3;   // tn == 4: tile 0 of the next super-block
+            half2v an[4];
+            static_for<R::park_lo(t, s), R::park_hi(t, s)>([&](auto O) { park_op<TYPE, decltype(O)::value>(tmp, la.wpark, lane); });
+            static_for<0, MF>([&](auto I) {
+                constexpr int i = decltype(I)::value;
+                bb[nxt][i] = lds_read16<(tn & 3) * kStageBytes + i * 32 * kBK * 2>(la.b[sn]);
+            });
+            static_for<R::fetch_lo(t, s), R::fetch_hi(t, s)>([&](auto O) { fetch_op<decltype(O)::value>(wn, la.wrow, la.wrow_h, la.wtail); });
+            wait_lgkmcnt_c<MF + R::fetch_hi(t, s) - R::fetch_lo(t, s)>();
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int j = 0; j < MF; j++) {
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b[j], acc[j], 0, 0, 0);
-                if (more_a) {
-#pragma unroll
-                    for (int q = j * UPM; q < (j + 1) * UPM && q < 4; q++) an[q] = expand_unit(w, k, tn, sn, q, G);
+            static_for<0, MF>([&](auto J) {
+                constexpr int j = decltype(J)::value;
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bb[cur][j], acc[j], 0, 0, 0);
+                static_for<j * UPM, (j + 1) * UPM < 4 ? (j + 1) * UPM : 4>([&](auto Q) {
+                    constexpr int q = decltype(Q)::value;
+                    if constexpr (tn < 4) an[q] = expand_unit(w, k, tn, sn, q, G);
+                    else an[q] = expand_unit(wn, kn, 0, 0, q, G);
+                    pin(an[q]);
+                });
+                if constexpr (t == 3 && (s == 1 || s == 2)) {
+                    constexpr int p0 = ((s - 1) * MF + j) * PPS, p1 = p0 + PPS < kPrepPieces ? p0 + PPS : kPrepPieces;
+                    static_for<p0, p1>([&](auto P) { prep_piece(kn, wn, h, decltype(P)::value); });
                 }
                 __builtin_amdgcn_sched_barrier(0);
-            }
-            if (more_a) a = half8v{ an[0][0], an[0][1], an[1][0], an[1][1], an[2][0], an[2][1], an[3][0], an[3][1] };
-            if (more_b) {
-#pragma unroll
-                for (int i = 0; i < MF; i++) b[i] = bn[i];
-            }
-        }
-    }
+            });
+            a = half8v{ an[0][0], an[0][1], an[1][0], an[1][1], an[2][0], an[2][1], an[3][0], an[3][1] };
+        });
+    });
 }
 
 // Grid: 1-D and XCD-aware.  Tiles are ordered by (m-tile, k-split) "slab" first, n-tile second; workgroup b
@@ -274,15 +460,17 @@ __device__ __forceinline__ void superblock(float16v (&acc)[MF], const WSb<TYPE> 
 // workgroups that share an L2 share an X slab and the slab is read from HBM once.
 // Y_out: Y itself (ksplit == 1; res, when given, is added) or the first of ksplit partial planes of
 // plane_stride floats each.
+// LDS: [4 stages][BM][64] fp16 of X, then NW wave-private areas of WGeo::stage_bytes.
 template <int TYPE, int NW, int MF>
 __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t row_bytes, int N, int K, const _Float16 *Xp,
                                                         const float *inv_scale, int M, float *Y_out, size_t plane_stride,
                                                         const float *res, int sb_per_split, int ksplit, int tiles_n,
                                                         int n_tiles_total, int per_xcd) {
+    using Geo = WGeo<TYPE>;
     constexpr int BM = 32 * MF, BN = 32 * NW, XI = BM / 8 / NW;
     static_assert(XI >= 1 && XI * 8 * NW == BM, "every wave issues whole 8-row LDS-DMA loads");
     constexpr int kStageHalves = BM * kBK;   // halves per stage (no padding: swizzled)
-    RT_DYN_LDS(_Float16, xs);                // [4][BM][64]
+    RT_DYN_LDS(_Float16, xs);
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, nl = lane & 31, h = lane >> 5;
     // tile of this workgroup
     const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
@@ -293,7 +481,11 @@ __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t
     const int sb0 = kz * sb_per_split, sb1 = min(K / 256, sb0 + sb_per_split);
     if (sb0 >= sb1) return;      // the launcher sizes the splits so that none is empty
 
-    const uint8_t *rp = W + (size_t)min(n0 + wave * 32 + nl, N - 1) * row_bytes;
+    // weights: the wave's first row (clamped into the matrix) and the per-lane chunk offsets from it
+    const int wrow0 = min(n0 + wave * 32, N - 1);
+    const uint8_t *wbase = W + (size_t)wrow0 * row_bytes;
+    WOff<TYPE> woff;
+    make_woff(woff, lane, N - wrow0, row_bytes);
 
     // LDS-DMA: instruction i of this wave fills LDS rows (wave*XI + i)*8 .. +8 of a stage; lane L lands at
     // row + L/8, position L%8, which must hold chunk (L%8) ^ ((row >> 1) & 7) of that X row.
@@ -304,13 +496,10 @@ __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t
         int c = (lane & 7) ^ ((row >> 1) & 7);
         xsrc[i] = Xp + (size_t)min(m0 + row, M - 1) * K + 8 * c;
     }
-    auto issue_x = [&](int kt, int st) {
-#pragma unroll
-        for (int i = 0; i < XI; i++) {
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(xsrc[i] + (size_t)kt * kBK),
-                                             (__attribute__((address_space(3))) void *)(xs + (size_t)st * kStageHalves + (size_t)(wave * XI + i) * 8 * kBK),
-                                             16, 0, 0);
-        }
+    auto issue_x = [&](int kt, int st, int i) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(xsrc[i] + (size_t)kt * kBK),
+                                         (__attribute__((address_space(3))) void *)(xs + (size_t)st * kStageHalves + (size_t)(wave * XI + i) * 8 * kBK),
+                                         16, 0, 0);
     };
 
     float16v acc[MF];
@@ -319,29 +508,55 @@ __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
 
-    // B fragment address pieces: lane (token nl of fragment i, half h) reads chunk 2s+h of row i*32 + nl
-    int brow[MF], bsw[MF];
+    // B fragments: lane (token nl of fragment i, half h) reads chunk 2s+h of stage row i*32 + nl
+    LaneLds la;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) _Float16 *)xs;
 #pragma unroll
-    for (int i = 0; i < MF; i++) {
-        brow[i] = i * 32 + nl;
-        bsw[i] = (brow[i] >> 1) & 7;
+    for (int sn = 0; sn < 4; sn++) la.b[sn] = lds0 + (uint32_t)nl * (kBK * 2) + 16u * (uint32_t)((2 * sn + h) ^ ((nl >> 1) & 7));
+    const uint32_t warea = lds0 + 4u * kStageHalves * 2u + (uint32_t)wave * Geo::stage_bytes;
+    la.wpark = warea + 16u * (uint32_t)lane;
+    la.wrow = warea + (uint32_t)nl * (16u * Geo::chunks);
+    la.wrow_h = la.wrow + 16u * (uint32_t)h;
+    la.wtail = warea + 32u * 208u + 4u * (uint32_t)nl;
+    ExpPat G;
+    if (TYPE == RT_GGML_Q4_K) {
+        asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(G.lo));
+        asm volatile("v_mov_b32 %0, 0x44004400" : "=v"(G.hi));
+    } else {
+        asm volatile("v_mov_b32 %0, 0x4c004c00" : "=v"(G.lo));
+        G.hi = 0;
     }
-    // the exponent pattern of the expansion, kept in a vector register (operand of v_and_or_b32)
-    uint32_t G;
-    asm volatile("v_mov_b32 %0, 0x3c003c00" : "=v"(G));
 
-    WSb<TYPE> wc, wn;
-    const int kt0 = 4 * sb0;
-    issue_x(kt0, 0);
-    issue_x(kt0 + 1, 1);
-    issue_x(kt0 + 2, 2);
-    load_sb(wc, rp, sb0, h);
-    for (int sb = sb0; sb < sb1 - 1; sb++) {
-        load_sb(wn, rp, sb + 1, h);
-        superblock<TYPE, MF, XI, false>(acc, wc, xs, kStageHalves, brow, bsw, h, G, 4 * sb, issue_x);
-        wc = wn;
+    // prologue: three X tiles and the first super-block's weights in flight, constants and operands of step 0
+    const int kt0 = 4 * sb0, kt_last = 4 * sb1 - 1;
+    WTmp<TYPE> tmp;
+    WSb<TYPE> wA, wB;
+    SbK<TYPE> kA, kB;
+#pragma unroll
+    for (int d = 0; d < 3; d++)
+#pragma unroll
+        for (int i = 0; i < XI; i++) issue_x(kt0 + d, d, i);
+    static_for<0, Ride<TYPE>::n_load>([&](auto O) { load_op<TYPE, decltype(O)::value>(tmp, woff, wbase + (size_t)sb0 * Geo::blk, lane); });
+    wait_vmcnt_c<0>();
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, Ride<TYPE>::n_park>([&](auto O) { park_op<TYPE, decltype(O)::value>(tmp, la.wpark, lane); });
+    static_for<0, Ride<TYPE>::n_fetch>([&](auto O) { fetch_op<decltype(O)::value>(wA, la.wrow, la.wrow_h, la.wtail); });
+    wait_lgkmcnt_c<0>();
+    __builtin_amdgcn_sched_barrier(0);     // the scheduler does not know that the wait guards wA
+    static_for<0, kPrepPieces>([&](auto P) { prep_piece(kA, wA, h, decltype(P)::value); });
+    half8v a = expand_step(wA, kA, 0, 0, G), bb[2][MF];
+    __builtin_amdgcn_s_barrier();
+    static_for<0, MF>([&](auto I) { bb[0][decltype(I)::value] = lds_read16<decltype(I)::value * 32 * kBK * 2>(la.b[0]); });
+
+    for (int sb = sb0;;) {
+        superblock<TYPE, MF, XI>(acc, wA, kA, tmp, woff, wbase + (size_t)min(sb + 1, sb1 - 1) * Geo::blk, wB, kB, a, bb, la, lane, h, G,
+                                 4 * sb, kt_last, issue_x);
+        if (++sb >= sb1) break;
+        superblock<TYPE, MF, XI>(acc, wB, kB, tmp, woff, wbase + (size_t)min(sb + 1, sb1 - 1) * Geo::blk, wA, kA, a, bb, la, lane, h, G,
+                                 4 * sb, kt_last, issue_x);
+        if (++sb >= sb1) break;
     }
-    superblock<TYPE, MF, XI, true>(acc, wc, xs, kStageHalves, brow, bsw, h, G, 4 * (sb1 - 1), issue_x);
+    wait_vmcnt_c<0>();           // the loads issued past the end of the range still target this workgroup's LDS
 
     // D[i][j]: j (token) = lane % 32; i (weight row) = 8*(r/4) + 4*(lane/32) + r%4
     float *Yp = Y_out + (size_t)kz * plane_stride;
@@ -380,21 +595,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *P, size
     }
 }
 
-struct GemmPlan { int nw, mf, ksplit, sb_per_split; };
+struct GemmPlan { int mf, ksplit, sb_per_split; };
 
-// Shape of the launch: waves per workgroup (tile 32*mf tokens x 32*nw rows) and k splits.
+constexpr int kGemmWaves = 8;     // waves per workgroup: two per SIMD, one workgroup per CU
+
+// Shape of the launch: token fragments per wave (tile 32*mf tokens x 256 rows) and k splits.
 GemmPlan gemm_plan(size_t M, size_t N, size_t K) {
     GemmPlan p;
     p.mf = M > 64 ? 4 : 2;
-    const size_t bm = 32 * (size_t)p.mf, tiles_m = (M + bm - 1) / bm, nsb = K / 256;
-    const size_t t8 = tiles_m * ((N + 255) / 256), t4 = tiles_m * ((N + 127) / 128);
+    const size_t bm = 32 * (size_t)p.mf, tiles = ((M + bm - 1) / bm) * ((N + 32 * kGemmWaves - 1) / (32 * kGemmWaves)), nsb = K / 256;
+    // split k while that fills more of the 256 CUs in whole rounds and leaves every split at least two super-blocks
     p.ksplit = 1;
-    if (t8 >= 224) {
-        p.nw = 8;                 // one 8-wave workgroup per CU already fills the chip
-    } else {
-        p.nw = 4;                 // two 4-wave workgroups per CU: split k until the 512 slots are taken
-        while (t4 * p.ksplit * 2 <= 512 && nsb / (p.ksplit * 2) >= 2 && p.ksplit < kMaxSplit) p.ksplit *= 2;
-    }
+    while (tiles * p.ksplit * 2 <= 256 && nsb / (p.ksplit * 2) >= 2 && p.ksplit < kMaxSplit) p.ksplit *= 2;
     p.sb_per_split = (int)((nsb + p.ksplit - 1) / p.ksplit);
     p.ksplit = (int)((nsb + p.sb_per_split - 1) / p.sb_per_split);     // no empty split
     return p;
@@ -404,8 +616,14 @@ template <int TYPE, int NW, int MF>
 hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const _Float16 *Xp,
                       const float *inv_scale, size_t M, float *Y, const float *res, float *partial) {
     constexpr int BM = 32 * MF, BN = 32 * NW;
-    const size_t lds = (size_t)4 * BM * kBK * sizeof(_Float16);
+    const size_t lds = (size_t)4 * BM * kBK * sizeof(_Float16) + (size_t)NW * WGeo<TYPE>::stage_bytes;
     auto kern = qgemm_kernel<TYPE, NW, MF>;
+    static bool attr_set = false;      // per instantiation
+    if (!attr_set && lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
     const int total = tiles_m * p.ksplit * tiles_n;
     const int per_xcd = (total + 7) / 8;
@@ -423,10 +641,8 @@ hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t
 template <int TYPE>
 hipError_t launch_type(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const _Float16 *Xp,
                        const float *inv_scale, size_t M, float *Y, const float *res, float *partial) {
-    if (p.nw == 8 && p.mf == 4) return launch_cfg<TYPE, 8, 4>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
-    if (p.nw == 4 && p.mf == 4) return launch_cfg<TYPE, 4, 4>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
-    if (p.nw == 8 && p.mf == 2) return launch_cfg<TYPE, 8, 2>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
-    return launch_cfg<TYPE, 4, 2>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
+    if (p.mf == 4) return launch_cfg<TYPE, kGemmWaves, 4>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
+    return launch_cfg<TYPE, kGemmWaves, 2>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
 }
 
 bool mfma_path(int type, size_t N, size_t K, size_t M) {
@@ -436,6 +652,7 @@ bool mfma_path(int type, size_t N, size_t K, size_t M) {
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace
+
 
 // workspace: fp16 X, one f32 per row of X, and the partial planes of a k-split launch
 size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K) {
