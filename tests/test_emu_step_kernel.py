@@ -1,0 +1,27 @@
+"""The persistent decode-step kernel (switched off on the GPU after an unexplained fault) keeps a CPU test:
+its device code, compiled as host C++ and run as fibers under AddressSanitizer (tests/emu/), must run clean
+and pick the tokens the oracle picks.  Takes about a minute and a half."""
+import os
+import shutil
+import subprocess
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parents[1]
+CLANG = "/opt/rocm/llvm/bin/clang++"
+
+
+@pytest.mark.skipif(not (Path(CLANG).exists() and shutil.which("gcc")), reason="needs ROCm's clang++ and gcc")
+def test_step_kernel_as_cpu_fibers_under_asan(tmp_path):
+    obj = tmp_path / "rt_oracle.o"
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-fopenmp", "-c", str(ROOT / "oracle" / "rt_oracle.c"), "-o", str(obj)], check=True)
+    exe = tmp_path / "emu_main"
+    subprocess.run([CLANG, "-std=c++17", "-O1", "-g", "-fsanitize=address", "-I", str(ROOT / "tests" / "emu"),
+                    "-I", str(ROOT / "rustorch_amd" / "csrc"), "-I", str(ROOT / "include"), str(ROOT / "tests" / "emu" / "emu_main.cpp"),
+                    str(ROOT / "rustorch_amd" / "csrc" / "rt_synth.cpp"), str(obj), "-o", str(exe), "-fopenmp"], check=True)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
+    r = subprocess.run([str(exe)], env=env, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "EMU OK" in r.stdout
+    assert "ERROR: AddressSanitizer" not in r.stderr
