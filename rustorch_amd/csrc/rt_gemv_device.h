@@ -192,6 +192,11 @@ __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_0> &x, const uint32_t *l
 
 #define RT_W4(v) { (v).x, (v).y, (v).z, (v).w }
 
+// The float tails of the dot products are written with explicit fused operations and contraction off, so
+// that every instantiation (one or two rows per step, any staging mode) rounds the same way: a row's result
+// does not depend on which code path computed it.
+#pragma clang fp contract(off)
+
 __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_K> &w, const XRegs<RT_GGML_Q4_K> &x, int u) {
     const int g = u & 3;
     uint32_t scw, mw;
@@ -223,7 +228,8 @@ __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_K> &w, const XR
         dl1 = sdot4(hi, (int)lhi[i], dl1);
     }
     float t0 = (float)((dh0 << 7) + dl0), t1 = (float)((dh1 << 7) + dl1);
-    return d * (sc0 * (x.sv.x * t0) + sc1 * (x.sv.y * t1)) - dmin * (m0 * x.sv.z + m1 * x.sv.w);
+    const float pos = __builtin_fmaf(sc0, x.sv.x * t0, sc1 * (x.sv.y * t1)), neg = __builtin_fmaf(m0, x.sv.z, m1 * x.sv.w);
+    return __builtin_fmaf(d, pos, -(dmin * neg));
 }
 
 __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q6_K> &w, const XRegs<RT_GGML_Q6_K> &x, int u) {
@@ -246,10 +252,10 @@ __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q6_K> &w, const XR
     uint32_t s01 = w.sc.x >> s8, s23 = w.sc.y >> s8;
     float sc0 = (float)(int)(int8_t)(s01 & 0xFF), sc1 = (float)(int)(int8_t)((s01 >> 16) & 0xFF);
     float sc2 = (float)(int)(int8_t)(s23 & 0xFF), sc3 = (float)(int)(int8_t)((s23 >> 16) & 0xFF);
-    float a = sc0 * (x.xs.x * (float)((dh[0] << 7) + dl[0]) - 32.f * x.xb.x);
-    a += sc1 * (x.xs.y * (float)((dh[1] << 7) + dl[1]) - 32.f * x.xb.y);
-    a += sc2 * (x.xs.z * (float)((dh[2] << 7) + dl[2]) - 32.f * x.xb.z);
-    a += sc3 * (x.xs.w * (float)((dh[3] << 7) + dl[3]) - 32.f * x.xb.w);
+    float a = sc0 * __builtin_fmaf(x.xs.x, (float)((dh[0] << 7) + dl[0]), -32.f * x.xb.x);
+    a = __builtin_fmaf(sc1, __builtin_fmaf(x.xs.y, (float)((dh[1] << 7) + dl[1]), -32.f * x.xb.y), a);
+    a = __builtin_fmaf(sc2, __builtin_fmaf(x.xs.z, (float)((dh[2] << 7) + dl[2]), -32.f * x.xb.z), a);
+    a = __builtin_fmaf(sc3, __builtin_fmaf(x.xs.w, (float)((dh[3] << 7) + dl[3]), -32.f * x.xb.w), a);
     return h2f(w.d) * a;
 }
 
@@ -263,7 +269,7 @@ __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q8_0> &w, const XR
         dh = sdot4(q[i], (int)xh[i], dh);
         dl = sdot4(q[i], (int)xl[i], dl);
     }
-    return h2f(w.d) * (x.s * ((float)dh * 128.f + (float)dl));
+    return h2f(w.d) * (x.s * __builtin_fmaf((float)dh, 128.f, (float)dl));
 }
 
 __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_0> &w, const XRegs<RT_GGML_Q4_0> &x, int) {
@@ -278,8 +284,9 @@ __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_0> &w, const XR
         dh = sdot4(hi, (int)hhi[i], dh);
         dl = sdot4(hi, (int)lhi[i], dl);
     }
-    return h2f(w.d) * (x.sv.x * (float)((dh << 7) + dl) - 8.f * x.sv.y);
+    return h2f(w.d) * __builtin_fmaf(x.sv.x, (float)((dh << 7) + dl), -8.f * x.sv.y);
 }
+#pragma clang fp contract(fast)
 
 // A wave walks "steps": step s = (row group s / n_iter, unit pass s % n_iter); a row group is R rows (with the
 // SwiGLU epilogue: R/2 gate rows and their up rows).  Row groups are dealt round-robin over all waves that work
@@ -314,7 +321,7 @@ struct Walker {
         const int uc = min(u, U - 1);
         const float live = u < U ? 1.f : 0.f;
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r] += live * dot_unit(w[r], x, uc);
+        for (int r = 0; r < R; r++) acc[r] = __builtin_fmaf(live, dot_unit(w[r], x, uc), acc[r]);
         if (s % n_iter != n_iter - 1) return;
         const int g = group_of(s);
 #pragma unroll
