@@ -184,6 +184,10 @@ __device__ __forceinline__ void unpack8(uint4 v, float *f) {
     }
 }
 
+// One workgroup per head.  The cache rows of the positions already stored do not depend on this step's
+// q, k, v, so their loads are issued first -- the key row of the thread's position and the value chunks of
+// the thread's first kVPre positions -- and the rope/append of the new token, the scores and the softmax run
+// while they are in flight: one memory round trip instead of three dependent ones.
 template <int HD, bool FUSED>
 __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float *k, const float *v, uint16_t *kc,
                                                           uint16_t *vc, const int *pos_dev, int n_pos_arg, int n_heads,
@@ -196,11 +200,28 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
     __shared__ __align__(16) float part[2048];
     constexpr int CH = HD / 8;          // 16-byte chunks per cache row of this head
     constexpr int NG = 256 / CH;        // position groups in the value phase
+    constexpr int kVPre = 16;           // value chunks a thread requests ahead (covers NG * kVPre positions)
     const int h = blockIdx.x, tid = threadIdx.x;
     const size_t row = (size_t)n_heads * HD;
     const int cur = FUSED ? *pos_dev : -1;
     const int n_pos = FUSED ? cur + 1 : n_pos_arg;
     const float scale = 1.0f / sqrtf((float)HD);
+    const int c = tid % CH, g = tid / CH;
+
+    // ---- requests that do not depend on the new token
+    uint4 kreg[CH], vreg[kVPre];
+    const bool k_pre = tid < n_pos && tid != cur;
+    if (k_pre) {
+        const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)tid * row + (size_t)h * HD);
+#pragma unroll
+        for (int i = 0; i < CH; i++) kreg[i] = kr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kVPre; i++) {
+        const int j = g + NG * i;
+        if (j < n_pos && j != cur) vreg[i] = reinterpret_cast<const uint4 *>(vc + (size_t)j * row + (size_t)h * HD)[c];
+    }
+
     if (FUSED) {
         if (tid < HD / 2) {
             int i = tid;
@@ -239,11 +260,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
         } else {
             const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)j * row + (size_t)h * HD);
 #pragma unroll
-            for (int c = 0; c < CH; c++) {
+            for (int cc = 0; cc < CH; cc++) {
                 float f[8];
-                unpack8(kr[c], f);
+                unpack8(j == tid ? kreg[cc] : kr[cc], f);
 #pragma unroll
-                for (int e = 0; e < 8; e++) s += qs[8 * c + e] * f[e];
+                for (int e = 0; e < 8; e++) s += qs[8 * cc + e] * f[e];
             }
         }
         s *= scale;
@@ -261,11 +282,26 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
     for (int j = tid; j < n_pos; j += 256) sc[j] = sc[j] / sum;
     __syncthreads();
     // ---- values
-    const int c = tid % CH, g = tid / CH;
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) acc[e] = 0.f;
-    for (int j = g; j < n_pos; j += NG) {
+#pragma unroll
+    for (int i = 0; i < kVPre; i++) {
+        const int j = g + NG * i;
+        if (j < n_pos) {
+            float f[8];
+            if (j == cur) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) f[e] = vcur[8 * c + e];
+            } else {
+                unpack8(vreg[i], f);
+            }
+            float p = sc[j];
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] += p * f[e];
+        }
+    }
+    for (int j = g + NG * kVPre; j < n_pos; j += NG) {
         float f[8];
         if (j == cur) {
 #pragma unroll
