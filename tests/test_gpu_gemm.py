@@ -86,3 +86,20 @@ def test_other_formats_and_small_m_use_the_row_form(ex, orc):
             y64, wn = orc.qgemv_f64(t, raw, 96, cols, X)
             xn = np.linalg.norm(X.astype(np.float64), axis=1)[:, None]
             assert (np.abs(ex.qgemm(w, X) - y64) / (wn[None, :] * xn)).max() <= HELD * np.sqrt(4096 / cols)
+
+
+@pytest.mark.parametrize("t", [12, 14])
+@pytest.mark.parametrize("rows,cols,M", [(36, 256, 40), (4, 512, 130), (260, 768, 65), (512, 2816, 96)])
+def test_single_superblock_odd_counts_and_tiny_matrices(ex, orc, t, rows, cols, M):
+    """One super-block per row (the pipeline's first and last body coincide), an odd number of super-blocks,
+    fewer weight rows than one wave holds, M one past a tile."""
+    from rustorch_amd import synth
+    print("gemm edge type", t, rows, cols, "M", M, flush=True)
+    raw = synth.blocks(t, 34, rows + cols, rows, cols)
+    w = ex.upload_qweight(t, rows, cols, raw)
+    X = synth.normal(34, M, M * cols).reshape(M, cols)
+    Y = ex.qgemm(w, X)
+    y64, wn = orc.qgemv_f64(t, raw, rows, cols, X)
+    xn = np.linalg.norm(X.astype(np.float64), axis=1)[:, None]
+    ratio = np.abs(Y - y64) / (wn[None, :] * xn)
+    assert np.isfinite(Y).all() and ratio.max() <= HELD * np.sqrt(4096 / cols), ratio.max()
