@@ -129,6 +129,13 @@ hipError_t launch_rope_kv(hipStream_t s, float *q, const float *k, const float *
 hipError_t launch_attn_decode(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
                               const int *pos_dev, int n_pos, int n_heads, int head_dim, const float *inv_freq_dev,
                               float *out, uint8_t *xq, bool fused);
+hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache,
+                                int pos0, size_t n_tok, int n_heads, int head_dim, const float *inv_freq_dev);
+hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
+                             const int *pos_dev, int n_pos, size_t n_queries, int n_heads, int head_dim,
+                             const float *inv_freq_dev, float *out, uint8_t *xq, bool fused);
+hipError_t launch_embed_rows(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,
+                             const int *tokens_dev, size_t n_tok, int vocab, float *out);
 hipError_t launch_add(hipStream_t s, float *x, const float *y, size_t n);
 hipError_t launch_argmax(hipStream_t s, const float *v, size_t n, int *out_dev);
 hipError_t launch_embed_row(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,

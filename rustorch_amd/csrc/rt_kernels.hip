@@ -24,11 +24,11 @@ __global__ void dequant_kernel(int type, const uint8_t *w, size_t row_bytes, siz
 
 __global__ void embed_row_kernel(int type, const uint8_t *w, size_t row_bytes, size_t n_cols, const int *token_dev,
                                  int vocab, float *out) {
-    int tok = *token_dev;
+    int tok = token_dev[blockIdx.y];          // grid.y tokens, one output row each
     if (tok < 0) tok = 0;
     if (tok >= vocab) tok = vocab - 1;
     size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (c < n_cols) out[c] = deq_elem(type, w + (size_t)tok * row_bytes, c);
+    if (c < n_cols) out[(size_t)blockIdx.y * n_cols + c] = deq_elem(type, w + (size_t)tok * row_bytes, c);
 }
 #pragma clang fp contract(fast)
 
@@ -166,6 +166,28 @@ __global__ void rope_kv_kernel(float *q, const float *k, const float *v, uint16_
     reinterpret_cast<uint32_t *>(vcache + (size_t)p * row)[t] = vp;
 }
 
+// Prefill form: blockIdx.y = token m of the batch at position pos0 + m; q [M][row] is rotated in place,
+// rotated k and v go to the fp16 cache rows pos0 + m.
+__global__ void rope_kv_batch_kernel(float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache,
+                                     int pos0, int n_heads, int head_dim, const float *inv_freq) {
+    int half = head_dim / 2;
+    int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_heads * half) return;
+    int i = t % half;
+    const size_t row = (size_t)n_heads * head_dim, m = blockIdx.y;
+    const int p = pos0 + (int)m;
+    float s, c;
+    sincosf((float)p * inv_freq[i], &s, &c);
+    float2 *qr = reinterpret_cast<float2 *>(q + m * row);
+    float2 qv = qr[t];
+    qr[t] = make_float2(qv.x * c - qv.y * s, qv.x * s + qv.y * c);
+    float2 kv = reinterpret_cast<const float2 *>(k + m * row)[t];
+    float k0 = kv.x * c - kv.y * s, k1 = kv.x * s + kv.y * c;
+    float2 vv = reinterpret_cast<const float2 *>(v + m * row)[t];
+    reinterpret_cast<uint32_t *>(kcache + (size_t)p * row)[t] = (uint32_t)f2h_rne(k0) | ((uint32_t)f2h_rne(k1) << 16);
+    reinterpret_cast<uint32_t *>(vcache + (size_t)p * row)[t] = (uint32_t)f2h_rne(vv.x) | ((uint32_t)f2h_rne(vv.y) << 16);
+}
+
 // -------------------------------------------------------- decode attention
 // One block (256 threads) per head; cache layout [pos][head][dim], fp16.
 //   scores_j = (q . k_j) / sqrt(dim);  p = softmax(scores) with max subtraction;  out = sum_j p_j v_j
@@ -204,7 +226,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
     const int h = blockIdx.x, tid = threadIdx.x;
     const size_t row = (size_t)n_heads * HD;
     const int cur = FUSED ? *pos_dev : -1;
-    const int n_pos = FUSED ? cur + 1 : n_pos_arg;
+    // not fused: blockIdx.y = query m of a causal batch; query m sees n_pos_arg + m positions
+    const int n_pos = FUSED ? cur + 1 : n_pos_arg + (int)blockIdx.y;
+    if (!FUSED) {
+        q += (size_t)blockIdx.y * row;
+        if (out) out += (size_t)blockIdx.y * row;
+    }
     const float scale = 1.0f / sqrtf((float)HD);
     const int c = tid % CH, g = tid / CH;
 
@@ -469,11 +496,27 @@ hipError_t launch_rope_kv(hipStream_t s, float *q, const float *k, const float *
     return hipGetLastError();
 }
 
+hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache,
+                                int pos0, size_t n_tok, int n_heads, int head_dim, const float *inv_freq_dev) {
+    int pairs = n_heads * head_dim / 2;
+    rope_kv_batch_kernel<<<dim3((unsigned)((pairs + 255) / 256), (unsigned)n_tok), 256, 0, s>>>(q, k, v, kcache, vcache, pos0, n_heads,
+                                                                                                head_dim, inv_freq_dev);
+    return hipGetLastError();
+}
+
 hipError_t launch_attn_decode(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
                               const int *pos_dev, int n_pos, int n_heads, int head_dim, const float *inv_freq_dev,
                               float *out, uint8_t *xq, bool fused) {
-    size_t lds = (size_t)n_pos * sizeof(float);  // fused: n_pos is the upper bound (max_pos)
-    dim3 grid((unsigned)n_heads);
+    return launch_attn_batch(s, q, k, v, kc, vc, pos_dev, n_pos, 1, n_heads, head_dim, inv_freq_dev, out, xq, fused);
+}
+
+// n_queries > 1 (not fused, xq == NULL): query m of q [n_queries][row] attends over the first n_pos + m cache rows
+hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
+                             const int *pos_dev, int n_pos, size_t n_queries, int n_heads, int head_dim,
+                             const float *inv_freq_dev, float *out, uint8_t *xq, bool fused) {
+    if (n_queries > 1 && (fused || xq)) return hipErrorInvalidValue;
+    size_t lds = ((size_t)n_pos + n_queries - 1) * sizeof(float);  // fused: n_pos is the upper bound (max_pos)
+    dim3 grid((unsigned)n_heads, (unsigned)n_queries);
     if (head_dim == 128 && fused)
         attn_decode_kernel<128, true><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, inv_freq_dev, out, xq);
     else if (head_dim == 128)
@@ -500,8 +543,13 @@ hipError_t launch_argmax(hipStream_t s, const float *v, size_t n, int *out_dev) 
 
 hipError_t launch_embed_row(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,
                             const int *token_dev, int vocab, float *out) {
-    embed_row_kernel<<<dim3((unsigned)((n_cols + 255) / 256)), 256, 0, s>>>(type, w, row_bytes, n_cols, token_dev,
-                                                                            vocab, out);
+    return launch_embed_rows(s, type, w, row_bytes, n_cols, token_dev, 1, vocab, out);
+}
+
+hipError_t launch_embed_rows(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,
+                             const int *tokens_dev, size_t n_tok, int vocab, float *out) {
+    embed_row_kernel<<<dim3((unsigned)((n_cols + 255) / 256), (unsigned)n_tok), 256, 0, s>>>(type, w, row_bytes, n_cols, tokens_dev,
+                                                                                             vocab, out);
     return hipGetLastError();
 }
 

@@ -12,6 +12,7 @@
 #include "rt_internal.h"
 
 #include <cmath>
+#include <algorithm>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -49,6 +50,11 @@ struct rt_hip_llama {
     unsigned *bar = nullptr;
     int mega_grid = 0, wg_q = 0, wg_k = 0;
     size_t mega_lds = 0;
+    // batched prefill (dense contraction path): activations of up to pf_cap tokens
+    size_t pf_cap = 0;
+    float *pf_x = nullptr, *pf_x2 = nullptr, *pf_n = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_a = nullptr;
+    float *pf_g = nullptr, *pf_u = nullptr;
+    int *pf_tok = nullptr;
     std::vector<void *> allocs;
 };
 
@@ -135,6 +141,75 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
 }
 
 bool gemv_type_ok(int t) { return t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_K || t == RT_GGML_Q6_K; }
+
+constexpr size_t kPrefillChunk = 512;     // tokens per pass of the batched prefill
+
+// The dense-contraction path serves a layer when all seven matrices are Q4_K / Q6_K with whole super-blocks.
+bool prefill_batchable(const rt_hip_llama *m) {
+    auto ok = [](const rt_hip_llama::T &t) {
+        return (t.type == RT_GGML_Q4_K || t.type == RT_GGML_Q6_K) && t.n_cols % 256 == 0 && t.n_rows % 4 == 0;
+    };
+    for (int l = 0; l < m->cfg.n_layers; l++)
+        if (!(ok(m->wq[l]) && ok(m->wk[l]) && ok(m->wv[l]) && ok(m->wo[l]) && ok(m->wgate[l]) && ok(m->wup[l]) && ok(m->wdown[l]))) return false;
+    return m->head_dim == 64 || m->head_dim == 128;
+}
+
+int ensure_prefill_buffers(rt_hip_ctx *ctx, rt_hip_llama *m, size_t n_tok) {
+    if (m->pf_cap >= n_tok) return RT_HIP_OK;
+    const size_t H = (size_t)m->cfg.hidden, F = (size_t)m->cfg.ffn, cap = n_tok;
+    int rc;
+    float **hs[] = { &m->pf_x, &m->pf_x2, &m->pf_n, &m->pf_q, &m->pf_k, &m->pf_v, &m->pf_a };
+    for (float **p : hs)
+        if ((rc = dev_alloc(ctx, m, (void **)p, cap * H * sizeof(float)))) return rc;     // earlier, smaller ones are freed with the model
+    if ((rc = dev_alloc(ctx, m, (void **)&m->pf_g, cap * F * sizeof(float)))) return rc;
+    if ((rc = dev_alloc(ctx, m, (void **)&m->pf_u, cap * F * sizeof(float)))) return rc;
+    if ((rc = dev_alloc(ctx, m, (void **)&m->pf_tok, cap * sizeof(int)))) return rc;
+    m->pf_cap = cap;
+    return RT_HIP_OK;
+}
+
+int gemm(rt_hip_ctx *ctx, const rt_hip_llama::T &t, const float *X, size_t M, float *Y, const float *res) {
+    RT_TRY_HIP(ctx, rt::launch_qgemm(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, X, M, Y, res, ctx->scratch, ctx->scratch_bytes));
+    return RT_HIP_OK;
+}
+
+// M tokens (already in pf_tok) at positions pos0 .. pos0+M-1 through all layers with the dense contraction:
+// per layer rmsnorm rows -> q,k,v GEMMs -> rope + cache append -> causal attention (query m over pos0+m+1 rows)
+// -> o-projection + residual -> rmsnorm -> gate, up GEMMs -> SwiGLU -> down-projection + residual.
+// The hidden state of the last token ends in m->x.  Enqueue only.
+int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) {
+    hipStream_t s = ctx->stream;
+    const rt_hip_llama_config &c = m->cfg;
+    const size_t H = (size_t)c.hidden, F = (size_t)c.ffn;
+    size_t need = 0;
+    for (const auto *t : { &m->wq[0], &m->wo[0], &m->wgate[0], &m->wdown[0], &m->wv[0] })
+        need = std::max(need, rt::qgemm_scratch_bytes(t->type, M, t->n_rows, t->n_cols));
+    int rc = ensure_scratch(ctx, need);
+    if (rc) return rc;
+    float *x = m->pf_x, *x2 = m->pf_x2;
+    RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, m->pf_tok, M, c.vocab, x));
+    for (int l = 0; l < c.n_layers; l++) {
+        uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * H;
+        uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * H;
+        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->attn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
+        if ((rc = gemm(ctx, m->wq[l], m->pf_n, M, m->pf_q, nullptr))) return rc;
+        if ((rc = gemm(ctx, m->wk[l], m->pf_n, M, m->pf_k, nullptr))) return rc;
+        if ((rc = gemm(ctx, m->wv[l], m->pf_n, M, m->pf_v, nullptr))) return rc;
+        RT_TRY_HIP(ctx, rt::launch_rope_kv_batch(s, m->pf_q, m->pf_k, m->pf_v, kc, vc, pos0, M, c.n_heads, m->head_dim, m->inv_freq));
+        RT_TRY_HIP(ctx, rt::launch_attn_batch(s, m->pf_q, nullptr, nullptr, kc, vc, nullptr, pos0 + 1, M, c.n_heads, m->head_dim,
+                                              m->inv_freq, m->pf_a, nullptr, false));
+        if ((rc = gemm(ctx, m->wo[l], m->pf_a, M, x2, x))) return rc;
+        std::swap(x, x2);
+        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->ffn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
+        if ((rc = gemm(ctx, m->wgate[l], m->pf_n, M, m->pf_g, nullptr))) return rc;
+        if ((rc = gemm(ctx, m->wup[l], m->pf_n, M, m->pf_u, nullptr))) return rc;
+        RT_TRY_HIP(ctx, rt::launch_swiglu(s, m->pf_g, m->pf_u, m->pf_g, nullptr, M * F));
+        if ((rc = gemm(ctx, m->wdown[l], m->pf_g, M, x2, x))) return rc;
+        std::swap(x, x2);
+    }
+    RT_TRY_HIP(ctx, hipMemcpyAsync(m->x, x + (M - 1) * H, H * sizeof(float), hipMemcpyDeviceToDevice, s));
+    return RT_HIP_OK;
+}
 
 }  // namespace
 
@@ -380,6 +455,38 @@ int rt_hip_llama_prefill(rt_hip_ctx *ctx, rt_hip_llama *m, const int *tokens, in
     int rc = check_complete(ctx, m);
     if (rc) return rc;
     Guard g(ctx);
+    if (n_tok >= 16 && prefill_batchable(m)) {
+        // dense-contraction path, kPrefillChunk tokens per pass; the logits of the last token come from the head GEMV
+        rc = ensure_prefill_buffers(ctx, m, std::min((size_t)n_tok, kPrefillChunk));
+        if (rc) return rc;
+        for (size_t t0 = 0; t0 < (size_t)n_tok; t0 += kPrefillChunk) {
+            const size_t M = std::min(kPrefillChunk, (size_t)n_tok - t0);
+            RT_TRY_HIP(ctx, hipMemcpyAsync(m->pf_tok, tokens + t0, M * sizeof(int), hipMemcpyHostToDevice, ctx->stream));
+            if (M >= 16) {
+                rc = enqueue_prefill_batch(ctx, m, M, pos0 + (int)t0);
+                if (rc) return rc;
+            } else {
+                // a short tail goes token by token (the row form of the contraction starts at 16 rows)
+                for (size_t i = 0; i < M; i++) {
+                    RT_TRY_HIP(ctx, rt::launch_set_state(ctx->stream, m->state, pos0 + (int)(t0 + i), tokens[t0 + i], 0));
+                    rc = enqueue_step(ctx, m, false);
+                    if (rc) return rc;
+                }
+            }
+            RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));       // `tokens` is the caller's buffer; pf_tok is reused by the next pass
+        }
+        // logits of the last token: rmsnorm + output head on its hidden state
+        rt::GemvArgs a;
+        memset(&a, 0, sizeof a);
+        a.n = 1;
+        a.p[0] = make_prob(m->output, m->x, rt::kStageRms, m->logits, nullptr);
+        a.p[0].gamma = m->out_norm; a.p[0].eps = m->cfg.rms_eps;
+        RT_TRY_HIP(ctx, rt::launch_qgemv(ctx->stream, a, 1));
+        RT_TRY_HIP(ctx, rt::launch_argmax(ctx->stream, m->logits, (size_t)m->cfg.vocab, m->state + 2));
+        RT_TRY_HIP(ctx, rt::launch_set_state(ctx->stream, m->state, pos0 + n_tok, tokens[n_tok - 1], 0));
+        m->n_fed = pos0 + n_tok;
+        return RT_HIP_OK;
+    }
     rc = ensure_mega(ctx, m);
     if (rc) return rc;
     // forced_dev[i] = token fed after step i (the last entry repeats the last token and is never used)

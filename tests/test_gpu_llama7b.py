@@ -36,10 +36,15 @@ def test_full_size_model_matches_oracle_golden(ex):
         if top_vals[0] - top_vals[1] > 2 * tol.max():
             assert pick == int(top_ids[0])
     print("worst |delta| / tol over %d positions: %.3e" % (toks.size, worst), flush=True)
-    # prefill of the same prefix reproduces the logits of stepping
+    # prefill of the same prefix (16 tokens or more: the dense-contraction path on the matrix cores) leaves the
+    # logits of its last token, and stepping on from its cache reproduces the next position
     gm.reset()
     gm.prefill(toks[:-1], 0)
+    err = np.abs(gm.logits()[rows].astype(np.float64) - want[-2])
+    print("prefill of %d tokens: max |delta| / tol = %.3e" % (toks.size - 1, float((err / tol).max())), flush=True)
+    assert np.all(err <= tol)
     gm.step(int(toks[-1]), toks.size - 1)
     err = np.abs(gm.logits()[rows].astype(np.float64) - want[-1])
+    print("step after prefill: max |delta| / tol = %.3e" % float((err / tol).max()), flush=True)
     assert np.all(err <= tol)
     gm.close()
