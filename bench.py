@@ -33,7 +33,7 @@ HBM_PEAK = 8.0e12
 # HBM bytes one launch of the GEMV kernel moves on this workload, from the FETCH_SIZE and WRITE_SIZE hardware
 # counters (each scaled by what the same counter reads for a plain x += y kernel of known size); measured
 # offline with the profiler, since counters cannot be read from inside this process.
-GEMV_TRAFFIC_BYTES = 132_250_931
+GEMV_TRAFFIC_BYTES = 132_266_700
 SEED = 20250127
 H, F, V, NH, NL = 4096, 11008, 32000, 32, 32
 
@@ -180,6 +180,7 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--prefill-only", action="store_true", help="run only the prefill contraction shapes (for kernel traces)")
     ap.add_argument("--decode-prompt", type=int, default=128)
     ap.add_argument("--decode-gen", type=int, default=128)
     ap.add_argument("--calibrate", action="store_true",
@@ -202,6 +203,11 @@ def main():
             ex.add_dev(a, b, n)
         ex.synchronize()
         print(json.dumps({"calibrate": "add_kernel", "launches": 8, "read_bytes_per_launch": 8 * n, "write_bytes_per_launch": 4 * n}), flush=True)
+        ex.close()
+        return
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": bench_prefill(ex)}), flush=True)
         ex.close()
         return
 
