@@ -90,10 +90,51 @@ def bench_layer_gemv(ex, steps, warmup, n_layers):
     k1.record()
     ex.synchronize()
     kern_ms = k0.elapsed_ms(k1) / steps
+    # the same launch on one layer over and over: its 130 MB stay in the 256 MB Infinity Cache
+    h0, h1 = ex.event(), ex.event()
+    for i in range(8):
+        ex.qgemv_xq_grouped_dev(layers[0], xqs, ys)
+    h0.record()
+    for i in range(steps):
+        ex.qgemv_xq_grouped_dev(layers[0], xqs, ys)
+    h1.record()
+    ex.synchronize()
+    hot_ms = h0.elapsed_ms(h1) / steps
     for ws in layers:
         for w in ws:
             w.free()
-    return dict(wbytes=wbytes, abytes=abytes, wall_s=wall, event_ms=ev_ms, kernel_ms=kern_ms)
+    return dict(wbytes=wbytes, abytes=abytes, wall_s=wall, event_ms=ev_ms, kernel_ms=kern_ms, hot_ms=hot_ms)
+
+
+def bench_single_gemv(ex, reps=200):
+    """The single-matrix decode configurations: Q8_0 4096x4096 and Q4_0 at the two FFN shapes, batch 1, x resident
+    in HBM as f32 (quantized in the kernel's staging).  Eight synthetic copies of each matrix are rotated so that
+    the larger ones come from HBM rather than from the Infinity Cache."""
+    from rustorch_amd import synth, GGMLType
+    out = []
+    for name, t, rows, cols in (("q8_0_4096x4096", GGMLType.Q8_0, 4096, 4096),
+                                ("q4_0_11008x4096", GGMLType.Q4_0, 11008, 4096),
+                                ("q4_0_4096x11008", GGMLType.Q4_0, 4096, 11008)):
+        ws = [ex.upload_qweight(t, rows, cols, synth.blocks(t, SEED, 8000 + i, rows, cols)) for i in range(8)]
+        x = ex.to_device(synth.normal(SEED, 8100, cols))
+        y = ex.buffer(4 * rows)
+        for i in range(16):
+            ex.qgemv_dev(ws[i % 8], x, y)
+        ex.synchronize()
+        e0, e1 = ex.event(), ex.event()
+        e0.record()
+        for i in range(reps):
+            ex.qgemv_dev(ws[i % 8], x, y)
+        e1.record()
+        ex.synchronize()
+        ms = e0.elapsed_ms(e1) / reps
+        wbytes = t.row_bytes(cols) * rows
+        out.append({"shape": name, "us": round(ms * 1e3, 2), "weight_gbps": round(wbytes / ms / 1e6, 1),
+                    "hbm_frac": round(wbytes / (ms * 1e-3) / HBM_PEAK, 4)})
+        for w in ws:
+            w.free()
+        x.free(); y.free()
+    return out
 
 
 def bench_decode(ex, n_prompt, n_gen):
@@ -225,8 +266,10 @@ def main():
                    "event_ms_per_step": round(g["event_ms"] / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": GEMV_TRAFFIC_BYTES, "kernel": "qgemv_kernel",
-                     "bytes_per_launch": g["abytes"], "avg_launch_ms": round(g["kernel_ms"], 5)},
+                     "bytes_per_launch": g["abytes"], "avg_launch_ms": round(g["kernel_ms"], 5),
+                     "cache_resident_launch_ms": round(g["hot_ms"], 5)},
     }
+    out["single_gemv"] = bench_single_gemv(ex)
     if not args.no_prefill:
         out["prefill"] = bench_prefill(ex)
     if not args.no_decode:
