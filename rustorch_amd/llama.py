@@ -185,3 +185,39 @@ def load_gguf(ex: HipKernelExecutor, path, max_pos: int | None = None) -> HipLla
             model.close()
             raise
         return model
+
+
+def generate(model: HipLlama, prompt: Iterable[int], max_new_tokens: int, config=None, eos_token: int | None = None,
+             rng=None, pos0: int = 0) -> list[int]:
+    """Prompt in, new tokens out: the loop of `InferenceEngine::generate_with_gpt`
+    (example-cli/src/model/inference.rs:135-192) -- forward, logits of the last position, pick, stop at the
+    end-of-sequence token or at max_new_tokens.  Greedy configurations run entirely on the device
+    (`rt_hip_llama_decode`); anything else reads the logits back each step and samples on the host."""
+    from .sampling import SamplingConfig, sample_token
+    config = config or SamplingConfig.greedy()
+    config.validate()
+    toks = [int(t) for t in prompt]
+    if not toks:
+        raise ValueError("generate: empty prompt")
+    room = model.cfg.max_pos - (pos0 + len(toks)) + 1
+    n_new = min(max_new_tokens, room)
+    if n_new <= 0:
+        return []
+    if len(toks) > 1:
+        model.prefill(toks[:-1], pos0)
+    pos = pos0 + len(toks) - 1
+    if config.is_greedy and config.repetition_penalty == 1.0:
+        out = [int(t) for t in model.decode(toks[-1], pos, n_new)]
+        if eos_token is not None and eos_token in out:
+            out = out[:out.index(eos_token) + 1]
+        return out
+    out: list[int] = []
+    cur = toks[-1]
+    for _ in range(n_new):
+        model.step(cur, pos, want_token=False)
+        cur = sample_token(model.logits(), config, toks + out, rng)
+        out.append(cur)
+        pos += 1
+        if eos_token is not None and cur == eos_token:
+            break
+    return out

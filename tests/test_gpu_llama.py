@@ -144,3 +144,30 @@ def test_model_from_gguf_file_equals_direct_upload(ex, orc, tmp_path):
     w.write(tmp_path / "empty.gguf")
     with pytest.raises(InvalidParameters):
         llama.load_gguf(ex, tmp_path / "empty.gguf")
+
+
+def test_generate_greedy_and_sampled(ex, orc):
+    from rustorch_amd import llama, synth
+    from rustorch_amd.sampling import SamplingConfig
+    cfg = dict(n_layers=2, hidden=256, n_heads=2, ffn=512, vocab=200, max_pos=40)
+    print("llama generate", cfg, flush=True)
+    gm, om, wn = build_pair(ex, orc, 41, **cfg)
+    prompt = [int(t) for t in synth.tokens(41, synth.TID_PROMPT, 6, cfg["vocab"])]
+    greedy = llama.generate(gm, prompt, 10)
+    assert len(greedy) == 10
+    # the host-sampled loop with top_k = 1 walks the same path as the device-side greedy loop
+    gm.reset()
+    again = llama.generate(gm, prompt, 10, SamplingConfig(temperature=0.7, top_k=1, repetition_penalty=1.0000001))
+    assert again == greedy
+    # a seeded draw is reproducible, stays inside the vocabulary and stops at the end-of-sequence token
+    runs = []
+    for _ in range(2):
+        gm.reset()
+        runs.append(llama.generate(gm, prompt, 12, SamplingConfig.with_top_k(5, 0.9), rng=np.random.default_rng(7)))
+    assert runs[0] == runs[1] and all(0 <= t < cfg["vocab"] for t in runs[0])
+    gm.reset()
+    stop = llama.generate(gm, prompt, 10, eos_token=greedy[3])
+    assert stop == greedy[:greedy.index(greedy[3]) + 1]
+    # never past the cache: 6 prompt tokens leave 35 positions
+    gm.reset()
+    assert len(llama.generate(gm, prompt, 1000)) == cfg["max_pos"] - len(prompt) + 1
