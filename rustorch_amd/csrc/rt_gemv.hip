@@ -1,17 +1,23 @@
 // Stand-alone dequant-fused GEMV launch (decode, batch 1..8): y = dequant(W) . x with W in raw GGUF blocks.
-// One workgroup of 1024 threads per CU; device code in rt_gemv_device.h.
+// Workgroups of 1024 threads (one per CU) for small launches, of 512 threads (two per CU) for large ones;
+// device code in rt_gemv_device.h.
 #include "rt_gemv_device.h"
 
 namespace rt {
 
 namespace {
 
-constexpr int kGemvThreads = 1024;
-constexpr int kGemvWaves = kGemvThreads / 64;
+// Launches that stream less than this many weight bytes use 1024-thread workgroups: with few rows per wave
+// the start-up (one staging of x per workgroup) dominates and fewer, larger workgroups pay it less often.
+// Larger launches run faster with two 512-thread workgroups per CU, which do not stall on each other's barriers.
+#ifndef RT_GEMV_BIG_BYTES
+#define RT_GEMV_BIG_BYTES (64.0 * 1024 * 1024)
+#endif
 
-__global__ __launch_bounds__(kGemvThreads) void qgemv_kernel(GemvArgs a, int r2) {
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void qgemv_kernel(GemvArgs a, int r2) {
     RT_DYN_LDS(uint4, lds4);
-    __shared__ float red[kGemvWaves];
+    __shared__ float red[THREADS / 64];
     uint32_t *lds = reinterpret_cast<uint32_t *>(lds4);
     const int wg = blockIdx.x;
     int pi = 0;
@@ -37,8 +43,10 @@ hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
         if ((size_t)a.p[i].K > maxK) maxK = (size_t)a.p[i].K;
     }
     if (total_bytes <= 0) return hipErrorInvalidValue;
-    // one resident workgroup (16 waves) per CU over 256 CUs
-    int budget = 256 / batch;
+    // 16 resident waves per CU over 256 CUs, as one or two workgroups
+    const int threads = total_bytes >= RT_GEMV_BIG_BYTES ? 512 : 1024;
+    const int kGemvWaves = threads / 64;
+    int budget = 256 * (1024 / threads) / batch;
     if (budget < a.n) budget = a.n;
     // two rows per wave step once every wave has at least three steps of work, else one
     const int r2 = total_rows >= (size_t)3 * 2 * (size_t)budget * kGemvWaves ? 1 : 0;
@@ -57,7 +65,8 @@ hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
     }
     size_t lds = xq_stride(maxK);
     dim3 grid((unsigned)wgs, (unsigned)batch);
-    qgemv_kernel<<<grid, kGemvThreads, lds, s>>>(a, r2);
+    if (threads == 512) qgemv_kernel<512><<<grid, 512, lds, s>>>(a, r2);
+    else qgemv_kernel<1024><<<grid, 1024, lds, s>>>(a, r2);
     return hipGetLastError();
 }
 
