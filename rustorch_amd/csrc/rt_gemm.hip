@@ -437,7 +437,7 @@ __device__ __forceinline__ void superblock(float16v (&acc)[MF], const WSb<TYPE> 
             __builtin_amdgcn_sched_barrier(0);
             static_for<0, MF>([&](auto J) {
                 constexpr int j = decltype(J)::value;
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bb[cur][j], acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bb[cur][j], a, acc[j], 0, 0, 0);
                 static_for<j * UPM, (j + 1) * UPM < 4 ? (j + 1) * UPM : 4>([&](auto Q) {
                     constexpr int q = decltype(Q)::value;
                     if constexpr (tn < 4) an[q] = expand_unit(w, k, tn, sn, q, G);
@@ -558,23 +558,56 @@ __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t
     }
     wait_vmcnt_c<0>();           // the loads issued past the end of the range still target this workgroup's LDS
 
-    // D[i][j]: j (token) = lane % 32; i (weight row) = 8*(r/4) + 4*(lane/32) + r%4
+    // X fragments are the first operand, so D = X . W^T: register r of lane L holds token 8*(r/4) + 4*(L/32) + r%4
+    // of the fragment and weight row L % 32.  A store instruction then writes two runs of 32 consecutive floats.
     float *Yp = Y_out + (size_t)kz * plane_stride;
+    const int n = n0 + wave * 32 + nl;
+    const bool add_res = res && ksplit == 1;
+    // the scales of the lane's tokens, four consecutive ones per load (the array is padded past M)
+    float4 inv[MF][4];
 #pragma unroll
-    for (int i = 0; i < MF; i++) {
-        const int m = m0 + i * 32 + nl;
-        if (m >= M) continue;
-        const float inv = inv_scale[m];
+    for (int i = 0; i < MF; i++)
 #pragma unroll
-        for (int g4 = 0; g4 < 4; g4++) {
-            const int n = n0 + wave * 32 + 8 * g4 + 4 * h;
-            if (n >= N) continue;   // N is a multiple of 4: a group of 4 rows is inside or outside as a whole
-            float4 v = make_float4(acc[i][4 * g4] * inv, acc[i][4 * g4 + 1] * inv, acc[i][4 * g4 + 2] * inv, acc[i][4 * g4 + 3] * inv);
-            if (res && ksplit == 1) {
-                float4 rv = *reinterpret_cast<const float4 *>(res + (size_t)m * N + n);
-                v.x += rv.x; v.y += rv.y; v.z += rv.z; v.w += rv.w;
+        for (int g = 0; g < 4; g++) {
+            const int mb = m0 + i * 32 + 8 * g + 4 * h;
+            inv[i][g] = mb < M ? *reinterpret_cast<const float4 *>(inv_scale + mb) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    auto scaled = [&](int i, int r) {
+        const float4 q = inv[i][r >> 2];
+        return acc[i][r] * ((r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w);
+    };
+    if (m0 + BM <= M && n0 + BN <= N) {
+        // whole tile inside the matrix: no per-element guards, so the stores go out back to back (a guard is a
+        // branch, and behind a branch the compiler waits for every earlier store before the next one)
+        float *yp = Yp + (size_t)(m0 + 4 * h) * N + n;
+        if (add_res) {
+            const float *rp = res + (size_t)(m0 + 4 * h) * N + n;
+#pragma unroll
+            for (int i = 0; i < MF; i++) {
+                float rv[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) rv[r] = rp[(size_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * N];
+#pragma unroll
+                for (int r = 0; r < 16; r++) yp[(size_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * N] = scaled(i, r) + rv[r];
             }
-            *reinterpret_cast<float4 *>(Yp + (size_t)m * N + n) = v;
+        } else {
+#pragma unroll
+            for (int i = 0; i < MF; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) yp[(size_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * N] = scaled(i, r);
+        }
+    } else if (n < N) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): the scales, before the guarded stores
+#pragma unroll
+        for (int i = 0; i < MF; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (m >= M) continue;
+                float v = scaled(i, r);
+                if (add_res) v += res[(size_t)m * N + n];
+                Yp[(size_t)m * N + n] = v;
+            }
         }
     }
 }
