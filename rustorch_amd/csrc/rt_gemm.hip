@@ -532,12 +532,12 @@ __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t
     WTmp<TYPE> tmp;
     WSb<TYPE> wA, wB;
     SbK<TYPE> kA, kB;
+    static_for<0, Ride<TYPE>::n_load>([&](auto O) { load_op<TYPE, decltype(O)::value>(tmp, woff, wbase + (size_t)sb0 * Geo::blk, lane); });
 #pragma unroll
     for (int d = 0; d < 3; d++)
 #pragma unroll
-        for (int i = 0; i < XI; i++) issue_x(kt0 + d, d, i);
-    static_for<0, Ride<TYPE>::n_load>([&](auto O) { load_op<TYPE, decltype(O)::value>(tmp, woff, wbase + (size_t)sb0 * Geo::blk, lane); });
-    wait_vmcnt_c<0>();
+        for (int i = 0; i < XI; i++) issue_x(min(kt0 + d, kt_last), d, i);
+    wait_vmcnt_c<3 * XI>();                // the weights have landed, the X tiles may still be in flight
     __builtin_amdgcn_sched_barrier(0);
     static_for<0, Ride<TYPE>::n_park>([&](auto O) { park_op<TYPE, decltype(O)::value>(tmp, la.wpark, lane); });
     static_for<0, Ride<TYPE>::n_fetch>([&](auto O) { fetch_op<decltype(O)::value>(wA, la.wrow, la.wrow_h, la.wtail); });
@@ -545,6 +545,7 @@ __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t
     __builtin_amdgcn_sched_barrier(0);     // the scheduler does not know that the wait guards wA
     static_for<0, kPrepPieces>([&](auto P) { prep_piece(kA, wA, h, decltype(P)::value); });
     half8v a = expand_step(wA, kA, 0, 0, G), bb[2][MF];
+    wait_vmcnt_c<2 * XI>();                // this wave's part of X tile 0
     __builtin_amdgcn_s_barrier();
     static_for<0, MF>([&](auto I) { bb[0][decltype(I)::value] = lds_read16<decltype(I)::value * 32 * kBK * 2>(la.b[0]); });
 

@@ -301,7 +301,9 @@ struct Walker {
     __device__ __forceinline__ int group_of(int s) const { return gw + (s / n_iter) * n_gw; }
     __device__ __forceinline__ int unit_of(int s) const { return lane + 64 * (s % n_iter); }
 
-    __device__ __forceinline__ void request(WRegs<TYPE> *w, int s) const {
+    // rv: the residual values of the step's rows, requested with the weights so that the row end has no load
+    // of its own to wait for (a wait for the youngest load would also wait for every prefetch before it)
+    __device__ __forceinline__ void request(WRegs<TYPE> *w, float *rv, int s) const {
         const int g = group_of(s);
         const int u = min(unit_of(s), U - 1);  // lanes past the end of the row reread the last unit; masked later
 #pragma unroll
@@ -310,13 +312,14 @@ struct Walker {
             row = min(row, P.N - 1);  // ragged tail: reread the last row, the store is skipped
             const uint8_t *rp = ((dual && (r & 1)) ? P.w2 : P.w) + (size_t)row * P.row_bytes;
             load_w(w[r], rp, u);
+            if (!dual && P.res) rv[r] = ld_f<COH>(&P.res[(size_t)m * P.N + row]);
         }
     }
 
     // x slice of the unit a lane works on in step s (rows of <= 64 units: the same slice in every step)
     __device__ __forceinline__ void fetch_x(XRegs<TYPE> &x, int s) const { load_x(x, lds, min(unit_of(s), U - 1), U, P.K); }
 
-    __device__ __forceinline__ void consume(const WRegs<TYPE> *w, const XRegs<TYPE> &x, int s, float *acc) const {
+    __device__ __forceinline__ void consume(const WRegs<TYPE> *w, const float *rv, const XRegs<TYPE> &x, int s, float *acc) const {
         const int u = unit_of(s);
         const int uc = min(u, U - 1);
         const float live = u < U ? 1.f : 0.f;
@@ -341,7 +344,7 @@ struct Walker {
                 int row = g * rows_per_group + r;
                 if (lane == r && row < P.N) {
                     size_t o = (size_t)m * P.N + row;
-                    st_f<COH>(&P.y[o], P.res ? ld_f<COH>(&P.res[o]) + acc[r] : acc[r]);
+                    st_f<COH>(&P.y[o], P.res ? rv[r] + acc[r] : acc[r]);
                 }
             }
         }
@@ -364,7 +367,10 @@ __device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg
     const int my_groups = W.gw < W.n_groups ? (W.n_groups - W.gw + W.n_gw - 1) / W.n_gw : 0;
     const int steps = my_groups * W.n_iter;
     WRegs<TYPE> a[R], b[R];
-    if (steps > 0) W.request(a, 0);      // in flight while x is being staged
+    float ra[R], rb[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) ra[r] = rb[r] = 0.f;
+    if (steps > 0) W.request(a, ra, 0);      // in flight while x is being staged
     stage_x<COH>(P, m, lds, red);
     float acc[R];
 #pragma unroll
@@ -374,22 +380,22 @@ __device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg
         // every step of this lane meets the same x slice: keep it in registers, LDS is read once
         W.fetch_x(x, 0);
         for (int s = 0; s < steps; s += 2) {
-            if (s + 1 < steps) W.request(b, s + 1);
-            W.consume(a, x, s, acc);
+            if (s + 1 < steps) W.request(b, rb, s + 1);
+            W.consume(a, ra, x, s, acc);
             if (s + 1 < steps) {
-                if (s + 2 < steps) W.request(a, s + 2);
-                W.consume(b, x, s + 1, acc);
+                if (s + 2 < steps) W.request(a, ra, s + 2);
+                W.consume(b, rb, x, s + 1, acc);
             }
         }
     } else {
         for (int s = 0; s < steps; s += 2) {
-            if (s + 1 < steps) W.request(b, s + 1);
+            if (s + 1 < steps) W.request(b, rb, s + 1);
             W.fetch_x(x, s);
-            W.consume(a, x, s, acc);
+            W.consume(a, ra, x, s, acc);
             if (s + 1 < steps) {
-                if (s + 2 < steps) W.request(a, s + 2);
+                if (s + 2 < steps) W.request(a, ra, s + 2);
                 W.fetch_x(x, s + 1);
-                W.consume(b, x, s + 1, acc);
+                W.consume(b, rb, x, s + 1, acc);
             }
         }
     }
