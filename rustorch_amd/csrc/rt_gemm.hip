@@ -557,7 +557,12 @@ __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t
                                  4 * sb, kt_last, issue_x);
         if (++sb >= sb1) break;
     }
-    wait_vmcnt_c<0>();           // the loads issued past the end of the range still target this workgroup's LDS
+    // The last step leaves loads in flight (X tiles past the end of the range into this workgroup's LDS, and
+    // the LDS reads of the operands of a step that does not follow).  Their destination registers are dead
+    // to the compiler, which would hand them to the code below while the data is still on its way.
+    wait_vmcnt_c<0>();
+    wait_lgkmcnt_c<0>();
+    __builtin_amdgcn_sched_barrier(0);
 
     // X fragments are the first operand, so D = X . W^T: register r of lane L holds token 8*(r/4) + 4*(L/32) + r%4
     // of the fragment and weight row L % 32.  A store instruction then writes two runs of 32 consecutive floats.
