@@ -298,34 +298,38 @@ struct Walker {
     int m, U, n_iter, lane, gw, n_gw, n_groups, rows_per_group;
     bool dual;
 
-    __device__ __forceinline__ int group_of(int s) const { return gw + (s / n_iter) * n_gw; }
-    __device__ __forceinline__ int unit_of(int s) const { return lane + 64 * (s % n_iter); }
+    // A step is (row group g, unit pass p); steps are walked in order, so the position is advanced, not divided out.
+    struct Pos { int g, p; };
+    __device__ __forceinline__ Pos first() const { return Pos{ gw, 0 }; }
+    __device__ __forceinline__ Pos next(Pos q) const { return q.p + 1 == n_iter ? Pos{ q.g + n_gw, 0 } : Pos{ q.g, q.p + 1 }; }
+    __device__ __forceinline__ int group_of(Pos q) const { return q.g; }
+    __device__ __forceinline__ int unit_of(Pos q) const { return lane + 64 * q.p; }
 
     // rv: the residual values of the step's rows, requested with the weights so that the row end has no load
     // of its own to wait for (a wait for the youngest load would also wait for every prefetch before it)
-    __device__ __forceinline__ void request(WRegs<TYPE> *w, float *rv, int s) const {
+    __device__ __forceinline__ void request(WRegs<TYPE> *w, float *rv, Pos s) const {
         const int g = group_of(s);
         const int u = min(unit_of(s), U - 1);  // lanes past the end of the row reread the last unit; masked later
 #pragma unroll
         for (int r = 0; r < R; r++) {
             int row = dual ? g * rows_per_group + (r >> 1) : g * rows_per_group + r;
             row = min(row, P.N - 1);  // ragged tail: reread the last row, the store is skipped
-            const uint8_t *rp = ((dual && (r & 1)) ? P.w2 : P.w) + (size_t)row * P.row_bytes;
+            const uint8_t *rp = ((dual && (r & 1)) ? P.w2 : P.w) + (uint32_t)row * (uint32_t)P.row_bytes;   // a tensor is below 4 GB (checked at launch)
             load_w(w[r], rp, u);
             if (!dual && P.res) rv[r] = ld_f<COH>(&P.res[(size_t)m * P.N + row]);
         }
     }
 
     // x slice of the unit a lane works on in step s (rows of <= 64 units: the same slice in every step)
-    __device__ __forceinline__ void fetch_x(XRegs<TYPE> &x, int s) const { load_x(x, lds, min(unit_of(s), U - 1), U, P.K); }
+    __device__ __forceinline__ void fetch_x(XRegs<TYPE> &x, Pos s) const { load_x(x, lds, min(unit_of(s), U - 1), U, P.K); }
 
-    __device__ __forceinline__ void consume(const WRegs<TYPE> *w, const float *rv, const XRegs<TYPE> &x, int s, float *acc) const {
+    __device__ __forceinline__ void consume(const WRegs<TYPE> *w, const float *rv, const XRegs<TYPE> &x, Pos s, float *acc) const {
         const int u = unit_of(s);
         const int uc = min(u, U - 1);
         const float live = u < U ? 1.f : 0.f;
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] = __builtin_fmaf(live, dot_unit(w[r], x, uc), acc[r]);
-        if (s % n_iter != n_iter - 1) return;
+        if (s.p != n_iter - 1) return;
         const int g = group_of(s);
 #pragma unroll
         for (int r = 0; r < R; r++) acc[r] = wave_sum_dpp(acc[r]);
@@ -370,7 +374,9 @@ __device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg
     float ra[R], rb[R];
 #pragma unroll
     for (int r = 0; r < R; r++) ra[r] = rb[r] = 0.f;
-    if (steps > 0) W.request(a, ra, 0);      // in flight while x is being staged
+    using Pos = typename Walker<TYPE, R, COH>::Pos;
+    Pos pa = W.first(), pb = W.next(pa);     // positions of the steps held in a and b
+    if (steps > 0) W.request(a, ra, pa);     // in flight while x is being staged
     stage_x<COH>(P, m, lds, red);
     float acc[R];
 #pragma unroll
@@ -378,24 +384,28 @@ __device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg
     XRegs<TYPE> x;
     if (R == 1 && W.n_iter == 1) {
         // every step of this lane meets the same x slice: keep it in registers, LDS is read once
-        W.fetch_x(x, 0);
+        W.fetch_x(x, pa);
         for (int s = 0; s < steps; s += 2) {
-            if (s + 1 < steps) W.request(b, rb, s + 1);
-            W.consume(a, ra, x, s, acc);
+            if (s + 1 < steps) W.request(b, rb, pb);
+            W.consume(a, ra, x, pa, acc);
+            pa = W.next(pb);
             if (s + 1 < steps) {
-                if (s + 2 < steps) W.request(a, ra, s + 2);
-                W.consume(b, rb, x, s + 1, acc);
+                if (s + 2 < steps) W.request(a, ra, pa);
+                W.consume(b, rb, x, pb, acc);
+                pb = W.next(pa);
             }
         }
     } else {
         for (int s = 0; s < steps; s += 2) {
-            if (s + 1 < steps) W.request(b, rb, s + 1);
-            W.fetch_x(x, s);
-            W.consume(a, ra, x, s, acc);
+            if (s + 1 < steps) W.request(b, rb, pb);
+            W.fetch_x(x, pa);
+            W.consume(a, ra, x, pa, acc);
+            pa = W.next(pb);
             if (s + 1 < steps) {
-                if (s + 2 < steps) W.request(a, ra, s + 2);
-                W.fetch_x(x, s + 1);
-                W.consume(b, rb, x, s + 1, acc);
+                if (s + 2 < steps) W.request(a, ra, pa);
+                W.fetch_x(x, pb);
+                W.consume(b, rb, x, pb, acc);
+                pb = W.next(pa);
             }
         }
     }
