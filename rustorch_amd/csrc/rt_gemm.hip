@@ -701,8 +701,10 @@ size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K) {
 }
 
 // res (optional) is added to the result; it may be Y itself only on the row-by-row path.
+// x_prepared: the workspace still holds the pre-pass of this very X (same M and K) from the previous call, as
+// when several weights meet one activation matrix; the pre-pass is then skipped.
 hipError_t launch_qgemm(hipStream_t s, int type, const uint8_t *w, size_t N, size_t K, size_t row_bytes,
-                        const float *X, size_t M, float *Y, const float *res, void *scratch, size_t scratch_bytes) {
+                        const float *X, size_t M, float *Y, const float *res, void *scratch, size_t scratch_bytes, bool x_prepared) {
     if (mfma_path(type, N, K, M) && res != Y) {
         if (scratch_bytes < qgemm_scratch_bytes(type, M, N, K)) return hipErrorInvalidValue;
         const GemmPlan p = gemm_plan(M, N, K);
@@ -710,9 +712,11 @@ hipError_t launch_qgemm(hipStream_t s, int type, const uint8_t *w, size_t N, siz
         _Float16 *Xp = reinterpret_cast<_Float16 *>(base);
         float *inv_scale = reinterpret_cast<float *>(base + align256(M * K * sizeof(_Float16)));
         float *partial = reinterpret_cast<float *>(base + align256(M * K * sizeof(_Float16)) + align256(M * sizeof(float)));
-        xprep_kernel<<<dim3((unsigned)M), 256, 0, s>>>(X, K, Xp, inv_scale);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
+        if (!x_prepared) {
+            xprep_kernel<<<dim3((unsigned)M), 256, 0, s>>>(X, K, Xp, inv_scale);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+        }
         if (type == RT_GGML_Q4_K) return launch_type<RT_GGML_Q4_K>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
         return launch_type<RT_GGML_Q6_K>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
     }

@@ -146,7 +146,8 @@ hipError_t launch_step_advance(hipStream_t s, int *pos_dev, int *token_dev, cons
                                const int *forced_dev, int *out_tokens_dev, int *step_dev);
 // prefill GEMM (rt_gemm.hip)
 hipError_t launch_qgemm(hipStream_t s, int type, const uint8_t *w, size_t N, size_t K, size_t row_bytes,
-                        const float *X, size_t M, float *Y, const float *res, void *scratch, size_t scratch_bytes);
+                        const float *X, size_t M, float *Y, const float *res, void *scratch, size_t scratch_bytes,
+                        bool x_prepared = false);
 size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K);
 
 inline size_t type_block_bytes(int t) {

@@ -168,8 +168,10 @@ int ensure_prefill_buffers(rt_hip_ctx *ctx, rt_hip_llama *m, size_t n_tok) {
     return RT_HIP_OK;
 }
 
-int gemm(rt_hip_ctx *ctx, const rt_hip_llama::T &t, const float *X, size_t M, float *Y, const float *res) {
-    RT_TRY_HIP(ctx, rt::launch_qgemm(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, X, M, Y, res, ctx->scratch, ctx->scratch_bytes));
+// same_x: X is the matrix the previous call was given, its pre-pass is still in the workspace
+int gemm(rt_hip_ctx *ctx, const rt_hip_llama::T &t, const float *X, size_t M, float *Y, const float *res, bool same_x = false) {
+    RT_TRY_HIP(ctx, rt::launch_qgemm(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, X, M, Y, res, ctx->scratch, ctx->scratch_bytes,
+                                     same_x));
     return RT_HIP_OK;
 }
 
@@ -193,8 +195,8 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
         uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * H;
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->attn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
         if ((rc = gemm(ctx, m->wq[l], m->pf_n, M, m->pf_q, nullptr))) return rc;
-        if ((rc = gemm(ctx, m->wk[l], m->pf_n, M, m->pf_k, nullptr))) return rc;
-        if ((rc = gemm(ctx, m->wv[l], m->pf_n, M, m->pf_v, nullptr))) return rc;
+        if ((rc = gemm(ctx, m->wk[l], m->pf_n, M, m->pf_k, nullptr, true))) return rc;
+        if ((rc = gemm(ctx, m->wv[l], m->pf_n, M, m->pf_v, nullptr, true))) return rc;
         RT_TRY_HIP(ctx, rt::launch_rope_kv_batch(s, m->pf_q, m->pf_k, m->pf_v, kc, vc, pos0, M, c.n_heads, m->head_dim, m->inv_freq));
         RT_TRY_HIP(ctx, rt::launch_attn_batch(s, m->pf_q, nullptr, nullptr, kc, vc, nullptr, pos0 + 1, M, c.n_heads, m->head_dim,
                                               m->inv_freq, m->pf_a, nullptr, false));
@@ -202,7 +204,7 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
         std::swap(x, x2);
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->ffn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
         if ((rc = gemm(ctx, m->wgate[l], m->pf_n, M, m->pf_g, nullptr))) return rc;
-        if ((rc = gemm(ctx, m->wup[l], m->pf_n, M, m->pf_u, nullptr))) return rc;
+        if ((rc = gemm(ctx, m->wup[l], m->pf_n, M, m->pf_u, nullptr, true))) return rc;
         RT_TRY_HIP(ctx, rt::launch_swiglu(s, m->pf_g, m->pf_u, m->pf_g, nullptr, M * F));
         if ((rc = gemm(ctx, m->wdown[l], m->pf_g, M, x2, x))) return rc;
         std::swap(x, x2);
