@@ -107,6 +107,18 @@ RT_HIP_API int rt_hip_event_destroy(rt_hip_ctx *ctx, rt_hip_event *ev);
 RT_HIP_API int rt_hip_matmul_f32(rt_hip_ctx *ctx, const float *a, const float *b, float *c, size_t m, size_t n,
                                  size_t k);
 
+/* ---- per-tensor affine int8 matmul: QuantizedOps::qmatmul
+ *      (src/quantization/operations.rs:195-260), which OptimizedOps::qmatmul
+ *      (src/quantization/hardware/mod.rs:25-46) reaches on every device through
+ *      qmatmul_cuda / qmatmul_cpu (hardware/cuda.rs:12-26, hardware/cpu.rs:281-288).
+ *      Row-major a[m,k] . b[k,n] with zero points removed, summed exactly; the
+ *      result is re-quantized to int8 with scale scale_a*scale_b (returned in
+ *      *out_scale) and zero point 0 (*out_zero_point).  Host slices, blocking.
+ *      Zero points beyond +-1024 are refused (RT_HIP_ERR_INVALID_ARG). */
+RT_HIP_API int rt_hip_qmatmul_i8(rt_hip_ctx *ctx, const int8_t *a, float scale_a, int zero_point_a, const int8_t *b,
+                                 float scale_b, int zero_point_b, size_t m, size_t n, size_t k, int8_t *out,
+                                 float *out_scale, int *out_zero_point);
+
 /* ---- quantized weights under Linear / qmatmul: the device arm of
  *      OptimizedOps::qmatmul (src/quantization/hardware/mod.rs:25-46) and the
  *      weight side of Linear::forward (src/nn/linear.rs:150-182, W stored [out,in]).

@@ -37,6 +37,7 @@ def load() -> C.CDLL:
         "orc_dequant": (i, [i, vp, sz, sz, vp]),
         "orc_dequant_nt": (i, [i, vp, sz, sz, vp, i]),
         "orc_matmul_xwt": (None, [vp, vp, vp, sz, sz, sz, i]),
+        "orc_qmatmul_i8": (C.c_float, [vp, C.c_float, i, vp, C.c_float, i, sz, sz, sz, vp]),
         "orc_qgemv": (i, [i, vp, sz, sz, vp, sz, vp, i]),
         "orc_qgemm": (i, [i, vp, sz, sz, vp, sz, vp, i]),
         "orc_qgemv_f64": (i, [i, vp, sz, sz, vp, sz, vp, vp, i]),
@@ -96,6 +97,18 @@ def matmul_xwt(x: np.ndarray, w: np.ndarray, nthreads: int = 0) -> np.ndarray:
     y = np.empty((x2.shape[0], w.shape[0]), dtype=np.float32)
     load().orc_matmul_xwt(_p(x2), _p(w), _p(y), x2.shape[0], w.shape[0], w.shape[1], nthreads or num_threads())
     return y[0] if x.ndim == 1 else y
+
+
+def qmatmul_i8(a: np.ndarray, scale_a: float, zp_a: int, b: np.ndarray, scale_b: float, zp_b: int):
+    """Per-tensor affine int8 matmul (operations.rs:195-260): returns (int8 [m,n], output scale, zero point 0)."""
+    a = np.ascontiguousarray(a, dtype=np.int8); b = np.ascontiguousarray(b, dtype=np.int8)
+    m, k = a.shape
+    k2, n = b.shape
+    if k != k2:
+        raise ValueError("oracle: inner dimensions differ")
+    out = np.empty((m, n), dtype=np.int8)
+    scale = load().orc_qmatmul_i8(_p(a), scale_a, zp_a, _p(b), scale_b, zp_b, m, n, k, _p(out))
+    return out, float(scale), 0
 
 
 def qgemv(ggml_type: int, raw, n_rows: int, n_cols: int, x: np.ndarray, nthreads: int = 0) -> np.ndarray:

@@ -253,6 +253,33 @@ ORC_API void orc_matmul_xwt(const float *x, const float *w, float *y, size_t M, 
 }
 
 /*
+ * Per-tensor affine int8 matmul: QuantizedOps::qmatmul (src/quantization/operations.rs:195-260), the routine
+ * OptimizedOps::qmatmul ends in on every device (hardware/mod.rs:25-46 -> hardware/cpu.rs:281-288).
+ * a[m,k], b[k,n] row-major; sum = sum_l (a - za)(b - zb) in 64-bit; the result is re-quantized with the
+ * output scale sa*sb and zero point 0:  q = round(((float)sum * scale) / scale), clamped to int8
+ * (Rust's `as i32` maps NaN to 0 and saturates; f32::round rounds halves away from zero, as roundf does).
+ * Returns the output scale.
+ */
+ORC_API float orc_qmatmul_i8(const int8_t *a, float sa, int za, const int8_t *b, float sb, int zb, size_t m, size_t n, size_t k,
+                             int8_t *out) {
+    const float scale = sa * sb;
+    for (size_t i = 0; i < m; i++)
+        for (size_t j = 0; j < n; j++) {
+            long long sum = 0;
+            for (size_t l = 0; l < k; l++) sum += (long long)((int)a[i * k + l] - za) * (long long)((int)b[l * n + j] - zb);
+            volatile float fp = (float)sum * scale;      /* two roundings, as written in the reference */
+            float q = roundf(fp / scale);
+            int v;
+            if (q != q) v = 0;
+            else if (q >= 2147483648.0f) v = 2147483647;
+            else if (q <= -2147483648.0f) v = -2147483647 - 1;
+            else v = (int)q;
+            out[i * n + j] = (int8_t)(v > 127 ? 127 : (v < -128 ? -128 : v));
+        }
+    return scale;
+}
+
+/*
  * Same numbers as orc_dequant + orc_matmul_xwt without materialising W: each
  * row is decoded into a scratch line and consumed at once.  Four rows are
  * interleaved so four independent chains hide the add latency; each chain is

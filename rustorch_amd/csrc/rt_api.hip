@@ -240,6 +240,30 @@ int rt_hip_matmul_f32(rt_hip_ctx *ctx, const float *a, const float *b, float *c,
     return RT_HIP_OK;
 }
 
+int rt_hip_qmatmul_i8(rt_hip_ctx *ctx, const int8_t *a, float scale_a, int zero_point_a, const int8_t *b, float scale_b,
+                      int zero_point_b, size_t m, size_t n, size_t k, int8_t *out, float *out_scale, int *out_zero_point) {
+    if (!ctx) return fail(nullptr, RT_HIP_ERR_INVALID_ARG, "ctx is NULL");
+    RT_REQUIRE(ctx, a && b && out, RT_HIP_ERR_INVALID_ARG, "qmatmul_i8: NULL operand");
+    RT_REQUIRE(ctx, m > 0 && n > 0 && k > 0, RT_HIP_ERR_SHAPE, "qmatmul_i8: empty dimension (m=%zu n=%zu k=%zu)", m, n, k);
+    RT_REQUIRE(ctx, zero_point_a >= -1024 && zero_point_a <= 1024 && zero_point_b >= -1024 && zero_point_b <= 1024,
+               RT_HIP_ERR_INVALID_ARG, "qmatmul_i8: zero points %d, %d outside -1024..1024", zero_point_a, zero_point_b);
+    Guard g(ctx);
+    size_t ab = align_up(m * k, 256), bb = align_up(k * n, 256), cb = m * n;
+    int rc = ensure_scratch(ctx, ab + bb + cb);
+    if (rc) return rc;
+    char *base = (char *)ctx->scratch;
+    int8_t *da = (int8_t *)base, *db = (int8_t *)(base + ab), *dc = (int8_t *)(base + ab + bb);
+    const float scale = scale_a * scale_b;       // "output scale is product of input scales"
+    RT_TRY_HIP(ctx, hipMemcpyAsync(da, a, m * k, hipMemcpyHostToDevice, ctx->stream));
+    RT_TRY_HIP(ctx, hipMemcpyAsync(db, b, k * n, hipMemcpyHostToDevice, ctx->stream));
+    RT_TRY_HIP(ctx, rt::launch_qmatmul_i8(ctx->stream, da, db, dc, m, n, k, zero_point_a, zero_point_b, scale));
+    RT_TRY_HIP(ctx, hipMemcpyAsync(out, dc, cb, hipMemcpyDeviceToHost, ctx->stream));
+    RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (out_scale) *out_scale = scale;
+    if (out_zero_point) *out_zero_point = 0;
+    return RT_HIP_OK;
+}
+
 // --------------------------------------------------------- quantized weights
 
 static int qweight_check(rt_hip_ctx *ctx, int type, size_t n_rows, size_t n_cols, size_t nbytes, size_t *row_bytes) {

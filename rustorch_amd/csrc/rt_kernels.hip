@@ -430,7 +430,79 @@ __global__ __launch_bounds__(1024) void matmul_f32_kernel(const float *a, const 
     if (row < m && col < n) c[row * n + col] = acc;
 }
 
+// Per-tensor affine int8 matmul (QuantizedOps::qmatmul, src/quantization/operations.rs:195-260):
+// out[i][j] = clamp_i8(round(((float)sum * scale) / scale)), sum = sum_l (a[i][l] - za)(b[l][j] - zb), scale = sa * sb.
+// 64x64 output tile per workgroup of 256 threads (4x4 outputs each), 64-deep k slices through LDS; a slice is
+// summed in 32-bit (|term| <= 383^2, 64 terms) and added to a 64-bit total, so the sum is exact as in the
+// reference's i64.  The float tail is kept free of contraction: its two roundings are part of the result.
+#pragma clang fp contract(off)
+__global__ __launch_bounds__(256) void qmatmul_i8_kernel(const int8_t *a, const int8_t *b, int8_t *out, size_t m, size_t n, size_t k,
+                                                         int za, int zb, float scale) {
+    __shared__ int16_t as[64][64 + 2];     // [row][l], zero point already removed
+    __shared__ int16_t bs[64][64 + 2];     // [l][col]
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const size_t row0 = (size_t)blockIdx.y * 64, col0 = (size_t)blockIdx.x * 64;
+    long long acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = 0;
+    for (size_t k0 = 0; k0 < k; k0 += 64) {
+        for (int e = threadIdx.x; e < 64 * 64; e += 256) {
+            const int r = e >> 6, c = e & 63;
+            as[r][c] = (row0 + r < m && k0 + c < k) ? (int16_t)((int)a[(row0 + r) * k + k0 + c] - za) : (int16_t)0;
+            bs[r][c] = (k0 + r < k && col0 + c < n) ? (int16_t)((int)b[(k0 + r) * n + col0 + c] - zb) : (int16_t)0;
+        }
+        __syncthreads();
+        int part[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) part[i][j] = 0;
+#pragma unroll 8
+        for (int l = 0; l < 64; l++) {
+            int av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) av[i] = as[ty + 16 * i][l];
+#pragma unroll
+            for (int j = 0; j < 4; j++) bv[j] = bs[l][tx + 16 * j];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) part[i][j] += av[i] * bv[j];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[i][j] += part[i][j];
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const size_t r = row0 + ty + 16 * i, c = col0 + tx + 16 * j;
+            if (r >= m || c >= n) continue;
+            const float fp = (float)acc[i][j] * scale;
+            const float q = roundf(fp / scale);
+            int v;
+            if (q != q) v = 0;                                   // Rust's float -> int cast: NaN -> 0, saturating
+            else if (q >= 2147483648.0f) v = 2147483647;
+            else if (q <= -2147483648.0f) v = -2147483647 - 1;
+            else v = (int)q;
+            out[r * n + c] = (int8_t)(v > 127 ? 127 : (v < -128 ? -128 : v));
+        }
+}
+#pragma clang fp contract(fast)
+
 // ================================================================ launchers
+
+hipError_t launch_qmatmul_i8(hipStream_t s, const int8_t *a, const int8_t *b, int8_t *out, size_t m, size_t n, size_t k, int za, int zb,
+                             float scale) {
+    dim3 grid((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64));
+    qmatmul_i8_kernel<<<grid, 256, 0, s>>>(a, b, out, m, n, k, za, zb, scale);
+    return hipGetLastError();
+}
 
 hipError_t launch_quantize_x(hipStream_t s, const float *x, uint8_t *xq, size_t K, size_t batch) {
     dim3 grid((unsigned)((K / 4 + 255) / 256), (unsigned)batch);

@@ -184,6 +184,22 @@ class HipKernelExecutor:
             raise InvalidParameters("matmul_f32: c must be a contiguous float32 array")
         _lib.check(self.lib.rt_hip_matmul_f32(self.ctx, _ptr(a), _ptr(b), _ptr(c), m, n, k), self.ctx)
 
+    # -- per-tensor affine int8 tensors: QuantizedOps::qmatmul (src/quantization/operations.rs:195-260)
+    def qmatmul_i8(self, a, scale_a: float, zero_point_a: int, b, scale_b: float, zero_point_b: int):
+        """(int8 [m, n], output scale = scale_a * scale_b, output zero point = 0)."""
+        a = np.ascontiguousarray(a); b = np.ascontiguousarray(b)
+        if a.dtype != np.int8 or b.dtype != np.int8:
+            raise InvalidParameters("qmatmul_i8: operands must be int8 arrays")
+        if a.ndim != 2 or b.ndim != 2:
+            raise InvalidParameters("qmatmul_i8: only 2D matrix multiplication is supported")      # operations.rs:218-223
+        if a.shape[1] != b.shape[0]:
+            raise ShapeMismatch("qmatmul_i8: expected %d rows in b, got %d" % (a.shape[1], b.shape[0]))
+        out = np.empty((a.shape[0], b.shape[1]), dtype=np.int8)
+        sc, zp = C.c_float(), C.c_int()
+        _lib.check(self.lib.rt_hip_qmatmul_i8(self.ctx, _ptr(a), float(scale_a), int(zero_point_a), _ptr(b), float(scale_b), int(zero_point_b),
+                                              a.shape[0], b.shape[1], a.shape[1], _ptr(out), C.byref(sc), C.byref(zp)), self.ctx)
+        return out, float(sc.value), int(zp.value)
+
     # -- quantized weights
     def upload_qweight(self, ggml_type: int, n_rows: int, n_cols: int, raw: np.ndarray | bytes) -> QWeight:
         raw = np.frombuffer(raw, dtype=np.uint8) if isinstance(raw, (bytes, bytearray, memoryview)) else np.ascontiguousarray(raw).view(np.uint8).reshape(-1)
