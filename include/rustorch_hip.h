@@ -203,7 +203,10 @@ RT_HIP_API int rt_hip_llama_destroy(rt_hip_ctx *ctx, rt_hip_llama *m);
 /* Upload one tensor's raw GGUF payload (norm vectors: F32). layer is ignored for the three global slots. */
 RT_HIP_API int rt_hip_llama_upload_tensor(rt_hip_ctx *ctx, rt_hip_llama *m, int slot, int layer, int ggml_type,
                                           size_t n_rows, size_t n_cols, const void *raw, size_t nbytes);
-/* How a decode step is issued: 1 (default) = one launch per operator group; 0 = one persistent launch per
+/* How a decode step is issued: 1 (default) = one launch per operator group; 2 = the same launches, captured
+ * into a HIP graph at the second step and replayed from then on (every argument of a step is a device
+ * pointer or a model constant, so one capture serves all later tokens; measured no faster than mode 1 on
+ * MI355X, where the cost of a launch is on the device side); 0 = one persistent launch per
  * token (one workgroup per CU, phases separated by a software grid barrier). Mode 0 is switched off in this
  * build and asking for it returns RT_HIP_ERR_UNSUPPORTED_TYPE. */
 RT_HIP_API int rt_hip_llama_set_mode(rt_hip_ctx *ctx, rt_hip_llama *m, int mode);

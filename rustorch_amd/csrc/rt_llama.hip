@@ -42,7 +42,12 @@ struct rt_hip_llama {
     int *forced_dev = nullptr, *out_tokens_dev = nullptr;
     int n_fed = 0;
     // persistent step kernel
-    int mode = 1;             // 0: persistent step kernel, 1: separate launches (default, see rt_hip_llama_set_mode)
+    int mode = 1;             // 0: persistent step kernel, 1: separate launches (default), 2: the same launches replayed from a captured graph
+    // mode 2: one graph per (want_logits, advance, use_forced); a combination runs eagerly once, is captured at its
+    // second use and replayed from then on.  Every argument of a step is a device pointer or a model constant
+    // (position and token live in `state`), so one capture serves every later token.
+    struct StepGraph { int uses = 0; hipGraph_t graph = nullptr; hipGraphExec_t exec = nullptr; };
+    StepGraph step_graphs[8];
     bool mega_ready = false;  // layer table uploaded and launch shape decided
     bool mega_ok = false;
     rt::MegaLayer *mega_layers = nullptr;
@@ -66,7 +71,17 @@ int dev_alloc(rt_hip_ctx *ctx, rt_hip_llama *m, void **p, size_t bytes) {
     return RT_HIP_OK;
 }
 
+// Captured steps name device pointers: drop them whenever a tensor or buffer they name may change.
+void drop_step_graphs(rt_hip_llama *m) {
+    for (auto &g : m->step_graphs) {
+        if (g.exec) (void)hipGraphExecDestroy(g.exec);
+        if (g.graph) (void)hipGraphDestroy(g.graph);
+        g = rt_hip_llama::StepGraph();
+    }
+}
+
 void free_all(rt_hip_llama *m) {
+    drop_step_graphs(m);
     for (void *p : m->allocs) (void)hipFree(p);
     m->allocs.clear();
 }
@@ -302,6 +317,7 @@ int rt_hip_llama_upload_tensor(rt_hip_ctx *ctx, rt_hip_llama *m, int slot, int l
     Guard g(ctx);
     m->mega_ready = false;
     void *dev = nullptr;
+    drop_step_graphs(m);      // a captured step names the old buffer of this slot
     int rc = dev_alloc(ctx, m, &dev, nbytes + 64);
     if (rc) return rc;
     RT_TRY_HIP(ctx, hipMemcpyAsync(dev, raw, nbytes, hipMemcpyHostToDevice, ctx->stream));
@@ -395,12 +411,33 @@ static int enqueue_token(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits, boo
         RT_TRY_HIP(ctx, rt::launch_llama_step(ctx->stream, a, m->mega_grid, m->mega_lds));
         return RT_HIP_OK;
     }
-    int rc = enqueue_step(ctx, m, want_logits);
-    if (rc) return rc;
-    if (want_logits) RT_TRY_HIP(ctx, rt::launch_argmax(ctx->stream, m->logits, (size_t)m->cfg.vocab, m->state + 2));
-    if (advance)
-        RT_TRY_HIP(ctx, rt::launch_step_advance(ctx->stream, m->state + 0, m->state + 1, m->state + 2, use_forced ? m->forced_dev : nullptr,
-                                                m->out_tokens_dev, m->state + 3));
+    auto enqueue = [&]() -> int {
+        int rc = enqueue_step(ctx, m, want_logits);
+        if (rc) return rc;
+        if (want_logits) RT_TRY_HIP(ctx, rt::launch_argmax(ctx->stream, m->logits, (size_t)m->cfg.vocab, m->state + 2));
+        if (advance)
+            RT_TRY_HIP(ctx, rt::launch_step_advance(ctx->stream, m->state + 0, m->state + 1, m->state + 2, use_forced ? m->forced_dev : nullptr,
+                                                    m->out_tokens_dev, m->state + 3));
+        return RT_HIP_OK;
+    };
+    if (m->mode != 2) return enqueue();
+    rt_hip_llama::StepGraph &sg = m->step_graphs[(want_logits ? 1 : 0) | (advance ? 2 : 0) | (use_forced ? 4 : 0)];
+    if (sg.exec) {
+        RT_TRY_HIP(ctx, hipGraphLaunch(sg.exec, ctx->stream));
+        return RT_HIP_OK;
+    }
+    if (sg.uses++ == 0) return enqueue();          // first use eagerly: whatever a launcher sets up lazily is set up outside a capture
+    RT_TRY_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    int rc = enqueue();
+    hipError_t e = hipStreamEndCapture(ctx->stream, &sg.graph);
+    if (rc) {
+        if (sg.graph) (void)hipGraphDestroy(sg.graph);
+        sg.graph = nullptr;
+        return rc;
+    }
+    RT_TRY_HIP(ctx, e);
+    RT_TRY_HIP(ctx, hipGraphInstantiate(&sg.exec, sg.graph, nullptr, nullptr, 0));
+    RT_TRY_HIP(ctx, hipGraphLaunch(sg.exec, ctx->stream));
     return RT_HIP_OK;
 }
 
@@ -416,12 +453,14 @@ static int check_barrier_flag(rt_hip_ctx *ctx, rt_hip_llama *m) {
 
 int rt_hip_llama_set_mode(rt_hip_ctx *ctx, rt_hip_llama *m, int mode) {
     if (!ctx || !m) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_set_mode: NULL argument");
-    RT_REQUIRE(ctx, mode == 0 || mode == 1, RT_HIP_ERR_INVALID_ARG, "mode %d (0 = persistent step kernel, 1 = separate launches)", mode);
+    RT_REQUIRE(ctx, mode >= 0 && mode <= 2, RT_HIP_ERR_INVALID_ARG,
+               "mode %d (0 = persistent step kernel, 1 = separate launches, 2 = separate launches replayed from a graph)", mode);
     // The persistent step kernel took a GPU memory fault on its first run and the cause has not been found:
     // the path stays switched off until it is, and asking for it is an error rather than a silent fallback.
-    RT_REQUIRE(ctx, mode == 1, RT_HIP_ERR_UNSUPPORTED_TYPE, "persistent step kernel is switched off in this build (unresolved GPU memory fault)");
+    RT_REQUIRE(ctx, mode != 0, RT_HIP_ERR_UNSUPPORTED_TYPE, "persistent step kernel is switched off in this build (unresolved GPU memory fault)");
     Guard g(ctx);
     m->mode = mode;
+    if (mode != 2) drop_step_graphs(m);
     return RT_HIP_OK;
 }
 

@@ -29,7 +29,7 @@ def logit_tol(wn, hidden):
 
 @pytest.mark.parametrize("mode", [
     pytest.param(0, marks=pytest.mark.skip(reason="persistent step kernel switched off: GPU memory fault on first run, cause not found")),
-    1])
+    1, 2])
 def test_small_model_teacher_forced(ex, orc, mode):
     from rustorch_amd import synth
     cfg = dict(n_layers=3, hidden=512, n_heads=4, ffn=1024, vocab=1000, max_pos=48)
@@ -61,7 +61,7 @@ def test_small_model_teacher_forced(ex, orc, mode):
 
 @pytest.mark.parametrize("mode", [
     pytest.param(0, marks=pytest.mark.skip(reason="persistent step kernel switched off: GPU memory fault on first run, cause not found")),
-    1])
+    1, 2])
 def test_decode_loop_without_host_round_trips(ex, orc, mode):
     from rustorch_amd import synth, InvalidParameters, ShapeMismatch
     cfg = dict(n_layers=2, hidden=256, n_heads=2, ffn=512, vocab=300, max_pos=32)
@@ -99,6 +99,42 @@ def test_decode_loop_without_host_round_trips(ex, orc, mode):
         gm.step(cfg["vocab"], 20)           # token outside the vocabulary
     with pytest.raises(ShapeMismatch):
         gm.decode(1, 20, 13)                # would run past max_pos
+
+
+def test_graph_replay_equals_eager_launches(ex, orc):
+    """Mode 2 replays the step from a captured graph.  Every replay is checked against the eager launches of mode 1:
+    same kernels, same arguments, so logits and picks are equal bit for bit -- with eager work (a cache reset, a
+    prefill through the other path, host reads) and synchronisations between the replays."""
+    from rustorch_amd import synth
+    cfg = dict(n_layers=2, hidden=256, n_heads=2, ffn=512, vocab=300, max_pos=40)
+    gm, om, wn = build_pair(ex, orc, 29, **cfg)
+    toks = synth.tokens(29, synth.TID_PROMPT, 30, cfg["vocab"])
+    forced = synth.tokens(29, 77, 10, cfg["vocab"])
+
+    def run(mode):
+        gm.set_mode(mode)
+        gm.reset()
+        logits, picks = [], []
+        for p, t in enumerate(toks[:14]):            # 14 steps: eager first, captured at the second, replayed 12 times
+            picks.append(gm.step(int(t), p))
+            logits.append(gm.logits().copy())        # a host read and a synchronisation between the replays
+        out_a = gm.decode(int(toks[14]), 14, 8)      # the advancing form of the step: its own capture
+        logits.append(gm.logits().copy())
+        gm.reset()
+        gm.prefill(toks[:20], 0)                     # 20 tokens: the batched path, eager kernels between the replays
+        out_b = gm.decode(int(toks[20]), 20, 10, forced)
+        logits.append(gm.logits().copy())
+        return logits, picks, out_a, out_b
+
+    l1, p1, a1, b1 = run(1)
+    l2, p2, a2, b2 = run(2)
+    l3, p3, a3, b3 = run(2)                          # graphs of the earlier run are still there: replays only
+    for other in ((l2, p2, a2, b2), (l3, p3, a3, b3)):
+        assert p1 == other[1] and list(a1) == list(other[2]) and list(b1) == list(other[3])
+        for x, y in zip(l1, other[0]):
+            assert np.array_equal(x, y)
+    want = om.forward(toks[:14], 0)
+    assert np.all(np.abs(l2[13] - want[13]) <= logit_tol(wn, cfg["hidden"]))
 
 
 def test_incomplete_model_is_an_error(ex):
