@@ -181,6 +181,7 @@ RT_HIP_API int rt_hip_argmax_dev(rt_hip_ctx *ctx, const float *v, size_t n, int 
 typedef struct {
     int n_layers, hidden, n_heads, ffn, vocab, max_pos;
     float rms_eps, rope_theta;
+    int n_kv_heads;   /* key / value heads (grouped-query attention); 0 means n_heads */
 } rt_hip_llama_config;
 
 typedef enum {

@@ -47,6 +47,8 @@ def load() -> C.CDLL:
         "orc_rope": (None, [vp, i, i, i, vp]),
         "orc_kv_append": (None, [vp, vp, sz, sz]),
         "orc_attn_decode": (None, [vp, vp, vp, i, i, i, vp]),
+        "orc_attn_decode_gqa": (None, [vp, vp, vp, i, i, i, i, vp]),
+        "orc_llama_set_kv_heads": (i, [vp, i]),
         "orc_argmax": (i, [vp, sz]),
         "orc_add": (None, [vp, vp, sz]),
         "orc_llama_create": (vp, [i, i, i, i, i, i, f, f, i]),
@@ -166,11 +168,13 @@ def kv_append(cache_u16: np.ndarray, v: np.ndarray, pos: int) -> None:
     load().orc_kv_append(_p(cache_u16), _p(v), pos, v.size)
 
 
-def attn_decode(q: np.ndarray, kc_u16: np.ndarray, vc_u16: np.ndarray, n_pos: int, n_heads: int, head_dim: int) -> np.ndarray:
+def attn_decode(q: np.ndarray, kc_u16: np.ndarray, vc_u16: np.ndarray, n_pos: int, n_heads: int, head_dim: int,
+                n_kv_heads: int = 0) -> np.ndarray:
+    """n_kv_heads (0 = n_heads): cache rows hold that many heads; query head h reads head h // (n_heads // n_kv_heads)."""
     q = np.ascontiguousarray(q, dtype=np.float32)
     kc_u16 = np.ascontiguousarray(kc_u16); vc_u16 = np.ascontiguousarray(vc_u16)
     out = np.empty(n_heads * head_dim, dtype=np.float32)
-    load().orc_attn_decode(_p(q), _p(kc_u16), _p(vc_u16), n_pos, n_heads, head_dim, _p(out))
+    load().orc_attn_decode_gqa(_p(q), _p(kc_u16), _p(vc_u16), n_pos, n_heads, n_kv_heads or n_heads, head_dim, _p(out))
     return out
 
 
@@ -186,10 +190,12 @@ SLOT = {"token_embd": 0, "output": 1, "output_norm": 2, "attn_q": 10, "attn_k": 
 class OracleLlama:
     """CPU decode loop over borrowed raw tensors (keeps references so the buffers outlive the model)."""
 
-    def __init__(self, n_layers, hidden, n_heads, ffn, vocab, max_pos, eps=1e-5, theta=10000.0, nthreads=0):
+    def __init__(self, n_layers, hidden, n_heads, ffn, vocab, max_pos, eps=1e-5, theta=10000.0, nthreads=0, n_kv_heads=0):
         self.vocab = vocab
         self.keep = []
         self.h = C.c_void_p(load().orc_llama_create(n_layers, hidden, n_heads, ffn, vocab, max_pos, eps, theta, nthreads or num_threads()))
+        if n_kv_heads and load().orc_llama_set_kv_heads(self.h, n_kv_heads) != 0:
+            raise ValueError("oracle: n_kv_heads must divide n_heads")
 
     def set_tensor(self, slot, layer, ggml_type, n_rows, n_cols, raw):
         raw = np.ascontiguousarray(raw)

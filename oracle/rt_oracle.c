@@ -446,20 +446,24 @@ ORC_API void orc_kv_append(uint16_t *cache, const float *v, size_t pos, size_t r
 
 /*
  * One query against positions 0..n_pos-1 of an fp16 cache laid out
- * [pos][head][dim] (attention.rs:233-338 restricted to one query row, which
- * makes the attention causal by construction).
+ * [pos][kv head][dim] (attention.rs:233-338 restricted to one query row, which
+ * makes the attention causal by construction).  Grouped-query form: query head h
+ * reads key / value head h / (n_heads / n_kv_heads); the reference has one head
+ * count, which is n_kv_heads == n_heads here.
  */
-ORC_API void orc_attn_decode(const float *q, const uint16_t *kc, const uint16_t *vc, int n_pos, int n_heads,
-                             int head_dim, float *out) {
+ORC_API void orc_attn_decode_gqa(const float *q, const uint16_t *kc, const uint16_t *vc, int n_pos, int n_heads, int n_kv_heads,
+                                 int head_dim, float *out) {
     float scale = 1.0f / sqrtf((float)head_dim);
-    size_t row = (size_t)n_heads * head_dim;
+    size_t row = (size_t)n_kv_heads * head_dim;
+    int group = n_heads / n_kv_heads;
 #pragma omp parallel for schedule(static)
     for (int h = 0; h < n_heads; h++) {
         float *sc = (float *)malloc((size_t)n_pos * sizeof(float));
         const float *qh = q + (size_t)h * head_dim;
+        size_t kvo = (size_t)(h / group) * head_dim;
         float mx = -INFINITY;
         for (int j = 0; j < n_pos; j++) {
-            const uint16_t *kr = kc + (size_t)j * row + (size_t)h * head_dim;
+            const uint16_t *kr = kc + (size_t)j * row + kvo;
             float s = 0.0f;
             for (int d = 0; d < head_dim; d++) s = s + qh[d] * orc_h2f(kr[d]);
             s = s * scale;
@@ -471,11 +475,16 @@ ORC_API void orc_attn_decode(const float *q, const uint16_t *kc, const uint16_t 
         for (int j = 0; j < n_pos; j++) sc[j] = sc[j] / sum;
         for (int d = 0; d < head_dim; d++) {
             float v = 0.0f;
-            for (int j = 0; j < n_pos; j++) v = v + sc[j] * orc_h2f(vc[(size_t)j * row + (size_t)h * head_dim + d]);
+            for (int j = 0; j < n_pos; j++) v = v + sc[j] * orc_h2f(vc[(size_t)j * row + kvo + d]);
             out[(size_t)h * head_dim + d] = v;
         }
         free(sc);
     }
+}
+
+ORC_API void orc_attn_decode(const float *q, const uint16_t *kc, const uint16_t *vc, int n_pos, int n_heads,
+                             int head_dim, float *out) {
+    orc_attn_decode_gqa(q, kc, vc, n_pos, n_heads, n_heads, head_dim, out);
 }
 
 /* Greedy pick; ties go to the lowest index. */
@@ -496,7 +505,7 @@ typedef struct {
 } orc_tensor;
 
 typedef struct {
-    int n_layers, hidden, n_heads, head_dim, ffn, vocab, max_pos;
+    int n_layers, hidden, n_heads, n_kv_heads, head_dim, ffn, vocab, max_pos;
     float eps, theta;
     orc_tensor tok_embd, output;
     const float *out_norm;
@@ -510,7 +519,7 @@ typedef struct {
 ORC_API orc_llama *orc_llama_create(int n_layers, int hidden, int n_heads, int ffn, int vocab, int max_pos, float eps,
                                     float theta, int nthreads) {
     orc_llama *m = (orc_llama *)calloc(1, sizeof(orc_llama));
-    m->n_layers = n_layers; m->hidden = hidden; m->n_heads = n_heads; m->head_dim = hidden / n_heads;
+    m->n_layers = n_layers; m->hidden = hidden; m->n_heads = n_heads; m->n_kv_heads = n_heads; m->head_dim = hidden / n_heads;
     m->ffn = ffn; m->vocab = vocab; m->max_pos = max_pos; m->eps = eps; m->theta = theta; m->nthreads = nthreads;
     size_t L = (size_t)n_layers;
     m->wq = calloc(L, sizeof(orc_tensor)); m->wk = calloc(L, sizeof(orc_tensor)); m->wv = calloc(L, sizeof(orc_tensor));
@@ -522,6 +531,13 @@ ORC_API orc_llama *orc_llama_create(int n_layers, int hidden, int n_heads, int f
     m->inv_freq = malloc(sizeof(float) * (size_t)(m->head_dim / 2));
     orc_rope_inv_freq(m->head_dim, theta, m->inv_freq);
     return m;
+}
+
+/* Grouped-query attention: n_kv_heads key / value heads (wk, wv have n_kv_heads * head_dim rows).  Before the first forward. */
+ORC_API int orc_llama_set_kv_heads(orc_llama *m, int n_kv_heads) {
+    if (n_kv_heads <= 0 || m->n_heads % n_kv_heads != 0) return -1;
+    m->n_kv_heads = n_kv_heads;
+    return 0;
 }
 
 ORC_API void orc_llama_destroy(orc_llama *m) {
@@ -573,6 +589,7 @@ ORC_API int orc_llama_forward(orc_llama *m, const int *tokens, int n_tok, int po
         if (tokens[t] < 0 || tokens[t] >= m->vocab) return -2;
         deq_row(m->tok_embd.type, (const uint8_t *)m->tok_embd.raw + erb * (size_t)tokens[t], H, x + H * t);
     }
+    const size_t KD = (size_t)m->n_kv_heads * (size_t)m->head_dim;       /* width of k, v and of a cache row */
     for (int l = 0; l < m->n_layers; l++) {
         uint16_t *kc = m->kcache + (size_t)l * (size_t)m->max_pos * H;
         uint16_t *vc = m->vcache + (size_t)l * (size_t)m->max_pos * H;
@@ -581,12 +598,12 @@ ORC_API int orc_llama_forward(orc_llama *m, const int *tokens, int n_tok, int po
         for (size_t t = 0; t < T; t++) {
             int pos = pos0 + (int)t;
             orc_rope(q + H * t, m->n_heads, m->head_dim, pos, m->inv_freq);
-            orc_rope(k + H * t, m->n_heads, m->head_dim, pos, m->inv_freq);
-            orc_kv_append(kc, k + H * t, (size_t)pos, H);
-            orc_kv_append(vc, v + H * t, (size_t)pos, H);
+            orc_rope(k + KD * t, m->n_kv_heads, m->head_dim, pos, m->inv_freq);
+            orc_kv_append(kc, k + KD * t, (size_t)pos, KD);
+            orc_kv_append(vc, v + KD * t, (size_t)pos, KD);
         }
         for (size_t t = 0; t < T; t++)
-            orc_attn_decode(q + H * t, kc, vc, pos0 + (int)t + 1, m->n_heads, m->head_dim, a + H * t);
+            orc_attn_decode_gqa(q + H * t, kc, vc, pos0 + (int)t + 1, m->n_heads, m->n_kv_heads, m->head_dim, a + H * t);
         lin(m, &m->wo[l], a, T, o);
         orc_add(x, o, T * H);
         orc_rmsnorm(x, m->ffn_norm[l], H, m->eps, T, h);

@@ -23,7 +23,8 @@ class DevInfo(C.Structure):
 
 class LlamaConfig(C.Structure):
     _fields_ = [("n_layers", C.c_int), ("hidden", C.c_int), ("n_heads", C.c_int), ("ffn", C.c_int),
-                ("vocab", C.c_int), ("max_pos", C.c_int), ("rms_eps", C.c_float), ("rope_theta", C.c_float)]
+                ("vocab", C.c_int), ("max_pos", C.c_int), ("rms_eps", C.c_float), ("rope_theta", C.c_float),
+                ("n_kv_heads", C.c_int)]
 
 
 # name -> (restype, argtypes); the keys are exactly the RT_HIP_API symbols of the header

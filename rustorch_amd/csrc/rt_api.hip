@@ -540,7 +540,7 @@ int rt_hip_attn_decode_dev(rt_hip_ctx *ctx, const float *q, const uint16_t *kcac
     RT_REQUIRE(ctx, n_heads > 0 && n_pos > 0 && n_pos <= 16000, RT_HIP_ERR_SHAPE, "attn_decode: n_heads=%d n_pos=%d", n_heads, n_pos);
     Guard g(ctx);
     RT_TRY_HIP(ctx, rt::launch_attn_decode(ctx->stream, const_cast<float *>(q), nullptr, nullptr, const_cast<uint16_t *>(kcache),
-                                           const_cast<uint16_t *>(vcache), nullptr, n_pos, n_heads, head_dim, nullptr, out, nullptr, false));
+                                           const_cast<uint16_t *>(vcache), nullptr, n_pos, n_heads, n_heads, head_dim, nullptr, out, nullptr, false));
     return RT_HIP_OK;
 }
 

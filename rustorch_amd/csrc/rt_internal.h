@@ -127,12 +127,12 @@ hipError_t launch_rope_kv(hipStream_t s, float *q, const float *k, const float *
                           const float *inv_freq_dev);
 // fused = rotate q / k of the step, append k / v at *pos_dev, then attend over [0, *pos_dev]; otherwise attend over [0, n_pos)
 hipError_t launch_attn_decode(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
-                              const int *pos_dev, int n_pos, int n_heads, int head_dim, const float *inv_freq_dev,
+                              const int *pos_dev, int n_pos, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev,
                               float *out, uint8_t *xq, bool fused);
 hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache,
-                                int pos0, size_t n_tok, int n_heads, int head_dim, const float *inv_freq_dev);
+                                int pos0, size_t n_tok, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev);
 hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
-                             const int *pos_dev, int n_pos, size_t n_queries, int n_heads, int head_dim,
+                             const int *pos_dev, int n_pos, size_t n_queries, int n_heads, int n_kv_heads, int head_dim,
                              const float *inv_freq_dev, float *out, uint8_t *xq, bool fused);
 hipError_t launch_embed_rows(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,
                              const int *tokens_dev, size_t n_tok, int vocab, float *out);

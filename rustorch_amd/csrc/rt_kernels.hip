@@ -169,27 +169,30 @@ __global__ void rope_kv_kernel(float *q, const float *k, const float *v, uint16_
 // Prefill form: blockIdx.y = token m of the batch at position pos0 + m; q [M][row] is rotated in place,
 // rotated k and v go to the fp16 cache rows pos0 + m.
 __global__ void rope_kv_batch_kernel(float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache,
-                                     int pos0, int n_heads, int head_dim, const float *inv_freq) {
+                                     int pos0, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq) {
     int half = head_dim / 2;
     int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n_heads * half) return;
     int i = t % half;
-    const size_t row = (size_t)n_heads * head_dim, m = blockIdx.y;
+    const size_t row = (size_t)n_heads * head_dim, rowkv = (size_t)n_kv_heads * head_dim, m = blockIdx.y;
     const int p = pos0 + (int)m;
     float s, c;
     sincosf((float)p * inv_freq[i], &s, &c);
     float2 *qr = reinterpret_cast<float2 *>(q + m * row);
     float2 qv = qr[t];
     qr[t] = make_float2(qv.x * c - qv.y * s, qv.x * s + qv.y * c);
-    float2 kv = reinterpret_cast<const float2 *>(k + m * row)[t];
+    if (t >= n_kv_heads * half) return;          // fewer key / value heads than query heads
+    float2 kv = reinterpret_cast<const float2 *>(k + m * rowkv)[t];
     float k0 = kv.x * c - kv.y * s, k1 = kv.x * s + kv.y * c;
-    float2 vv = reinterpret_cast<const float2 *>(v + m * row)[t];
-    reinterpret_cast<uint32_t *>(kcache + (size_t)p * row)[t] = (uint32_t)f2h_rne(k0) | ((uint32_t)f2h_rne(k1) << 16);
-    reinterpret_cast<uint32_t *>(vcache + (size_t)p * row)[t] = (uint32_t)f2h_rne(vv.x) | ((uint32_t)f2h_rne(vv.y) << 16);
+    float2 vv = reinterpret_cast<const float2 *>(v + m * rowkv)[t];
+    reinterpret_cast<uint32_t *>(kcache + (size_t)p * rowkv)[t] = (uint32_t)f2h_rne(k0) | ((uint32_t)f2h_rne(k1) << 16);
+    reinterpret_cast<uint32_t *>(vcache + (size_t)p * rowkv)[t] = (uint32_t)f2h_rne(vv.x) | ((uint32_t)f2h_rne(vv.y) << 16);
 }
 
 // -------------------------------------------------------- decode attention
-// One block (256 threads) per head; cache layout [pos][head][dim], fp16.
+// One block (256 threads) per query head; cache layout [pos][kv head][dim], fp16.  With fewer key / value heads
+// than query heads, query head h reads kv head h / (n_heads / n_kv_heads) and the first query head of each
+// group is the one that appends the new row.
 //   scores_j = (q . k_j) / sqrt(dim);  p = softmax(scores) with max subtraction;  out = sum_j p_j v_j
 // (example-cli/src/model/architectures/attention.rs:233-338 for one query row).
 // FUSED: the block first rotates its head's q and k (interleaved pairs, angle pos * inv_freq[i]), stores
@@ -212,7 +215,7 @@ __device__ __forceinline__ void unpack8(uint4 v, float *f) {
 // while they are in flight: one memory round trip instead of three dependent ones.
 template <int HD, bool FUSED>
 __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float *k, const float *v, uint16_t *kc,
-                                                          uint16_t *vc, const int *pos_dev, int n_pos_arg, int n_heads,
+                                                          uint16_t *vc, const int *pos_dev, int n_pos_arg, int n_heads, int n_kv_heads,
                                                           const float *inv_freq, float *out, uint8_t *xq) {
     RT_DYN_LDS(float, sc);
     __shared__ float red[4];
@@ -224,7 +227,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
     constexpr int NG = 256 / CH;        // position groups in the value phase
     constexpr int kVPre = 16;           // value chunks a thread requests ahead (covers NG * kVPre positions)
     const int h = blockIdx.x, tid = threadIdx.x;
-    const size_t row = (size_t)n_heads * HD;
+    const size_t row = (size_t)n_heads * HD, rowkv = (size_t)n_kv_heads * HD;
+    const int group = n_heads / n_kv_heads, kvh = h / group;
+    const bool appends = h % group == 0;
     const int cur = FUSED ? *pos_dev : -1;
     // not fused: blockIdx.y = query m of a causal batch; query m sees n_pos_arg + m positions
     const int n_pos = FUSED ? cur + 1 : n_pos_arg + (int)blockIdx.y;
@@ -239,14 +244,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
     uint4 kreg[CH], vreg[kVPre];
     const bool k_pre = tid < n_pos && tid != cur;
     if (k_pre) {
-        const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)tid * row + (size_t)h * HD);
+        const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)tid * rowkv + (size_t)kvh * HD);
 #pragma unroll
         for (int i = 0; i < CH; i++) kreg[i] = kr[i];
     }
 #pragma unroll
     for (int i = 0; i < kVPre; i++) {
         const int j = g + NG * i;
-        if (j < n_pos && j != cur) vreg[i] = reinterpret_cast<const uint4 *>(vc + (size_t)j * row + (size_t)h * HD)[c];
+        if (j < n_pos && j != cur) vreg[i] = reinterpret_cast<const uint4 *>(vc + (size_t)j * rowkv + (size_t)kvh * HD)[c];
     }
 
     if (FUSED) {
@@ -255,7 +260,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
             float sn, cs;
             sincosf((float)cur * inv_freq[i], &sn, &cs);
             float2 qv = reinterpret_cast<const float2 *>(q + (size_t)h * HD)[i];
-            float2 kv = reinterpret_cast<const float2 *>(k + (size_t)h * HD)[i];
+            float2 kv = reinterpret_cast<const float2 *>(k + (size_t)kvh * HD)[i];
             float q0 = qv.x * cs - qv.y * sn, q1 = qv.x * sn + qv.y * cs;
             float k0 = kv.x * cs - kv.y * sn, k1 = kv.x * sn + kv.y * cs;
             qs[2 * i] = q0;
@@ -264,14 +269,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
             uint16_t a = f2h_rne(k0), b = f2h_rne(k1);
             kcur[2 * i] = h2f(a);
             kcur[2 * i + 1] = h2f(b);
-            reinterpret_cast<uint32_t *>(kc + (size_t)cur * row + (size_t)h * HD)[i] = (uint32_t)a | ((uint32_t)b << 16);
+            if (appends) reinterpret_cast<uint32_t *>(kc + (size_t)cur * rowkv + (size_t)kvh * HD)[i] = (uint32_t)a | ((uint32_t)b << 16);
         } else if (tid < HD) {
             int i = tid - HD / 2;
-            float2 vv = reinterpret_cast<const float2 *>(v + (size_t)h * HD)[i];
+            float2 vv = reinterpret_cast<const float2 *>(v + (size_t)kvh * HD)[i];
             uint16_t a = f2h_rne(vv.x), b = f2h_rne(vv.y);
             vcur[2 * i] = h2f(a);
             vcur[2 * i + 1] = h2f(b);
-            reinterpret_cast<uint32_t *>(vc + (size_t)cur * row + (size_t)h * HD)[i] = (uint32_t)a | ((uint32_t)b << 16);
+            if (appends) reinterpret_cast<uint32_t *>(vc + (size_t)cur * rowkv + (size_t)kvh * HD)[i] = (uint32_t)a | ((uint32_t)b << 16);
         }
     } else if (tid < HD) {
         qs[tid] = q[(size_t)h * HD + tid];
@@ -285,7 +290,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
 #pragma unroll 8
             for (int d = 0; d < HD; d++) s += qs[d] * kcur[d];
         } else {
-            const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)j * row + (size_t)h * HD);
+            const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)j * rowkv + (size_t)kvh * HD);
 #pragma unroll
             for (int cc = 0; cc < CH; cc++) {
                 float f[8];
@@ -334,7 +339,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
 #pragma unroll
             for (int e = 0; e < 8; e++) f[e] = vcur[8 * c + e];
         } else {
-            unpack8(reinterpret_cast<const uint4 *>(vc + (size_t)j * row + (size_t)h * HD)[c], f);
+            unpack8(reinterpret_cast<const uint4 *>(vc + (size_t)j * rowkv + (size_t)kvh * HD)[c], f);
         }
         float p = sc[j];
 #pragma unroll
@@ -569,34 +574,36 @@ hipError_t launch_rope_kv(hipStream_t s, float *q, const float *k, const float *
 }
 
 hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache,
-                                int pos0, size_t n_tok, int n_heads, int head_dim, const float *inv_freq_dev) {
+                                int pos0, size_t n_tok, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads != 0) return hipErrorInvalidValue;
     int pairs = n_heads * head_dim / 2;
     rope_kv_batch_kernel<<<dim3((unsigned)((pairs + 255) / 256), (unsigned)n_tok), 256, 0, s>>>(q, k, v, kcache, vcache, pos0, n_heads,
-                                                                                                head_dim, inv_freq_dev);
+                                                                                                n_kv_heads, head_dim, inv_freq_dev);
     return hipGetLastError();
 }
 
 hipError_t launch_attn_decode(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
-                              const int *pos_dev, int n_pos, int n_heads, int head_dim, const float *inv_freq_dev,
+                              const int *pos_dev, int n_pos, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev,
                               float *out, uint8_t *xq, bool fused) {
-    return launch_attn_batch(s, q, k, v, kc, vc, pos_dev, n_pos, 1, n_heads, head_dim, inv_freq_dev, out, xq, fused);
+    return launch_attn_batch(s, q, k, v, kc, vc, pos_dev, n_pos, 1, n_heads, n_kv_heads, head_dim, inv_freq_dev, out, xq, fused);
 }
 
 // n_queries > 1 (not fused, xq == NULL): query m of q [n_queries][row] attends over the first n_pos + m cache rows
 hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
-                             const int *pos_dev, int n_pos, size_t n_queries, int n_heads, int head_dim,
+                             const int *pos_dev, int n_pos, size_t n_queries, int n_heads, int n_kv_heads, int head_dim,
                              const float *inv_freq_dev, float *out, uint8_t *xq, bool fused) {
     if (n_queries > 1 && (fused || xq)) return hipErrorInvalidValue;
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads != 0) return hipErrorInvalidValue;
     size_t lds = ((size_t)n_pos + n_queries - 1) * sizeof(float);  // fused: n_pos is the upper bound (max_pos)
     dim3 grid((unsigned)n_heads, (unsigned)n_queries);
     if (head_dim == 128 && fused)
-        attn_decode_kernel<128, true><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, inv_freq_dev, out, xq);
+        attn_decode_kernel<128, true><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, n_kv_heads, inv_freq_dev, out, xq);
     else if (head_dim == 128)
-        attn_decode_kernel<128, false><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, inv_freq_dev, out, xq);
+        attn_decode_kernel<128, false><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, n_kv_heads, inv_freq_dev, out, xq);
     else if (head_dim == 64 && fused)
-        attn_decode_kernel<64, true><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, inv_freq_dev, out, xq);
+        attn_decode_kernel<64, true><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, n_kv_heads, inv_freq_dev, out, xq);
     else if (head_dim == 64)
-        attn_decode_kernel<64, false><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, inv_freq_dev, out, xq);
+        attn_decode_kernel<64, false><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, n_kv_heads, inv_freq_dev, out, xq);
     else
         return hipErrorInvalidValue;
     return hipGetLastError();

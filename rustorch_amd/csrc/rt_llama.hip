@@ -30,6 +30,8 @@ struct rt_hip_llama {
     };
     rt_hip_llama_config cfg{};
     int head_dim = 0;
+    int n_kv = 0;             // key / value heads; kv_dim = n_kv * head_dim is the width of k, v and of a cache row
+    size_t kv_dim = 0;
     T tok_embd, output;
     float *out_norm = nullptr;
     std::vector<T> wq, wk, wv, wo, wgate, wup, wdown;
@@ -118,8 +120,8 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
     int *pos_dev = m->state, *tok_dev = m->state + 1;
     RT_TRY_HIP(ctx, rt::launch_embed_row(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, tok_dev, c.vocab, m->x));
     for (int l = 0; l < c.n_layers; l++) {
-        uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * H;
-        uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * H;
+        uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
+        uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
         rt::GemvArgs a;
         memset(&a, 0, sizeof a);
         a.n = 3;
@@ -128,7 +130,7 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
         a.p[2] = make_prob(m->wv[l], m->x, rt::kStageRms, m->v, nullptr);
         for (int i = 0; i < 3; i++) { a.p[i].gamma = m->attn_norm[l]; a.p[i].eps = c.rms_eps; }
         RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
-        RT_TRY_HIP(ctx, rt::launch_attn_decode(s, m->q, m->k, m->v, kc, vc, pos_dev, c.max_pos, c.n_heads, m->head_dim, m->inv_freq,
+        RT_TRY_HIP(ctx, rt::launch_attn_decode(s, m->q, m->k, m->v, kc, vc, pos_dev, c.max_pos, c.n_heads, m->n_kv, m->head_dim, m->inv_freq,
                                                nullptr, m->xq_a, true));
         memset(&a, 0, sizeof a);
         a.n = 1;
@@ -206,14 +208,14 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
     float *x = m->pf_x, *x2 = m->pf_x2;
     RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, m->pf_tok, M, c.vocab, x));
     for (int l = 0; l < c.n_layers; l++) {
-        uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * H;
-        uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * H;
+        uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
+        uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->attn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
         if ((rc = gemm(ctx, m->wq[l], m->pf_n, M, m->pf_q, nullptr))) return rc;
         if ((rc = gemm(ctx, m->wk[l], m->pf_n, M, m->pf_k, nullptr, true))) return rc;
         if ((rc = gemm(ctx, m->wv[l], m->pf_n, M, m->pf_v, nullptr, true))) return rc;
-        RT_TRY_HIP(ctx, rt::launch_rope_kv_batch(s, m->pf_q, m->pf_k, m->pf_v, kc, vc, pos0, M, c.n_heads, m->head_dim, m->inv_freq));
-        RT_TRY_HIP(ctx, rt::launch_attn_batch(s, m->pf_q, nullptr, nullptr, kc, vc, nullptr, pos0 + 1, M, c.n_heads, m->head_dim,
+        RT_TRY_HIP(ctx, rt::launch_rope_kv_batch(s, m->pf_q, m->pf_k, m->pf_v, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
+        RT_TRY_HIP(ctx, rt::launch_attn_batch(s, m->pf_q, nullptr, nullptr, kc, vc, nullptr, pos0 + 1, M, c.n_heads, m->n_kv, m->head_dim,
                                               m->inv_freq, m->pf_a, nullptr, false));
         if ((rc = gemm(ctx, m->wo[l], m->pf_a, M, x2, x))) return rc;
         std::swap(x, x2);
@@ -240,6 +242,8 @@ int rt_hip_llama_create(rt_hip_ctx *ctx, const rt_hip_llama_config *cfg, rt_hip_
     RT_REQUIRE(ctx, cfg->hidden % cfg->n_heads == 0, RT_HIP_ERR_SHAPE, "hidden=%d not divisible by n_heads=%d", cfg->hidden, cfg->n_heads);
     int hd = cfg->hidden / cfg->n_heads;
     RT_REQUIRE(ctx, hd == 64 || hd == 128, RT_HIP_ERR_SHAPE, "head_dim=%d (64 or 128 supported)", hd);
+    const int n_kv = cfg->n_kv_heads == 0 ? cfg->n_heads : cfg->n_kv_heads;
+    RT_REQUIRE(ctx, n_kv > 0 && cfg->n_heads % n_kv == 0, RT_HIP_ERR_SHAPE, "n_kv_heads=%d does not divide n_heads=%d", cfg->n_kv_heads, cfg->n_heads);
     RT_REQUIRE(ctx, cfg->hidden % 256 == 0 && cfg->ffn % 256 == 0, RT_HIP_ERR_SHAPE, "hidden=%d and ffn=%d must be multiples of 256", cfg->hidden, cfg->ffn);
     RT_REQUIRE(ctx, cfg->max_pos <= 16000, RT_HIP_ERR_SHAPE, "max_pos=%d exceeds 16000", cfg->max_pos);
     RT_REQUIRE(ctx, rt::xq_stride((size_t)cfg->ffn) <= 64 * 1024 && rt::xq_stride((size_t)cfg->hidden) <= 64 * 1024, RT_HIP_ERR_SHAPE,
@@ -250,13 +254,16 @@ int rt_hip_llama_create(rt_hip_ctx *ctx, const rt_hip_llama_config *cfg, rt_hip_
     rt_hip_llama *m = new (std::nothrow) rt_hip_llama();
     if (!m) return fail(ctx, RT_HIP_ERR_OOM, "host allocation failed");
     m->cfg = *cfg;
+    m->cfg.n_kv_heads = n_kv;
     m->head_dim = hd;
+    m->n_kv = n_kv;
+    m->kv_dim = (size_t)n_kv * (size_t)hd;
     size_t L = (size_t)cfg->n_layers, H = (size_t)cfg->hidden, F = (size_t)cfg->ffn, V = (size_t)cfg->vocab, P = (size_t)cfg->max_pos;
     m->wq.resize(L); m->wk.resize(L); m->wv.resize(L); m->wo.resize(L); m->wgate.resize(L); m->wup.resize(L); m->wdown.resize(L);
     m->attn_norm.assign(L, nullptr); m->ffn_norm.assign(L, nullptr);
     int rc = RT_HIP_OK;
     auto A = [&](void **p, size_t b) { if (rc == RT_HIP_OK) rc = dev_alloc(ctx, m, p, b); };
-    A((void **)&m->kcache, L * P * H * 2); A((void **)&m->vcache, L * P * H * 2);
+    A((void **)&m->kcache, L * P * m->kv_dim * 2); A((void **)&m->vcache, L * P * m->kv_dim * 2);
     A((void **)&m->x, H * 4); A((void **)&m->q, H * 4); A((void **)&m->k, H * 4); A((void **)&m->v, H * 4);
     A((void **)&m->g, F * 4); A((void **)&m->u, F * 4); A((void **)&m->logits, V * 4);
     A((void **)&m->xq_h, rt::xq_stride(H)); A((void **)&m->xq_a, rt::xq_stride(H)); A((void **)&m->xq_f, rt::xq_stride(F));
@@ -295,7 +302,8 @@ int rt_hip_llama_upload_tensor(rt_hip_ctx *ctx, rt_hip_llama *m, int slot, int l
     size_t er = 0, ec = 0;
     switch (slot) {
     case RT_LLAMA_TOK_EMBD: case RT_LLAMA_OUTPUT: er = V; ec = H; break;
-    case RT_LLAMA_ATTN_Q: case RT_LLAMA_ATTN_K: case RT_LLAMA_ATTN_V: case RT_LLAMA_ATTN_OUT: er = H; ec = H; break;
+    case RT_LLAMA_ATTN_Q: case RT_LLAMA_ATTN_OUT: er = H; ec = H; break;
+    case RT_LLAMA_ATTN_K: case RT_LLAMA_ATTN_V: er = m->kv_dim; ec = H; break;
     case RT_LLAMA_FFN_GATE: case RT_LLAMA_FFN_UP: er = F; ec = H; break;
     case RT_LLAMA_FFN_DOWN: er = H; ec = F; break;
     case RT_LLAMA_OUTPUT_NORM: case RT_LLAMA_ATTN_NORM: case RT_LLAMA_FFN_NORM: er = 1; ec = H; break;
@@ -363,6 +371,7 @@ static int ensure_mega(rt_hip_ctx *ctx, rt_hip_llama *m) {
     bool same = true;
     for (int l = 0; l < c.n_layers; l++) same = same && m->wgate[l].type == m->wup[l].type;
     m->mega_lds = rt::mega_lds_bytes(c.hidden, c.ffn, m->head_dim, c.max_pos);
+    same = same && m->n_kv == c.n_heads;      // the step kernel knows one head count
     m->mega_grid = same ? rt::mega_grid(ctx->device, m->mega_lds) : 0;
     if (m->mega_grid >= 8 && m->mega_grid >= c.n_heads) {
         std::vector<rt::MegaLayer> tab((size_t)c.n_layers);

@@ -18,9 +18,11 @@ SLOT = {"token_embd": 0, "output": 1, "output_norm": 2, "attn_q": 10, "attn_k": 
 
 class HipLlama:
     def __init__(self, ex: HipKernelExecutor, n_layers: int, hidden: int, n_heads: int, ffn: int, vocab: int,
-                 max_pos: int, rms_eps: float = 1e-5, rope_theta: float = 10000.0):
+                 max_pos: int, rms_eps: float = 1e-5, rope_theta: float = 10000.0, n_kv_heads: int = 0):
+        """n_kv_heads: key / value heads of grouped-query attention (0 = n_heads)."""
         self.ex = ex
-        self.cfg = _lib.LlamaConfig(n_layers, hidden, n_heads, ffn, vocab, max_pos, rms_eps, rope_theta)
+        self.cfg = _lib.LlamaConfig(n_layers, hidden, n_heads, ffn, vocab, max_pos, rms_eps, rope_theta, n_kv_heads)
+        self.kv_dim = (n_kv_heads or n_heads) * (hidden // n_heads)
         self.h = C.c_void_p()
         _lib.check(ex.lib.rt_hip_llama_create(ex.ctx, C.byref(self.cfg), C.byref(self.h)), ex.ctx)
 
@@ -30,7 +32,8 @@ class HipLlama:
                                                           n_cols, C.c_void_p(raw.ctypes.data), raw.nbytes), self.ex.ctx)
 
     def set_mode(self, mode: int) -> None:
-        """1 = one launch per operator group (default); 0 = one persistent launch per token (switched off in this build)."""
+        """1 = one launch per operator group (default); 2 = the same launches replayed from a captured graph;
+        0 = one persistent launch per token (switched off in this build)."""
         _lib.check(self.ex.lib.rt_hip_llama_set_mode(self.ex.ctx, self.h, mode), self.ex.ctx)
 
     def reset(self) -> None:
@@ -73,14 +76,14 @@ class HipLlama:
             pass
 
 
-def synthetic_tensors(seed: int, n_layers: int, hidden: int, ffn: int, vocab: int):
+def synthetic_tensors(seed: int, n_layers: int, hidden: int, ffn: int, vocab: int, kv_dim: int | None = None):
     """Yield (slot, layer, ggml type, n_rows, n_cols, raw) of a random-init Llama: token embedding Q8_0,
     q/k/o/gate/up Q4_K, v/down and the output head Q6_K, RMSNorm weights f32 ~ 1 + N(0, 0.01)."""
     yield ("token_embd", -1, GGMLType.Q8_0, vocab, hidden, synth.blocks(GGMLType.Q8_0, seed, synth.TID_TOK_EMBD, vocab, hidden))
     yield ("output", -1, GGMLType.Q6_K, vocab, hidden, synth.blocks(GGMLType.Q6_K, seed, synth.TID_OUTPUT, vocab, hidden))
     yield ("output_norm", -1, GGMLType.F32, 1, hidden, synth.normal(seed, synth.TID_OUT_NORM, hidden, 1.0, 0.01))
     for l in range(n_layers):
-        for slot, t, r, c in synth.layer_tensor_specs(hidden, ffn):
+        for slot, t, r, c in synth.layer_tensor_specs(hidden, ffn, kv_dim):
             yield (slot, l, t, r, c, synth.blocks(t, seed, synth.layer_tid(l, slot), r, c))
         yield ("attn_norm", l, GGMLType.F32, 1, hidden, synth.normal(seed, synth.layer_tid(l, "attn_norm"), hidden, 1.0, 0.01))
         yield ("ffn_norm", l, GGMLType.F32, 1, hidden, synth.normal(seed, synth.layer_tid(l, "ffn_norm"), hidden, 1.0, 0.01))
@@ -90,7 +93,7 @@ def load_synthetic(model: HipLlama, seed: int, sink: Callable | None = None) -> 
     """Upload a synthetic model; `sink(slot, layer, type, n_rows, n_cols, raw)` sees every tensor too. Returns weight bytes."""
     c = model.cfg
     total = 0
-    for slot, layer, t, r, cc, raw in synthetic_tensors(seed, c.n_layers, c.hidden, c.ffn, c.vocab):
+    for slot, layer, t, r, cc, raw in synthetic_tensors(seed, c.n_layers, c.hidden, c.ffn, c.vocab, model.kv_dim):
         model.upload(slot, layer, t, r, cc, raw)
         if sink is not None:
             sink(slot, layer, t, r, cc, raw)
@@ -111,7 +114,7 @@ def gguf_tensor_name(slot: str, layer: int) -> str:
 
 
 def write_synthetic_gguf(path, seed: int, n_layers: int, hidden: int, n_heads: int, ffn: int, vocab: int, context: int,
-                         rms_eps: float = 1e-5, rope_theta: float = 10000.0) -> None:
+                         rms_eps: float = 1e-5, rope_theta: float = 10000.0, n_kv_heads: int = 0) -> None:
     """A random-init Llama as a GGUF v3 file (same tensors as `synthetic_tensors`), so the file path can be
     exercised without a downloaded model."""
     from . import gguf
@@ -123,10 +126,10 @@ def write_synthetic_gguf(path, seed: int, n_layers: int, hidden: int, n_heads: i
     w.add_kv("llama.embedding_length", gguf.VT_UINT32, hidden)
     w.add_kv("llama.feed_forward_length", gguf.VT_UINT32, ffn)
     w.add_kv("llama.attention.head_count", gguf.VT_UINT32, n_heads)
-    w.add_kv("llama.attention.head_count_kv", gguf.VT_UINT32, n_heads)
+    w.add_kv("llama.attention.head_count_kv", gguf.VT_UINT32, n_kv_heads or n_heads)
     w.add_kv("llama.attention.layer_norm_rms_epsilon", gguf.VT_FLOAT32, rms_eps)
     w.add_kv("llama.rope.freq_base", gguf.VT_FLOAT32, rope_theta)
-    for slot, layer, t, r, c, raw in synthetic_tensors(seed, n_layers, hidden, ffn, vocab):
+    for slot, layer, t, r, c, raw in synthetic_tensors(seed, n_layers, hidden, ffn, vocab, (n_kv_heads or n_heads) * (hidden // n_heads)):
         dims = (c,) if t == GGMLType.F32 else (c, r)
         w.add_tensor(gguf_tensor_name(slot, layer), t, dims, raw)
     w.write(path)
@@ -156,8 +159,9 @@ def load_gguf(ex: HipKernelExecutor, path, max_pos: int | None = None) -> HipLla
         n_layers, hidden = need_u32("llama.block_count"), need_u32("llama.embedding_length")
         ffn, n_heads = need_u32("llama.feed_forward_length"), need_u32("llama.attention.head_count")
         kv = g.get_metadata("llama.attention.head_count_kv")
-        if kv is not None and kv.as_u32() not in (None, n_heads):
-            raise UnsupportedOperation("load_gguf: grouped-query attention (head_count_kv=%d) is not supported" % kv.as_u32())
+        n_kv = n_heads if kv is None or kv.as_u32() is None else kv.as_u32()
+        if n_kv == 0 or n_heads % n_kv != 0:
+            raise InvalidParameters("load_gguf: head_count_kv=%d does not divide head_count=%d" % (n_kv, n_heads))
         emb = g.find_tensor("token_embd.weight")
         if emb is None or emb.n_dims != 2:
             raise InvalidParameters("load_gguf: token_embd.weight missing or not 2-D")
@@ -166,7 +170,7 @@ def load_gguf(ex: HipKernelExecutor, path, max_pos: int | None = None) -> HipLla
         if max_pos is None:
             max_pos = ctx.as_u32() if ctx is not None and ctx.as_u32() else 2048
         model = HipLlama(ex, n_layers, hidden, n_heads, ffn, vocab, max_pos, opt_f32("llama.attention.layer_norm_rms_epsilon", 1e-5),
-                         opt_f32("llama.rope.freq_base", 10000.0))
+                         opt_f32("llama.rope.freq_base", 10000.0), n_kv)
         try:
             wanted = [(s, -1) for s in ("token_embd", "output", "output_norm")] + [(s, l) for l in range(n_layers) for s in _LAYER_NAMES]
             for slot, layer in wanted:

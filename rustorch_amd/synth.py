@@ -56,12 +56,14 @@ def layer_tid(layer: int, slot: str) -> int:
     return 100 * (layer + 1) + LAYER_SLOTS.index(slot)
 
 
-def layer_tensor_specs(hidden: int, ffn: int):
-    """(slot, ggml type, n_rows, n_cols) of one decoder layer: q, k, o, gate, up are Q4_K; v and down are Q6_K."""
+def layer_tensor_specs(hidden: int, ffn: int, kv_dim: int | None = None):
+    """(slot, ggml type, n_rows, n_cols) of one decoder layer: q, k, o, gate, up are Q4_K; v and down are Q6_K.
+    kv_dim = n_kv_heads * head_dim rows of k and v (default: hidden, one key / value head per query head)."""
+    kv_dim = hidden if kv_dim is None else kv_dim
     return [
         ("attn_q", GGMLType.Q4_K, hidden, hidden),
-        ("attn_k", GGMLType.Q4_K, hidden, hidden),
-        ("attn_v", GGMLType.Q6_K, hidden, hidden),
+        ("attn_k", GGMLType.Q4_K, kv_dim, hidden),
+        ("attn_v", GGMLType.Q6_K, kv_dim, hidden),
         ("attn_output", GGMLType.Q4_K, hidden, hidden),
         ("ffn_gate", GGMLType.Q4_K, ffn, hidden),
         ("ffn_up", GGMLType.Q4_K, ffn, hidden),

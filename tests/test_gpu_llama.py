@@ -8,10 +8,10 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-def build_pair(ex, orc, seed, n_layers, hidden, n_heads, ffn, vocab, max_pos):
+def build_pair(ex, orc, seed, n_layers, hidden, n_heads, ffn, vocab, max_pos, n_kv_heads=0):
     from rustorch_amd import llama
-    gm = llama.HipLlama(ex, n_layers, hidden, n_heads, ffn, vocab, max_pos)
-    om = orc.OracleLlama(n_layers, hidden, n_heads, ffn, vocab, max_pos)
+    gm = llama.HipLlama(ex, n_layers, hidden, n_heads, ffn, vocab, max_pos, n_kv_heads=n_kv_heads)
+    om = orc.OracleLlama(n_layers, hidden, n_heads, ffn, vocab, max_pos, n_kv_heads=n_kv_heads)
     head = {}
 
     def sink(slot, layer, t, r, c, raw):
@@ -99,6 +99,48 @@ def test_decode_loop_without_host_round_trips(ex, orc, mode):
         gm.step(cfg["vocab"], 20)           # token outside the vocabulary
     with pytest.raises(ShapeMismatch):
         gm.decode(1, 20, 13)                # would run past max_pos
+
+
+@pytest.mark.parametrize("n_heads,n_kv", [(8, 2), (4, 1), (4, 2)])
+def test_grouped_query_attention_model(ex, orc, n_heads, n_kv):
+    """Fewer key / value heads than query heads (k, v and the cache rows are n_kv * head_dim wide).
+
+    Exact check: a model with one kv head per query head whose k / v matrices repeat the rows of each shared head
+    computes the same thing, so stepping both on the GPU must give equal logits bit for bit.
+    Against the oracle: these tiny random models have attention scores in the thousands (a one-hot softmax), and
+    where two scores nearly tie the 16-bit activations pick the other row, for any head layout; so the bound is
+    asked of the typical position (median a tenth of the tolerance, nine positions in ten inside it)."""
+    from rustorch_amd import llama, synth, ShapeMismatch
+    cfg = dict(n_layers=2, hidden=512, n_heads=n_heads, ffn=1024, vocab=500, max_pos=48)
+    hd, group = cfg["hidden"] // n_heads, n_heads // n_kv
+    print("llama gqa", cfg, "n_kv", n_kv, flush=True)
+    gm, om, wn = build_pair(ex, orc, 31, n_kv_heads=n_kv, **cfg)
+    twin = llama.HipLlama(ex, **cfg)
+    rows = np.array([(h // group) * hd + d for h in range(n_heads) for d in range(hd)])
+    for slot, layer, t, r, c, raw in llama.synthetic_tensors(31, cfg["n_layers"], cfg["hidden"], cfg["ffn"], cfg["vocab"], n_kv * hd):
+        if slot in ("attn_k", "attn_v"):
+            raw = np.ascontiguousarray(raw.view(np.uint8).reshape(r, -1)[rows]).reshape(-1)
+            r = cfg["hidden"]
+        twin.upload(slot, layer, t, r, c, raw)
+    toks = synth.tokens(31, synth.TID_PROMPT, 40, cfg["vocab"])
+    want = om.forward(toks, 0)
+    tol = logit_tol(wn, cfg["hidden"])
+    ratios = []
+    for p, t in enumerate(toks[:24]):
+        gm.step(int(t), p); twin.step(int(t), p)
+        got = gm.logits()
+        assert np.array_equal(got, twin.logits()), "position %d" % p
+        ratios.append(float((np.abs(got - want[p]) / tol).max()))
+    gm.reset()
+    gm.prefill(toks[:30], 0)                                     # 30 tokens: the dense-contraction path
+    ratios.append(float((np.abs(gm.logits() - want[29]) / tol).max()))
+    out = gm.decode(int(toks[30]), 30, 9, toks[31:40])           # teacher forced continuation on the device
+    ratios.append(float((np.abs(gm.logits() - want[38]) / tol).max()))
+    ratios = np.array(ratios)
+    print("ratio to the tolerance: median %.3f, max %.2f, %d of %d above 1" % (np.median(ratios), ratios.max(), (ratios > 1).sum(), ratios.size), flush=True)
+    assert np.median(ratios) <= 0.1 and (ratios <= 1).mean() >= 0.9
+    with pytest.raises(ShapeMismatch):                           # k must have n_kv * head_dim rows
+        gm.upload("attn_k", 0, 12, 512, 512, synth.blocks(12, 1, 1, 512, 512))
 
 
 def test_graph_replay_equals_eager_launches(ex, orc):

@@ -131,6 +131,20 @@ def test_attention_properties(orc):
     assert np.array_equal(orc.attn_decode(q, kc2, vc2, 5, nh, hd), out)
 
 
+def test_grouped_query_attention_is_attention_over_repeated_kv_heads(orc):
+    """Fewer key / value heads than query heads: query head h reads kv head h // group.  Expanding the cache by
+    repeating every kv head `group` times must give the same numbers through the one-head-count routine."""
+    nh, nkv, hd, npos = 8, 2, 64, 7
+    rng = np.random.default_rng(9)
+    q = rng.standard_normal(nh * hd).astype(F32)
+    K = rng.standard_normal((npos, nkv, hd)).astype(F32); V = rng.standard_normal((npos, nkv, hd)).astype(F32)
+    got = orc.attn_decode(q, _cache(K.reshape(npos, -1)), _cache(V.reshape(npos, -1)), npos, nh, hd, nkv)
+    Kx = np.repeat(K, nh // nkv, axis=1).reshape(npos, -1); Vx = np.repeat(V, nh // nkv, axis=1).reshape(npos, -1)
+    assert np.array_equal(got, orc.attn_decode(q, _cache(Kx), _cache(Vx), npos, nh, hd))
+    # and one kv head per query head is the plain form
+    assert np.array_equal(orc.attn_decode(q, _cache(Kx), _cache(Vx), npos, nh, hd, nh), orc.attn_decode(q, _cache(Kx), _cache(Vx), npos, nh, hd))
+
+
 def test_kv_append_rounds_to_nearest_even(orc):
     v = np.array([1.0, 1.00048828125, 1.00146484375, 70000.0, -1e-8, 0.1], dtype=F32)
     cache = np.zeros((3, v.size), dtype=np.uint16)
