@@ -129,6 +129,9 @@ hipError_t launch_rope_kv(hipStream_t s, float *q, const float *k, const float *
 hipError_t launch_attn_decode(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
                               const int *pos_dev, int n_pos, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev,
                               float *out, uint8_t *xq, bool fused);
+hipError_t launch_attn_decode_split(hipStream_t s, const float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
+                                    const int *pos_dev, int max_pos, int n_splits, int n_heads, int n_kv_heads, int head_dim,
+                                    const float *inv_freq_dev, float *partials, float *out, uint8_t *xq);
 hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache,
                                 int pos0, size_t n_tok, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev);
 hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,

@@ -366,6 +366,151 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
     }
 }
 
+// ---- long contexts: the positions of a head are split over several workgroups
+// Workgroup (h, s) of the fused decode step covers positions [s * chunk, (s + 1) * chunk) of query head h and leaves
+// a partial result {m = max score, l = sum of exp(score - m), acc[HD] = sum of exp(score - m) * v} in
+// partials[(h * n_splits + s) * (HD + 2)]; attn_combine_kernel folds the splits of a head:
+//   M = max m_s,  out = sum_s acc_s * exp(m_s - M) / sum_s l_s * exp(m_s - M).
+// The workgroup whose range holds the current position rotates k, stores the new cache row (first query head of
+// a kv group only) and takes that row from LDS.  Splits past the current position report l = 0.
+// Dynamic LDS: chunk floats.
+template <int HD>
+__global__ __launch_bounds__(256) void attn_split_kernel(const float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
+                                                         const int *pos_dev, int chunk, int n_heads, int n_kv_heads,
+                                                         const float *inv_freq, float *partials) {
+    RT_DYN_LDS(float, sc);
+    __shared__ float red[4];
+    __shared__ __align__(16) float qs[HD];
+    __shared__ __align__(16) float kcur[HD];
+    __shared__ __align__(16) float vcur[HD];
+    __shared__ __align__(16) float part[2048];
+    constexpr int CH = HD / 8, NG = 256 / CH;
+    const int h = blockIdx.x, sp = blockIdx.y, n_splits = gridDim.y, tid = threadIdx.x;
+    const size_t rowkv = (size_t)n_kv_heads * HD;
+    const int group = n_heads / n_kv_heads, kvh = h / group;
+    const int cur = *pos_dev, n_pos = cur + 1;
+    const int j0 = sp * chunk, j1 = min(n_pos, j0 + chunk);
+    float *P = partials + ((size_t)h * n_splits + sp) * (HD + 2);
+    if (j0 >= n_pos) {                        // nothing stored in this range yet
+        if (tid == 0) { P[0] = -INFINITY; P[1] = 0.f; }
+        return;
+    }
+    const bool owns_cur = cur >= j0 && cur < j1;
+    const float scale = 1.0f / sqrtf((float)HD);
+    const int c = tid % CH, g = tid / CH;
+    // the thread's first key row does not depend on the new token: request it before the rotation
+    uint4 kreg[CH];
+    const int jt = j0 + tid;
+    const bool k_pre = jt < j1 && jt != cur;
+    if (k_pre) {
+        const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)jt * rowkv + (size_t)kvh * HD);
+#pragma unroll
+        for (int i = 0; i < CH; i++) kreg[i] = kr[i];
+    }
+    if (tid < HD / 2) {
+        const int i = tid;
+        float sn, cs;
+        sincosf((float)cur * inv_freq[i], &sn, &cs);
+        const float2 qv = reinterpret_cast<const float2 *>(q + (size_t)h * HD)[i];
+        qs[2 * i] = qv.x * cs - qv.y * sn;
+        qs[2 * i + 1] = qv.x * sn + qv.y * cs;
+        if (owns_cur) {
+            const float2 kv = reinterpret_cast<const float2 *>(k + (size_t)kvh * HD)[i];
+            const uint16_t a = f2h_rne(kv.x * cs - kv.y * sn), b = f2h_rne(kv.x * sn + kv.y * cs);
+            kcur[2 * i] = h2f(a);
+            kcur[2 * i + 1] = h2f(b);
+            if (h % group == 0) reinterpret_cast<uint32_t *>(kc + (size_t)cur * rowkv + (size_t)kvh * HD)[i] = (uint32_t)a | ((uint32_t)b << 16);
+        }
+    } else if (tid < HD && owns_cur) {
+        const int i = tid - HD / 2;
+        const float2 vv = reinterpret_cast<const float2 *>(v + (size_t)kvh * HD)[i];
+        const uint16_t a = f2h_rne(vv.x), b = f2h_rne(vv.y);
+        vcur[2 * i] = h2f(a);
+        vcur[2 * i + 1] = h2f(b);
+        if (h % group == 0) reinterpret_cast<uint32_t *>(vc + (size_t)cur * rowkv + (size_t)kvh * HD)[i] = (uint32_t)a | ((uint32_t)b << 16);
+    }
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int j = jt; j < j1; j += 256) {
+        float sum = 0.f;
+        if (j == cur) {
+#pragma unroll 8
+            for (int d = 0; d < HD; d++) sum += qs[d] * kcur[d];
+        } else {
+            const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)j * rowkv + (size_t)kvh * HD);
+#pragma unroll
+            for (int cc = 0; cc < CH; cc++) {
+                float f[8];
+                unpack8(j == jt ? kreg[cc] : kr[cc], f);
+#pragma unroll
+                for (int e = 0; e < 8; e++) sum += qs[8 * cc + e] * f[e];
+            }
+        }
+        sum *= scale;
+        sc[j - j0] = sum;
+        mx = fmaxf(mx, sum);
+    }
+    mx = block_max(mx, red);
+    float l = 0.f;
+    for (int j = jt; j < j1; j += 256) {
+        const float e = expf(sc[j - j0] - mx);
+        sc[j - j0] = e;
+        l += e;
+    }
+    l = block_sum(l, red);          // ends with a barrier: the weights are visible to every thread
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] = 0.f;
+    for (int j = j0 + g; j < j1; j += NG) {
+        float f[8];
+        if (j == cur) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) f[e] = vcur[8 * c + e];
+        } else {
+            unpack8(reinterpret_cast<const uint4 *>(vc + (size_t)j * rowkv + (size_t)kvh * HD)[c], f);
+        }
+        const float w = sc[j - j0];
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += w * f[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) part[g * HD + 8 * c + e] = acc[e];
+    __syncthreads();
+    if (tid < HD) {
+        float o = 0.f;
+        for (int gg = 0; gg < NG; gg++) o += part[gg * HD + tid];
+        P[2 + tid] = o;
+    }
+    if (tid == 0) { P[0] = mx; P[1] = l; }
+}
+
+// One workgroup of HD threads per query head: fold the partial results of its splits, write the head's slice of the
+// attention output (f32 when out != NULL) and its quantized form for the o-projection (when xq != NULL).
+template <int HD>
+__global__ __launch_bounds__(HD) void attn_combine_kernel(const float *partials, int n_splits, int n_heads, float *out, uint8_t *xq) {
+    __shared__ __align__(16) float res[HD];
+    const int h = blockIdx.x, tid = threadIdx.x;
+    const float *P = partials + (size_t)h * n_splits * (HD + 2);
+    float M = -INFINITY;
+    for (int s = 0; s < n_splits; s++) M = fmaxf(M, P[(size_t)s * (HD + 2)]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < n_splits; s++) {
+        const float *Ps = P + (size_t)s * (HD + 2);
+        if (Ps[1] > 0.f) {                     // a split past the current position holds nothing (its acc is not written)
+            const float w = expf(Ps[0] - M);
+            num += Ps[2 + tid] * w;
+            den += Ps[1] * w;
+        }
+    }
+    const float o = num / den;
+    res[tid] = o;
+    if (out) out[(size_t)h * HD + tid] = o;
+    if (xq) {
+        __syncthreads();
+        if (tid < HD / 4) quantize_store4(reinterpret_cast<const float4 *>(res)[tid], (size_t)h * HD + tid * 4, xq, (size_t)n_heads * HD);
+    }
+}
+
 // ------------------------------------------------------------- small pieces
 __global__ void add_kernel(float *x, const float *y, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -606,6 +751,27 @@ hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const floa
         attn_decode_kernel<64, false><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, n_pos, n_heads, n_kv_heads, inv_freq_dev, out, xq);
     else
         return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+// Fused decode step over a long context: n_splits workgroups per head (positions in chunks of ceil(max_pos / n_splits)),
+// then the fold.  partials: n_heads * n_splits * (head_dim + 2) floats.
+hipError_t launch_attn_decode_split(hipStream_t s, const float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
+                                    const int *pos_dev, int max_pos, int n_splits, int n_heads, int n_kv_heads, int head_dim,
+                                    const float *inv_freq_dev, float *partials, float *out, uint8_t *xq) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads != 0 || n_splits < 1) return hipErrorInvalidValue;
+    const int chunk = (max_pos + n_splits - 1) / n_splits;
+    const size_t lds = (size_t)chunk * sizeof(float);
+    dim3 grid((unsigned)n_heads, (unsigned)n_splits);
+    if (head_dim == 128) {
+        attn_split_kernel<128><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, chunk, n_heads, n_kv_heads, inv_freq_dev, partials);
+        attn_combine_kernel<128><<<dim3((unsigned)n_heads), 128, 0, s>>>(partials, n_splits, n_heads, out, xq);
+    } else if (head_dim == 64) {
+        attn_split_kernel<64><<<grid, 256, lds, s>>>(q, k, v, kc, vc, pos_dev, chunk, n_heads, n_kv_heads, inv_freq_dev, partials);
+        attn_combine_kernel<64><<<dim3((unsigned)n_heads), 64, 0, s>>>(partials, n_splits, n_heads, out, xq);
+    } else {
+        return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

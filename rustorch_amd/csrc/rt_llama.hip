@@ -32,6 +32,8 @@ struct rt_hip_llama {
     int head_dim = 0;
     int n_kv = 0;             // key / value heads; kv_dim = n_kv * head_dim is the width of k, v and of a cache row
     size_t kv_dim = 0;
+    int attn_splits = 1;      // workgroups per head in the decode step's attention (long contexts), fixed by max_pos
+    float *attn_part = nullptr;
     T tok_embd, output;
     float *out_norm = nullptr;
     std::vector<T> wq, wk, wv, wo, wgate, wup, wdown;
@@ -66,6 +68,10 @@ struct rt_hip_llama {
 };
 
 namespace {
+
+#ifndef RT_ATTN_SPLIT_MIN
+#define RT_ATTN_SPLIT_MIN 512
+#endif
 
 int dev_alloc(rt_hip_ctx *ctx, rt_hip_llama *m, void **p, size_t bytes) {
     RT_TRY_HIP(ctx, hipMalloc(p, bytes ? bytes : 1));
@@ -130,8 +136,12 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
         a.p[2] = make_prob(m->wv[l], m->x, rt::kStageRms, m->v, nullptr);
         for (int i = 0; i < 3; i++) { a.p[i].gamma = m->attn_norm[l]; a.p[i].eps = c.rms_eps; }
         RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
-        RT_TRY_HIP(ctx, rt::launch_attn_decode(s, m->q, m->k, m->v, kc, vc, pos_dev, c.max_pos, c.n_heads, m->n_kv, m->head_dim, m->inv_freq,
-                                               nullptr, m->xq_a, true));
+        if (m->attn_splits > 1)
+            RT_TRY_HIP(ctx, rt::launch_attn_decode_split(s, m->q, m->k, m->v, kc, vc, pos_dev, c.max_pos, m->attn_splits, c.n_heads, m->n_kv,
+                                                         m->head_dim, m->inv_freq, m->attn_part, nullptr, m->xq_a));
+        else
+            RT_TRY_HIP(ctx, rt::launch_attn_decode(s, m->q, m->k, m->v, kc, vc, pos_dev, c.max_pos, c.n_heads, m->n_kv, m->head_dim, m->inv_freq,
+                                                   nullptr, m->xq_a, true));
         memset(&a, 0, sizeof a);
         a.n = 1;
         a.p[0] = make_prob(m->wo[l], m->xq_a, rt::kStageXq, m->x, m->x);
@@ -263,6 +273,10 @@ int rt_hip_llama_create(rt_hip_ctx *ctx, const rt_hip_llama_config *cfg, rt_hip_
     m->attn_norm.assign(L, nullptr); m->ffn_norm.assign(L, nullptr);
     int rc = RT_HIP_OK;
     auto A = [&](void **p, size_t b) { if (rc == RT_HIP_OK) rc = dev_alloc(ctx, m, p, b); };
+    // One workgroup per head serves a short cache; from RT_ATTN_SPLIT_MIN positions on, a head's positions are spread over
+    // up to eight workgroups of at least half that many each (a fixed shape per model, so a captured step stays valid).
+    m->attn_splits = cfg->max_pos >= RT_ATTN_SPLIT_MIN ? std::min(8, (cfg->max_pos + RT_ATTN_SPLIT_MIN / 2 - 1) / (RT_ATTN_SPLIT_MIN / 2)) : 1;
+    A((void **)&m->attn_part, (size_t)cfg->n_heads * (size_t)m->attn_splits * (size_t)(hd + 2) * sizeof(float));
     A((void **)&m->kcache, L * P * m->kv_dim * 2); A((void **)&m->vcache, L * P * m->kv_dim * 2);
     A((void **)&m->x, H * 4); A((void **)&m->q, H * 4); A((void **)&m->k, H * 4); A((void **)&m->v, H * 4);
     A((void **)&m->g, F * 4); A((void **)&m->u, F * 4); A((void **)&m->logits, V * 4);
