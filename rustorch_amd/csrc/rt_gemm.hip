@@ -304,15 +304,23 @@ __device__ __forceinline__ void prep_piece(SbK<RT_GGML_Q4_K> &k, const WSb<RT_GG
 // A step's operand is four such pairs; they are produced one at a time so that each can be issued behind
 // one matrix instruction.  w = (n/16) * (16*d*sc) - dmin*m: the subtraction of the exponent's 2^E is exact, so
 // the only roundings are those of the scale, of the offset and of the final fma.
-__device__ __forceinline__ half2v expand_unit(const WSb<RT_GGML_Q4_K> &w, const SbK<RT_GGML_Q4_K> &k, int t, int s, int u, ExpPat G) {
+// The three dependent operations of a pair are separate stages (bits -> fp16 with the exponent, exact subtraction
+// of the exponent's value, scale and offset), so that the caller can interleave the stages of different pairs:
+// two dependent vector operations issued back to back cost a wait state each.
+__device__ __forceinline__ uint32_t expand_s1(const WSb<RT_GGML_Q4_K> &w, const SbK<RT_GGML_Q4_K> &, int t, int s, int u, ExpPat G) {
     const int hi = s >> 1;
     const u32x4 qs = w.qs[t];
     const uint32_t q = (s & 1) ? ((u & 2) ? qs.w : qs.z) : ((u & 2) ? qs.y : qs.x);
     // pair u & 1 = 0 takes bytes 0 and 2 of the word, pair 1 bytes 1 and 3 (one shift brings them down)
     const uint32_t src = (u & 1) ? (q >> 8) : q;
-    const half2v a = splat_h(k.a[t][hi]), c = splat_h(k.c[t][hi]);
-    if (hi) return (as_h2(and_or(src, 0x00F000F0u, G.hi)) - splat(4.f)) * a + c;
-    return (as_h2(and_or(src, 0x000F000Fu, G.lo)) - splat(64.f)) * a + c;
+    return hi ? and_or(src, 0x00F000F0u, G.hi) : and_or(src, 0x000F000Fu, G.lo);
+}
+__device__ __forceinline__ half2v expand_s2(const SbK<RT_GGML_Q4_K> &, uint32_t x, int, int s) {
+    return as_h2(x) - ((s >> 1) ? splat(4.f) : splat(64.f));
+}
+__device__ __forceinline__ half2v expand_s3(const SbK<RT_GGML_Q4_K> &k, half2v y, int t, int s) {
+    const int hi = s >> 1;
+    return y * splat_h(k.a[t][hi]) + splat_h(k.c[t][hi]);
 }
 
 __device__ __forceinline__ void prep_piece(SbK<RT_GGML_Q6_K> &k, const WSb<RT_GGML_Q6_K> &w, int h, int piece) {
@@ -330,7 +338,7 @@ __device__ __forceinline__ void prep_piece(SbK<RT_GGML_Q6_K> &k, const WSb<RT_GG
     }
 }
 
-__device__ __forceinline__ half2v expand_unit(const WSb<RT_GGML_Q6_K> &w, const SbK<RT_GGML_Q6_K> &k, int t, int s, int u, ExpPat G) {
+__device__ __forceinline__ uint32_t expand_s1(const WSb<RT_GGML_Q6_K> &w, const SbK<RT_GGML_Q6_K> &, int t, int s, int u, ExpPat G) {
     const int hf = t >> 1, p = t & 1, j = s >> 1, tt = s & 1;
     const u32x4 L = j ? w.B[hf] : w.A[hf];    // run parity = j: even runs read ql[l], odd runs ql[l + 32]
     const u32x4 H = w.H[hf];
@@ -341,10 +349,17 @@ __device__ __forceinline__ half2v expand_unit(const WSb<RT_GGML_Q6_K> &w, const 
     const int shh = 2 * (2 * p + j);
     const uint32_t hb = shh <= 4 ? (hq << (4 - shh)) : (hq >> (shh - 4));
     const uint32_t v = (hb & 0x30303030u) | lo;
-    // 16 + v/64 minus 16.5 is (v - 32)/64 exactly, so w = 64*d*sc * (v - 32)/64 carries only the rounding of the
-    // scale and of the product
     const uint32_t src = (u & 1) ? (v >> 8) : v;
-    return (as_h2(and_or(src, 0x003F003Fu, G.lo)) - splat(16.5f)) * splat_h(k.a[t][j]);
+    return and_or(src, 0x003F003Fu, G.lo);
+}
+// 16 + v/64 minus 16.5 is (v - 32)/64 exactly, so w = 64*d*sc * (v - 32)/64 carries only the rounding of the
+// scale and of the product
+__device__ __forceinline__ half2v expand_s2(const SbK<RT_GGML_Q6_K> &, uint32_t x, int, int) { return as_h2(x) - splat(16.5f); }
+__device__ __forceinline__ half2v expand_s3(const SbK<RT_GGML_Q6_K> &k, half2v y, int t, int s) { return y * splat_h(k.a[t][s >> 1]); }
+
+template <int TYPE>
+__device__ __forceinline__ half2v expand_unit(const WSb<TYPE> &w, const SbK<TYPE> &k, int t, int s, int u, ExpPat G) {
+    return expand_s3(k, expand_s2(k, expand_s1(w, k, t, s, u, G), t, s), t, s);
 }
 
 template <int TYPE>
@@ -401,6 +416,9 @@ template <int TYPE> struct Ride {
     static constexpr int fetch_hi(int t, int s) { int k = 4 * (t - 2) + s - 3; return k < 0 ? n_fetch : (2 * k + 2 < n_fetch ? 2 * k + 2 : n_fetch); }
 };
 
+// (stage, pair) in issue order, three per matrix instruction at MF = 4, six at MF = 2
+constexpr int kExpandOrder[12][2] = { {1, 0}, {1, 1}, {1, 2}, {1, 3}, {2, 0}, {2, 1}, {2, 2}, {2, 3}, {3, 0}, {3, 1}, {3, 2}, {3, 3} };
+
 template <int TYPE, int MF, int XI, class IssueX>
 __device__ __forceinline__ void superblock(float16v (&acc)[MF], const WSb<TYPE> &w, const SbK<TYPE> &k, WTmp<TYPE> &tmp,
                                            const WOff<TYPE> &woff, const uint8_t *wnext, WSb<TYPE> &wn, SbK<TYPE> &kn, half8v &a,
@@ -409,7 +427,7 @@ __device__ __forceinline__ void superblock(float16v (&acc)[MF], const WSb<TYPE> 
     using Geo = WGeo<TYPE>;
     using R = Ride<TYPE>;
     constexpr int WL = Geo::loads + Geo::tail;
-    constexpr int UPM = (4 + MF - 1) / MF;                        // expansion pairs issued behind each matrix instruction
+    static_assert(12 % MF == 0, "the stage operations are dealt evenly over the matrix instructions");
     constexpr int PPS = (kPrepPieces + 2 * MF - 1) / (2 * MF);   // preparation pieces per slot of tile 3, steps 1 and 2
     constexpr int kStageBytes = 32 * MF * kBK * 2;
     static_for<0, 4>([&](auto T) {
@@ -435,14 +453,29 @@ __device__ __forceinline__ void superblock(float16v (&acc)[MF], const WSb<TYPE> 
             static_for<R::fetch_lo(t, s), R::fetch_hi(t, s)>([&](auto O) { fetch_op<decltype(O)::value>(wn, la.wrow, la.wrow_h, la.wtail); });
             wait_lgkmcnt_c<MF + R::fetch_hi(t, s) - R::fetch_lo(t, s)>();
             __builtin_amdgcn_sched_barrier(0);
+            uint32_t ex[4];
+            half2v ey[4];
+            // stage g (1 bits, 2 subtraction, 3 scale) of pair q of the next step's operand
+            auto stage = [&](auto Gc, auto Qc) {
+                constexpr int g = decltype(Gc)::value, q = decltype(Qc)::value;
+                if constexpr (tn < 4) {
+                    if constexpr (g == 1) { ex[q] = expand_s1(w, k, tn, sn, q, G); pin(ex[q]); }
+                    else if constexpr (g == 2) { ey[q] = expand_s2(k, ex[q], tn, sn); pin(ey[q]); }
+                    else { an[q] = expand_s3(k, ey[q], tn, sn); pin(an[q]); }
+                } else {
+                    if constexpr (g == 1) { ex[q] = expand_s1(wn, kn, 0, 0, q, G); pin(ex[q]); }
+                    else if constexpr (g == 2) { ey[q] = expand_s2(kn, ex[q], 0, 0); pin(ey[q]); }
+                    else { an[q] = expand_s3(kn, ey[q], 0, 0); pin(an[q]); }
+                }
+            };
             static_for<0, MF>([&](auto J) {
                 constexpr int j = decltype(J)::value;
                 acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bb[cur][j], a, acc[j], 0, 0, 0);
-                static_for<j * UPM, (j + 1) * UPM < 4 ? (j + 1) * UPM : 4>([&](auto Q) {
-                    constexpr int q = decltype(Q)::value;
-                    if constexpr (tn < 4) an[q] = expand_unit(w, k, tn, sn, q, G);
-                    else an[q] = expand_unit(wn, kn, 0, 0, q, G);
-                    pin(an[q]);
+                // The 12 stage operations of the four pairs are dealt over the MF slots in the order of
+                // kExpandOrder: three other operations lie between an operation and the one that depends on it.
+                static_for<j * (12 / MF), (j + 1) * (12 / MF)>([&](auto I) {
+                    constexpr int i = decltype(I)::value;
+                    stage(std::integral_constant<int, kExpandOrder[i][0]>{}, std::integral_constant<int, kExpandOrder[i][1]>{});
                 });
                 if constexpr (t == 3 && (s == 1 || s == 2)) {
                     constexpr int p0 = ((s - 1) * MF + j) * PPS, p1 = p0 + PPS < kPrepPieces ? p0 + PPS : kPrepPieces;
