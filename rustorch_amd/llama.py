@@ -192,7 +192,7 @@ def load_gguf(ex: HipKernelExecutor, path, max_pos: int | None = None) -> HipLla
 
 
 def generate(model: HipLlama, prompt: Iterable[int], max_new_tokens: int, config=None, eos_token: int | None = None,
-             rng=None, pos0: int = 0) -> list[int]:
+             rng=None, pos0: int = 0, on_token: Callable[[int], None] | None = None) -> list[int]:
     """Prompt in, new tokens out: the loop of `InferenceEngine::generate_with_gpt`
     (example-cli/src/model/inference.rs:135-192) -- forward, logits of the last position, pick, stop at the
     end-of-sequence token or at max_new_tokens.  Greedy configurations run entirely on the device
@@ -211,9 +211,18 @@ def generate(model: HipLlama, prompt: Iterable[int], max_new_tokens: int, config
         model.prefill(toks[:-1], pos0)
     pos = pos0 + len(toks) - 1
     if config.is_greedy and config.repetition_penalty == 1.0:
-        out = [int(t) for t in model.decode(toks[-1], pos, n_new)]
-        if eos_token is not None and eos_token in out:
-            out = out[:out.index(eos_token) + 1]
+        # the first token comes back on its own (the caller's time to first token), the rest in one device-side loop
+        out = [int(model.step(toks[-1], pos))]
+        if on_token is not None:
+            on_token(out[0])
+        if n_new > 1 and out[0] != eos_token:
+            rest = [int(t) for t in model.decode(out[0], pos + 1, n_new - 1)]
+            if eos_token is not None and eos_token in rest:
+                rest = rest[:rest.index(eos_token) + 1]
+            if on_token is not None:
+                for t in rest:
+                    on_token(t)
+            out += rest
         return out
     out: list[int] = []
     cur = toks[-1]
@@ -221,6 +230,8 @@ def generate(model: HipLlama, prompt: Iterable[int], max_new_tokens: int, config
         model.step(cur, pos, want_token=False)
         cur = sample_token(model.logits(), config, toks + out, rng)
         out.append(cur)
+        if on_token is not None:
+            on_token(cur)
         pos += 1
         if eos_token is not None and cur == eos_token:
             break
