@@ -690,11 +690,13 @@ hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t
     constexpr int BM = 32 * MF, BN = 32 * NW;
     const size_t lds = (size_t)4 * BM * kBK * sizeof(_Float16) + (size_t)NW * WGeo<TYPE>::stage_bytes;
     auto kern = qgemm_kernel<TYPE, NW, MF>;
-    static bool attr_set = false;      // per instantiation
-    if (!attr_set && lds > 64 * 1024) {
+    static bool attr_set[64] = {};     // per instantiation and device: the attribute belongs to the function as loaded on a device
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    if (!attr_set[dev] && lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        attr_set = true;
+        attr_set[dev] = true;
     }
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
     const int total = tiles_m * p.ksplit * tiles_n;

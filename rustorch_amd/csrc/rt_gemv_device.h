@@ -134,31 +134,50 @@ template <> struct XRegs<RT_GGML_Q8_0> { uint4 h[2], l[2]; float s; };
 template <> struct WRegs<RT_GGML_Q4_0> { uint4 a; uint32_t d; };
 template <> struct XRegs<RT_GGML_Q4_0> { uint4 h[2], l[2]; float2 sv; };
 
-// row is wave-uniform; the lane part of the address is a 32-bit offset
-__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_K> &w, const uint8_t *row, int u) {
+// Weight loads go through a buffer resource: the matrix is the buffer, the row (wave-uniform) a scalar byte
+// offset, the lane's place in the row a 32-bit vector offset -- no 64-bit address arithmetic per load.
+struct WRow {
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t soff;      // row * row_bytes
+};
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t weight_rsrc(const uint8_t *w) {
+    // raw buffer (stride 0), no range limit of its own (rows and units are clamped by the caller), dword 3 as for 32-bit data
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w), 0, 0xFFFFFFFFu, 0x00020000);
+}
+__device__ __forceinline__ uint4 bld16(WRow r, uint32_t off) {
+    return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r.rsrc, off, r.soff, 0));
+}
+__device__ __forceinline__ uint2 bld8(WRow r, uint32_t off) {
+    return __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r.rsrc, off, r.soff, 0));
+}
+__device__ __forceinline__ uint32_t bld2(WRow r, uint32_t off) {
+    return (uint32_t)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r.rsrc, off, r.soff, 0);
+}
+
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_K> &w, WRow row, int u) {
     uint32_t off = (uint32_t)(u >> 2) * 144u, g = (uint32_t)(u & 3);
-    w.hdr = ld16a(row + off);
-    w.qa = ld16a(row + off + 16u + 32u * g);
-    w.qb = ld16a(row + off + 32u + 32u * g);
+    w.hdr = bld16(row, off);
+    w.qa = bld16(row, off + 16u + 32u * g);
+    w.qb = bld16(row, off + 32u + 32u * g);
 }
-__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q6_K> &w, const uint8_t *row, int u) {
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q6_K> &w, WRow row, int u) {
     uint32_t off = (uint32_t)(u >> 2) * 210u, h = (uint32_t)((u >> 1) & 1), c = (uint32_t)(u & 1);
-    w.A = ld16u(row + off + 64u * h + 16u * c);
-    w.B = ld16u(row + off + 64u * h + 32u + 16u * c);
-    w.H = ld16u(row + off + 128u + 32u * h + 16u * c);
-    w.sc = ld8u(row + off + 192u + 8u * h);
-    w.d = ld2u(row + off + 208u);
+    w.A = bld16(row, off + 64u * h + 16u * c);
+    w.B = bld16(row, off + 64u * h + 32u + 16u * c);
+    w.H = bld16(row, off + 128u + 32u * h + 16u * c);
+    w.sc = bld8(row, off + 192u + 8u * h);
+    w.d = bld2(row, off + 208u);
 }
-__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q8_0> &w, const uint8_t *row, int u) {
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q8_0> &w, WRow row, int u) {
     uint32_t off = (uint32_t)u * 34u;
-    w.d = ld2u(row + off);
-    w.a = ld16u(row + off + 2u);
-    w.b = ld16u(row + off + 18u);
+    w.d = bld2(row, off);
+    w.a = bld16(row, off + 2u);
+    w.b = bld16(row, off + 18u);
 }
-__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_0> &w, const uint8_t *row, int u) {
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_0> &w, WRow row, int u) {
     uint32_t off = (uint32_t)u * 18u;
-    w.d = ld2u(row + off);
-    w.a = ld16u(row + off + 2u);
+    w.d = bld2(row, off);
+    w.a = bld16(row, off + 2u);
 }
 
 __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_K> &x, const uint32_t *lds, int u, int U, int K) {
@@ -297,6 +316,7 @@ struct Walker {
     const uint32_t *lds;
     int m, U, n_iter, lane, gw, n_gw, n_groups, rows_per_group;
     bool dual;
+    __amdgpu_buffer_rsrc_t rsrc, rsrc2;
 
     // A step is (row group g, unit pass p); steps are walked in order, so the position is advanced, not divided out.
     struct Pos { int g, p; };
@@ -314,8 +334,8 @@ struct Walker {
         for (int r = 0; r < R; r++) {
             int row = dual ? g * rows_per_group + (r >> 1) : g * rows_per_group + r;
             row = min(row, P.N - 1);  // ragged tail: reread the last row, the store is skipped
-            const uint8_t *rp = ((dual && (r & 1)) ? P.w2 : P.w) + (uint32_t)row * (uint32_t)P.row_bytes;   // a tensor is below 4 GB (checked at launch)
-            load_w(w[r], rp, u);
+            // a tensor is below 4 GB (checked at launch), so the row offset fits the 32-bit scalar offset of the load
+            load_w(w[r], WRow{ (dual && (r & 1)) ? rsrc2 : rsrc, (uint32_t)row * (uint32_t)P.row_bytes }, u);
             if (!dual && P.res) rv[r] = ld_f<COH>(&P.res[(size_t)m * P.N + row]);
         }
     }
@@ -362,7 +382,8 @@ struct Walker {
 template <int TYPE, int R, bool COH>
 __device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg, int m, uint32_t *lds, float *red) {
     const int waves = (int)(blockDim.x >> 6);
-    Walker<TYPE, R, COH> W{ P, lds, m, units_of(TYPE, P.K), 0, (int)(threadIdx.x & 63), 0, 0, 0, 0, P.epi == kEpiSwiglu };
+    Walker<TYPE, R, COH> W{ P, lds, m, units_of(TYPE, P.K), 0, (int)(threadIdx.x & 63), 0, 0, 0, 0, P.epi == kEpiSwiglu,
+                            weight_rsrc(P.w), weight_rsrc(P.epi == kEpiSwiglu ? P.w2 : P.w) };
     W.n_iter = (W.U + 63) / 64;
     W.rows_per_group = W.dual ? R / 2 : R;
     W.n_groups = (P.N + W.rows_per_group - 1) / W.rows_per_group;
