@@ -54,6 +54,7 @@ typedef enum {
     RT_GGML_Q4_0 = 2,
     RT_GGML_Q8_0 = 8,
     RT_GGML_Q4_K = 12,
+    RT_GGML_Q5_K = 13,
     RT_GGML_Q6_K = 14
 } rt_ggml_type;
 

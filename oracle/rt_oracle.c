@@ -43,7 +43,7 @@
 
 #define ORC_API __attribute__((visibility("default")))
 
-enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q6_K = 14 };
+enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };
 
 /* ------------------------------------------------------------------ fp16 */
 
@@ -105,7 +105,7 @@ static inline uint16_t rd_u16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1]
 ORC_API int orc_block_elems(int type) {
     switch (type) {
     case ORC_Q8_0: case ORC_Q4_0: return 32;
-    case ORC_Q4_K: case ORC_Q6_K: return 256;
+    case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 256;
     case ORC_F32: case ORC_F16: return 1;
     default: return 0;
     }
@@ -117,6 +117,7 @@ ORC_API int orc_block_bytes(int type) {
     case ORC_Q8_0: return 34;
     case ORC_Q4_0: return 18;
     case ORC_Q4_K: return 144;
+    case ORC_Q5_K: return 176;
     case ORC_Q6_K: return 210;
     case ORC_F32: return 4;
     case ORC_F16: return 2;
@@ -172,6 +173,30 @@ static void deq_q4_k(const uint8_t *b, float *y) {
     }
 }
 
+/*
+ * Q5_K: { f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128] } (176 B, type id 13, gguf.rs:91,137): Q4_K with a
+ * fifth bit per element; sub-block j takes bit j of qh[l].  Build-owned like the other block decoders
+ * (the public ggml definition); the reference holds nothing that pins it: parity unpinned.
+ */
+static void deq_q5_k(const uint8_t *b, float *y) {
+    float d = orc_h2f(rd_u16(b));
+    float dmin = orc_h2f(rd_u16(b + 2));
+    const uint8_t *scales = b + 4;
+    const uint8_t *qh = b + 16;
+    const uint8_t *q = b + 48;
+    for (int g = 0; g < 4; g++) {
+        uint8_t sc, m;
+        q4k_scale_min(2 * g, scales, &sc, &m);
+        float d1 = d * (float)sc, m1 = dmin * (float)m;
+        q4k_scale_min(2 * g + 1, scales, &sc, &m);
+        float d2 = d * (float)sc, m2 = dmin * (float)m;
+        int u1 = 1 << (2 * g), u2 = 2 << (2 * g);
+        for (int l = 0; l < 32; l++) y[64 * g + l] = d1 * (float)((q[l] & 0x0F) + ((qh[l] & u1) ? 16 : 0)) - m1;
+        for (int l = 0; l < 32; l++) y[64 * g + 32 + l] = d2 * (float)((q[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - m2;
+        q += 32;
+    }
+}
+
 /* Q6_K: { u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d } */
 static void deq_q6_k(const uint8_t *b, float *y) {
     const uint8_t *ql = b;
@@ -199,6 +224,7 @@ static void deq_row(int type, const uint8_t *row, size_t n_cols, float *y) {
     case ORC_Q8_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q8_0(row + 34 * b, y + 32 * b); break;
     case ORC_Q4_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q4_0(row + 18 * b, y + 32 * b); break;
     case ORC_Q4_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q4_k(row + 144 * b, y + 256 * b); break;
+    case ORC_Q5_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q5_k(row + 176 * b, y + 256 * b); break;
     case ORC_Q6_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q6_k(row + 210 * b, y + 256 * b); break;
     case ORC_F32: memcpy(y, row, n_cols * 4); break;
     case ORC_F16: for (size_t i = 0; i < n_cols; i++) y[i] = orc_h2f(rd_u16(row + 2 * i)); break;

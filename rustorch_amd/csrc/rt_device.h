@@ -99,6 +99,21 @@ __device__ inline float deq_elem(int type, const uint8_t *row, size_t col) {
         int q = (j & 1) ? (qb >> 4) : (qb & 0x0F);
         return d * (float)q - mn;
     }
+    case RT_GGML_Q5_K: {       // { f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128] }: Q4_K with a fifth bit per element in qh
+        const uint8_t *b = row + 176 * (col >> 8);
+        int e = (int)(col & 255);
+        int j = e >> 5;             // sub-block 0..7: its fifth bits are bit j of qh[l]
+        int l = e & 31;
+        const uint8_t *s = b + 4;
+        int sc, m;
+        if (j < 4) { sc = s[j] & 63; m = s[j + 4] & 63; }
+        else { sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4); m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4); }
+        float d = h2f(ld2u(b)) * (float)sc;
+        float mn = h2f(ld2u(b + 2)) * (float)m;
+        uint8_t qb = b[48 + 32 * (j >> 1) + l];
+        int q = ((j & 1) ? (qb >> 4) : (qb & 0x0F)) + (((b[16 + l] >> j) & 1) ? 16 : 0);
+        return d * (float)q - mn;
+    }
     case RT_GGML_Q6_K: {
         const uint8_t *b = row + 210 * (col >> 8);
         int e = (int)(col & 255);

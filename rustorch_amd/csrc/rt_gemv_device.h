@@ -26,14 +26,14 @@
 namespace rt {
 
 __device__ __forceinline__ int units_of(int type, int K) {
-    return (type == RT_GGML_Q4_K || type == RT_GGML_Q6_K) ? K / 64 : K / 32;
+    return (type == RT_GGML_Q4_K || type == RT_GGML_Q5_K || type == RT_GGML_Q6_K) ? K / 64 : K / 32;
 }
 
 // dword index inside a plane (xh or xl) of the 4 elements starting at e (e % 4 == 0)
 __device__ __forceinline__ int x_slot_dword(int type, int e, int U) {
     int j = e >> 4, w = (e >> 2) & 3;
     int slot;
-    if (type == RT_GGML_Q4_K) slot = (j & 3) * U + (j >> 2);
+    if (type == RT_GGML_Q4_K || type == RT_GGML_Q5_K) slot = (j & 3) * U + (j >> 2);
     else if (type == RT_GGML_Q6_K) slot = ((j >> 1) & 3) * U + (2 * (j >> 3) + (j & 1));
     else slot = (j & 1) * U + (j >> 1);
     return slot * 4 + w;
@@ -41,7 +41,7 @@ __device__ __forceinline__ int x_slot_dword(int type, int e, int U) {
 
 // Place 4 quantized elements and the block metadata they carry into the per-type LDS layout.
 //   planes: xh at dword 0, xl at dword K/4; floats S from dword K/2:
-//   Q4_K : S[4u + {0,1}] = scale of the unit's two 32-blocks, S[4u + {2,3}] = scale * sum of each block
+//   Q4_K, Q5_K : S[4u + {0,1}] = scale of the unit's two 32-blocks, S[4u + {2,3}] = scale * sum of each block
 //   Q6_K : S[b] = scale of 32-block b (= 4 * half + run);  S[2U + 4u + r] = scale * sum of the unit's run r
 //   Q8_0 : S[u] = scale;   Q4_0 : S[2u] = scale, S[2u+1] = scale * sum of the block
 __device__ __forceinline__ void stage_store(int type, int K, int U, uint32_t *lds, int e, uint32_t hi, uint32_t lo,
@@ -50,7 +50,7 @@ __device__ __forceinline__ void stage_store(int type, int K, int U, uint32_t *ld
     lds[d] = hi;
     lds[K / 4 + d] = lo;
     float *S = reinterpret_cast<float *>(lds + K / 2);
-    if (type == RT_GGML_Q4_K) {
+    if (type == RT_GGML_Q4_K || type == RT_GGML_Q5_K) {
         if ((e & 31) == 0) {
             int b = e >> 5, u = b >> 1, half = b & 1;
             S[4 * u + half] = s;
@@ -127,6 +127,8 @@ template <int TYPE> struct XRegs;
 
 template <> struct WRegs<RT_GGML_Q4_K> { uint4 hdr, qa, qb; };
 template <> struct XRegs<RT_GGML_Q4_K> { uint4 h[4], l[4]; float4 sv; };
+template <> struct WRegs<RT_GGML_Q5_K> { uint4 hdr, ha, hb, qa, qb; };     // header, the 32 bytes of fifth bits, the unit's 32 nibble bytes
+template <> struct XRegs<RT_GGML_Q5_K> : XRegs<RT_GGML_Q4_K> {};              // same 64-element units, same x slice
 template <> struct WRegs<RT_GGML_Q6_K> { uint4 A, B, H; uint2 sc; uint32_t d; };
 template <> struct XRegs<RT_GGML_Q6_K> { uint4 h[4], l[4]; float4 xs, xb; };
 template <> struct WRegs<RT_GGML_Q8_0> { uint4 a, b; uint32_t d; };
@@ -160,6 +162,14 @@ __device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_K> &w, WRow row, int u) 
     w.qa = bld16(row, off + 16u + 32u * g);
     w.qb = bld16(row, off + 32u + 32u * g);
 }
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q5_K> &w, WRow row, int u) {
+    uint32_t off = (uint32_t)(u >> 2) * 176u, g = (uint32_t)(u & 3);
+    w.hdr = bld16(row, off);
+    w.ha = bld16(row, off + 16u);
+    w.hb = bld16(row, off + 32u);
+    w.qa = bld16(row, off + 48u + 32u * g);
+    w.qb = bld16(row, off + 64u + 32u * g);
+}
 __device__ __forceinline__ void load_w(WRegs<RT_GGML_Q6_K> &w, WRow row, int u) {
     uint32_t off = (uint32_t)(u >> 2) * 210u, h = (uint32_t)((u >> 1) & 1), c = (uint32_t)(u & 1);
     w.A = bld16(row, off + 64u * h + 16u * c);
@@ -186,6 +196,9 @@ __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_K> &x, const uint32_t *l
 #pragma unroll
     for (int c = 0; c < 4; c++) { x.h[c] = XH[c * U + u]; x.l[c] = XL[c * U + u]; }
     x.sv = reinterpret_cast<const float4 *>(lds + K / 2)[u];
+}
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q5_K> &x, const uint32_t *lds, int u, int U, int K) {
+    load_x(static_cast<XRegs<RT_GGML_Q4_K> &>(x), lds, u, U, K);
 }
 __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q6_K> &x, const uint32_t *lds, int u, int U, int K) {
     const uint4 *XH = reinterpret_cast<const uint4 *>(lds);
@@ -241,6 +254,46 @@ __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_K> &w, const XR
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         uint32_t lo = q[i] & 0x0f0f0f0fu, hi = (q[i] >> 4) & 0x0f0f0f0fu;
+        dh0 = sdot4(lo, (int)hlo[i], dh0);
+        dl0 = sdot4(lo, (int)llo[i], dl0);
+        dh1 = sdot4(hi, (int)hhi[i], dh1);
+        dl1 = sdot4(hi, (int)lhi[i], dl1);
+    }
+    float t0 = (float)((dh0 << 7) + dl0), t1 = (float)((dh1 << 7) + dl1);
+    const float pos = __builtin_fmaf(sc0, x.sv.x * t0, sc1 * (x.sv.y * t1)), neg = __builtin_fmaf(m0, x.sv.z, m1 * x.sv.w);
+    return __builtin_fmaf(d, pos, -(dmin * neg));
+}
+
+// Q5_K: the Q4_K unit with the fifth bit of every element taken from qh (bit 2g of byte l for the low-nibble
+// sub-block of unit g, bit 2g+1 for the high-nibble one); values 0..31, the -min term as in Q4_K.
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q5_K> &w, const XRegs<RT_GGML_Q5_K> &x, int u) {
+    const int g = u & 3;
+    uint32_t scw, mw;
+    if (g < 2) {
+        scw = w.hdr.y & 0x3f3f3f3fu;
+        mw = w.hdr.z & 0x3f3f3f3fu;
+    } else {
+        scw = (w.hdr.w & 0x0f0f0f0fu) | ((w.hdr.y >> 2) & 0x30303030u);
+        mw = ((w.hdr.w >> 4) & 0x0f0f0f0fu) | ((w.hdr.z >> 2) & 0x30303030u);
+    }
+    const int sh = (g & 1) * 16;
+    scw >>= sh;
+    mw >>= sh;
+    float sc0 = (float)(scw & 0xFF), sc1 = (float)((scw >> 8) & 0xFF);
+    float m0 = (float)(mw & 0xFF), m1 = (float)((mw >> 8) & 0xFF);
+    float d = h2f(w.hdr.x & 0xFFFF), dmin = h2f(w.hdr.x >> 16);
+    const uint32_t q[8] = { w.qa.x, w.qa.y, w.qa.z, w.qa.w, w.qb.x, w.qb.y, w.qb.z, w.qb.w };
+    const uint32_t hb[8] = { w.ha.x, w.ha.y, w.ha.z, w.ha.w, w.hb.x, w.hb.y, w.hb.z, w.hb.w };
+    const uint32_t hlo[8] = { x.h[0].x, x.h[0].y, x.h[0].z, x.h[0].w, x.h[1].x, x.h[1].y, x.h[1].z, x.h[1].w };
+    const uint32_t hhi[8] = { x.h[2].x, x.h[2].y, x.h[2].z, x.h[2].w, x.h[3].x, x.h[3].y, x.h[3].z, x.h[3].w };
+    const uint32_t llo[8] = { x.l[0].x, x.l[0].y, x.l[0].z, x.l[0].w, x.l[1].x, x.l[1].y, x.l[1].z, x.l[1].w };
+    const uint32_t lhi[8] = { x.l[2].x, x.l[2].y, x.l[2].z, x.l[2].w, x.l[3].x, x.l[3].y, x.l[3].z, x.l[3].w };
+    int dh0 = 0, dl0 = 0, dh1 = 0, dl1 = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t bits = hb[i] >> (2 * g);      // bit 0 of each byte: fifth bit of the low-nibble element, bit 1: of the high-nibble one
+        uint32_t lo = (q[i] & 0x0f0f0f0fu) | ((bits << 4) & 0x10101010u);
+        uint32_t hi = ((q[i] >> 4) & 0x0f0f0f0fu) | ((bits << 3) & 0x10101010u);
         dh0 = sdot4(lo, (int)hlo[i], dh0);
         dl0 = sdot4(lo, (int)llo[i], dl0);
         dh1 = sdot4(hi, (int)hhi[i], dh1);
@@ -438,6 +491,9 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
     if ((ALLOW_R2 && r2) || P.epi == kEpiSwiglu) {
         switch (P.type) {
         case RT_GGML_Q4_K: gemv_problem<RT_GGML_Q4_K, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        // 80 bytes of registers per row and unit: Q5_K runs one row per step (two would spill); the launcher refuses
+        // the gate / up pair form for it, the caller issues gate and up as two problems and a separate SwiGLU
+        case RT_GGML_Q5_K: gemv_problem<RT_GGML_Q5_K, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q6_K: gemv_problem<RT_GGML_Q6_K, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
@@ -445,6 +501,7 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
     } else {
         switch (P.type) {
         case RT_GGML_Q4_K: gemv_problem<RT_GGML_Q4_K, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q5_K: gemv_problem<RT_GGML_Q5_K, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q6_K: gemv_problem<RT_GGML_Q6_K, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 1, COH>(P, wg, n_wg, m, lds, red); break;

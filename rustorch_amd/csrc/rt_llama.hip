@@ -147,10 +147,20 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
         a.p[0] = make_prob(m->wo[l], m->xq_a, rt::kStageXq, m->x, m->x);
         RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
         memset(&a, 0, sizeof a);
-        a.n = 1;
-        a.p[0] = make_prob(m->wgate[l], m->x, rt::kStageRms, m->g, nullptr);
-        a.p[0].w2 = m->wup[l].dev; a.p[0].epi = rt::kEpiSwiglu; a.p[0].gamma = m->ffn_norm[l]; a.p[0].eps = c.rms_eps;
-        RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
+        if (m->wgate[l].type == m->wup[l].type && m->wgate[l].type != RT_GGML_Q5_K) {
+            a.n = 1;
+            a.p[0] = make_prob(m->wgate[l], m->x, rt::kStageRms, m->g, nullptr);
+            a.p[0].w2 = m->wup[l].dev; a.p[0].epi = rt::kEpiSwiglu; a.p[0].gamma = m->ffn_norm[l]; a.p[0].eps = c.rms_eps;
+            RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
+        } else {
+            // gate and up of different block formats, or of one without the pair form: two problems in one launch, then SwiGLU
+            a.n = 2;
+            a.p[0] = make_prob(m->wgate[l], m->x, rt::kStageRms, m->g, nullptr);
+            a.p[1] = make_prob(m->wup[l], m->x, rt::kStageRms, m->u, nullptr);
+            for (int i = 0; i < 2; i++) { a.p[i].gamma = m->ffn_norm[l]; a.p[i].eps = c.rms_eps; }
+            RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
+            RT_TRY_HIP(ctx, rt::launch_swiglu(s, m->g, m->u, m->g, nullptr, (size_t)c.ffn));
+        }
         memset(&a, 0, sizeof a);
         a.n = 1;
         a.p[0] = make_prob(m->wdown[l], m->g, rt::kStageF32, m->x, m->x);
@@ -167,7 +177,7 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
     return RT_HIP_OK;
 }
 
-bool gemv_type_ok(int t) { return t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_K || t == RT_GGML_Q6_K; }
+bool gemv_type_ok(int t) { return t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_K || t == RT_GGML_Q5_K || t == RT_GGML_Q6_K; }
 
 constexpr size_t kPrefillChunk = 512;     // tokens per pass of the batched prefill
 

@@ -9,6 +9,7 @@
 //   Q4_0 : w0 -> d;  w1,w2 -> the 16 qs bytes verbatim
 //   Q4_K : w0 -> d from u24(r), dmin from u24(r >> 32);  w1 -> 8 scales (byte & 63);
 //          w2 -> 8 mins (byte & 63), packed into the 12-byte field;  w3..w18 -> qs
+//   Q5_K : w0..w2 as Q4_K;  w3..w6 -> qh;  w7..w22 -> qs
 //   Q6_K : w0..w15 -> ql;  w16..w23 -> qh;  w24,w25 -> scales = (byte & 63) - 32;  w26 -> d
 // The block layouts are the public ggml ones; the byte sizes match
 // GGMLType::type_size (example-cli/src/model/formats/gguf.rs:125-144).
@@ -99,6 +100,20 @@ void gen_block(int type, uint64_t key, uint64_t b, double lo, double hi, uint8_t
         }
         pack_q4k_scales(sc, mn, o + 4);
         for (int w = 0; w < 16; w++) put64(o + 16 + 8 * w, mix(base + 3 + w));
+        break;
+    }
+    case RT_GGML_Q5_K: {       // as Q4_K, then 4 words of fifth bits and 16 words of nibbles
+        uint64_t r0 = mix(base);
+        put16(o, scale_f16(lo, hi, u24(r0)));
+        put16(o + 2, scale_f16(lo, hi, u24(r0 >> 32)));
+        uint64_t r1 = mix(base + 1), r2 = mix(base + 2);
+        uint8_t sc[8], mn[8];
+        for (int j = 0; j < 8; j++) {
+            sc[j] = (uint8_t)((r1 >> (8 * j)) & 63);
+            mn[j] = (uint8_t)((r2 >> (8 * j)) & 63);
+        }
+        pack_q4k_scales(sc, mn, o + 4);
+        for (int w = 0; w < 20; w++) put64(o + 16 + 8 * w, mix(base + 3 + w));
         break;
     }
     case RT_GGML_Q6_K: {

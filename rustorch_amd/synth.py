@@ -18,6 +18,7 @@ D_RANGE = {
     GGMLType.Q8_0: (1e-4, 2e-3),
     GGMLType.Q4_0: (1e-3, 2e-2),
     GGMLType.Q4_K: (1e-3, 1e-2),
+    GGMLType.Q5_K: (1e-3, 1e-2),
     GGMLType.Q6_K: (1e-3, 1e-2),
 }
 

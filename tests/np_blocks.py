@@ -1,4 +1,4 @@
-"""Independent NumPy decoders / encoders of the four GGML block formats.
+"""Independent NumPy decoders / encoders of the GGML block formats the kernels read.
 
 Written from the element's point of view (which byte and which bits hold
 element e), not as the grouped loops the C oracle uses, so an indexing mistake
@@ -56,6 +56,23 @@ def decode_q4_k(blk: np.ndarray) -> np.ndarray:
     return out
 
 
+def decode_q5_k(blk: np.ndarray) -> np.ndarray:
+    """{ f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128] }: element e of sub-block j = e // 32 is the nibble of
+    Q4_K plus 16 when bit j of qh[e % 32] is set."""
+    d, dmin = _f16(blk, 0), _f16(blk, 2)
+    out = np.empty(256, dtype=F32)
+    for e in range(256):
+        j = e // 32
+        sc, mn = q4k_scale_min(blk[4:16], j)
+        byte = int(blk[48 + 32 * (j // 2) + e % 32])
+        nib = (byte >> 4) if (j % 2) else (byte & 15)
+        q = nib + (16 if (int(blk[16 + e % 32]) >> j) & 1 else 0)
+        dd = F32(d * F32(sc))
+        mm = F32(dmin * F32(mn))
+        out[e] = F32(F32(dd * F32(q)) - mm)
+    return out
+
+
 def decode_q6_k(blk: np.ndarray) -> np.ndarray:
     d = _f16(blk, 208)
     sc = blk[192:208].view(np.int8)
@@ -72,7 +89,8 @@ def decode_q6_k(blk: np.ndarray) -> np.ndarray:
     return out
 
 
-DECODERS = {8: (34, 32, decode_q8_0), 2: (18, 32, decode_q4_0), 12: (144, 256, decode_q4_k), 14: (210, 256, decode_q6_k)}
+DECODERS = {8: (34, 32, decode_q8_0), 2: (18, 32, decode_q4_0), 12: (144, 256, decode_q4_k), 14: (210, 256, decode_q6_k),
+            13: (176, 256, decode_q5_k)}
 
 
 def decode(ggml_type: int, raw: np.ndarray) -> np.ndarray:
@@ -126,6 +144,20 @@ def encode_q4_k(d, dmin, sc, mn, q) -> np.ndarray:
     blk[4:16] = pack_q4k_scales(sc, mn)
     q = np.asarray(q, dtype=np.uint8).reshape(4, 2, 32)
     blk[16:] = (q[:, 0, :] | (q[:, 1, :] << 4)).reshape(-1)
+    return blk
+
+
+def encode_q5_k(d, dmin, sc, mn, q) -> np.ndarray:
+    """q: 256 values in 0..31."""
+    blk = np.zeros(176, dtype=np.uint8)
+    _put_f16(blk, 0, d)
+    _put_f16(blk, 2, dmin)
+    blk[4:16] = pack_q4k_scales(sc, mn)
+    q = np.asarray(q, dtype=np.uint8).reshape(8, 32)
+    for j in range(8):
+        blk[16:48] |= ((q[j] >> 4) & 1) << j
+    lo = (q & 15).reshape(4, 2, 32)
+    blk[48:] = (lo[:, 0, :] | (lo[:, 1, :] << 4)).reshape(-1)
     return blk
 
 

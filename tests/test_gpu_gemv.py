@@ -18,6 +18,8 @@ SHAPES = {
     "C3_gate": (12, 11008, 4096),
     "C3_v": (14, 4096, 4096),
     "C3_down": (14, 4096, 11008),
+    "q5_k_gate": (13, 11008, 4096),          # not a benchmark configuration: the Q5_K_M files' format, same shapes
+    "q5_k_down": (13, 4096, 11008),
 }
 
 
@@ -49,7 +51,7 @@ def test_gemv_config_shapes_batch1_and_8(ex, orc, name):
     check(yo, y64[:2], wn, x[:2], name + " oracle f32 vs f64")
 
 
-@pytest.mark.parametrize("t", [8, 2, 12, 14])
+@pytest.mark.parametrize("t", [8, 2, 12, 13, 14])
 def test_gemv_edge_inputs(ex, orc, t):
     from rustorch_amd import synth
     be = 32 if t in (8, 2) else 256

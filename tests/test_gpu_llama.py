@@ -174,6 +174,38 @@ def test_long_context_attention_split_over_workgroups(ex, orc, n_heads, n_kv):
     assert np.median(ratios) <= 0.2
 
 
+def test_q5_k_model(ex, orc):
+    """All seven matrices of every layer in Q5_K: one row per GEMV step, gate and up as two problems of one launch
+    followed by the separate SwiGLU (the format has no gate / up pair form), prefill token by token."""
+    from rustorch_amd import llama, synth, GGMLType
+    cfg = dict(n_layers=2, hidden=512, n_heads=4, ffn=1024, vocab=500, max_pos=40)
+    print("llama q5_k", cfg, flush=True)
+    gm = llama.HipLlama(ex, **cfg)
+    om = orc.OracleLlama(**cfg)
+    head = {}
+    for slot, layer, t, r, c, raw in llama.synthetic_tensors(29, cfg["n_layers"], cfg["hidden"], cfg["ffn"], cfg["vocab"]):
+        if layer >= 0 and t != GGMLType.F32:
+            t = GGMLType.Q5_K
+            raw = synth.blocks(t, 29, synth.layer_tid(layer, slot), r, c)
+        gm.upload(slot, layer, t, r, c, raw)
+        om.set_tensor(slot, layer, t, r, c, raw)
+        if slot == "output":
+            head["wn"] = np.linalg.norm(orc.dequant(t, raw, r, c).astype(np.float64), axis=1)
+    toks = synth.tokens(29, synth.TID_PROMPT, 36, cfg["vocab"])
+    want = om.forward(toks, 0)
+    tol = logit_tol(head["wn"], cfg["hidden"])
+    ratios = []
+    for p, t in enumerate(toks[:20]):
+        gm.step(int(t), p)
+        ratios.append(float((np.abs(gm.logits() - want[p]) / tol).max()))
+    gm.reset()
+    gm.prefill(toks[:30], 0)
+    ratios.append(float((np.abs(gm.logits() - want[29]) / tol).max()))
+    ratios = np.array(ratios)
+    print("ratio to the tolerance: median %.3f, max %.2f" % (np.median(ratios), ratios.max()), flush=True)
+    assert np.median(ratios) <= 0.1 and (ratios <= 1).mean() >= 0.9
+
+
 def test_graph_replay_equals_eager_launches(ex, orc):
     """Mode 2 replays the step from a captured graph.  Every replay is checked against the eager launches of mode 1:
     same kernels, same arguments, so logits and picks are equal bit for bit -- with eager work (a cache reset, a

@@ -9,7 +9,7 @@ import pytest
 import np_blocks as nb
 
 GOLDEN = Path(__file__).resolve().parent / "golden" / "blocks_golden.npz"
-TYPES = [8, 2, 12, 14]
+TYPES = [8, 2, 12, 13, 14]
 
 
 def bits(a):
@@ -48,8 +48,8 @@ def test_f32_to_fp16_rne(orc):
 
 def test_block_geometry_matches_reference_type_size(orc):
     # example-cli/src/model/formats/gguf.rs:125-144
-    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 8, 12, 14)] == [4, 2, 18, 34, 144, 210]
-    assert [orc.load().orc_block_elems(t) for t in (2, 8, 12, 14)] == [32, 32, 256, 256]
+    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 8, 12, 13, 14)] == [4, 2, 18, 34, 144, 176, 210]
+    assert [orc.load().orc_block_elems(t) for t in (2, 8, 12, 13, 14)] == [32, 32, 256, 256, 256]
     assert orc.load().orc_row_bytes(12, 4096) == 2304 and orc.load().orc_row_bytes(14, 11008) == 9030
     assert orc.load().orc_row_bytes(12, 100) == 0
 
@@ -132,6 +132,31 @@ def test_q4_k_nibbles_and_positions(orc):
             y = orc.dequant(12, nb.encode_q4_k(1.0, 1.0, sc, np.zeros(8, np.uint8), q), 1, 256)[0]
             want = np.zeros(256, dtype=np.float32); want[e] = 2 * v
             assert np.array_equal(y, want), (e, v)
+
+
+def test_q5_k_values_fifth_bits_and_positions(orc):
+    # one-hot quants: value v (0..31) at element e, scale 2 at e's sub-block only: the nibble, the fifth bit and its
+    # place in qh (bit = sub-block, byte = position in the sub-block) are all exercised
+    for e in (0, 31, 32, 63, 64, 100, 127, 128, 191, 192, 224, 255):
+        for v in range(32):
+            q = np.zeros(256, dtype=np.uint8); q[e] = v
+            sc = np.zeros(8, dtype=np.uint8); sc[e // 32] = 2
+            y = orc.dequant(13, nb.encode_q5_k(1.0, 1.0, sc, np.zeros(8, np.uint8), q), 1, 256)[0]
+            want = np.zeros(256, dtype=np.float32); want[e] = 2 * v
+            assert np.array_equal(y, want), (e, v)
+    # a set fifth bit reaches no other sub-block: all 31s in one sub-block, scale 1 everywhere
+    for j in range(8):
+        q = np.zeros(256, dtype=np.uint8); q[32 * j:32 * j + 32] = 31
+        y = orc.dequant(13, nb.encode_q5_k(1.0, 1.0, np.ones(8, np.uint8), np.zeros(8, np.uint8), q), 1, 256)[0]
+        want = np.zeros(256, dtype=np.float32); want[32 * j:32 * j + 32] = 31
+        assert np.array_equal(y, want), j
+    # scales and mins go through the Q4_K packer: d * sc * q - dmin * m with every field distinct
+    d, dmin = np.float32(np.float16(0.5)), np.float32(np.float16(0.25))
+    sc = np.array([1, 7, 13, 22, 35, 41, 56, 63], dtype=np.uint8); mn = np.array([63, 50, 44, 31, 20, 9, 3, 0], dtype=np.uint8)
+    q = (np.arange(256) * 7 % 32).astype(np.uint8)
+    y = orc.dequant(13, nb.encode_q5_k(0.5, 0.25, sc, mn, q), 1, 256)[0]
+    want = (d * np.repeat(sc, 32).astype(np.float32)) * q.astype(np.float32) - dmin * np.repeat(mn, 32).astype(np.float32)
+    assert np.array_equal(y, want.astype(np.float32))
 
 
 def test_q6_k_all_values_all_positions(orc):

@@ -43,12 +43,17 @@ def ref_block(t, seed, tid, b, lo, hi):
         sc = w[1:2].view(np.uint8) & 63
         mn = w[2:3].view(np.uint8) & 63
         return np.concatenate([scale(lo, hi, w[0]), scale(lo, hi, int(w[0]) >> 32), nb.pack_q4k_scales(sc, mn), w[3:].view(np.uint8)])
+    if t == 13:
+        w = words(seed, tid, b, 23)
+        sc = w[1:2].view(np.uint8) & 63
+        mn = w[2:3].view(np.uint8) & 63
+        return np.concatenate([scale(lo, hi, w[0]), scale(lo, hi, int(w[0]) >> 32), nb.pack_q4k_scales(sc, mn), w[3:].view(np.uint8)])
     w = words(seed, tid, b, 27)
     sc = ((w[24:26].view(np.uint8) & 63).astype(np.int32) - 32).astype(np.int8).view(np.uint8)
     return np.concatenate([w[:24].view(np.uint8), sc, scale(lo, hi, w[26])])
 
 
-@pytest.mark.parametrize("t", [8, 2, 12, 14])
+@pytest.mark.parametrize("t", [8, 2, 12, 13, 14])
 def test_blocks_follow_the_specification(lib, t):
     from rustorch_amd import synth, GGMLType
     lo, hi = synth.D_RANGE[GGMLType(t)]
