@@ -22,7 +22,7 @@
  * What the reference does NOT hold and this file therefore owns (parity with
  * the reference is unpinned for these; they are pinned by closed forms,
  * exhaustive packer round trips and an independent NumPy decoder in tests/):
- *   - the Q8_0 / Q4_0 / Q4_K / Q6_K block decoders.  The reference only fixes
+ *   - the Q8_0 / Q4_0 / Q4_K / Q5_K / Q6_K block decoders.  The reference only fixes
  *     type ids and block byte sizes (example-cli/src/model/formats/gguf.rs:78-144)
  *     and decodes every quantized type with a placeholder
  *     (tensor_loader.rs:125-141,213-218).  The layouts below are the public
