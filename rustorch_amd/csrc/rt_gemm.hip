@@ -729,6 +729,8 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 
 // workspace: fp16 X, one f32 per row of X, and the partial planes of a k-split launch
+bool qgemm_on_matrix_cores(int type, size_t M, size_t N, size_t K) { return mfma_path(type, N, K, M); }
+
 size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K) {
     if (!mfma_path(type, N, K, M)) return 0;
     GemmPlan p = gemm_plan(M, N, K);

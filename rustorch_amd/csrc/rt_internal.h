@@ -154,6 +154,8 @@ hipError_t launch_qgemm(hipStream_t s, int type, const uint8_t *w, size_t N, siz
                         const float *X, size_t M, float *Y, const float *res, void *scratch, size_t scratch_bytes,
                         bool x_prepared = false);
 size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K);
+// true: launch_qgemm runs the matrix-core contraction (with its pre-pass of X); false: the GEMV kernel, one grid slice per row of X
+bool qgemm_on_matrix_cores(int type, size_t M, size_t N, size_t K);
 
 inline size_t type_block_bytes(int t) {
     switch (t) {

@@ -181,15 +181,9 @@ bool gemv_type_ok(int t) { return t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t ==
 
 constexpr size_t kPrefillChunk = 512;     // tokens per pass of the batched prefill
 
-// The dense-contraction path serves a layer when all seven matrices are Q4_K / Q6_K with whole super-blocks.
-bool prefill_batchable(const rt_hip_llama *m) {
-    auto ok = [](const rt_hip_llama::T &t) {
-        return (t.type == RT_GGML_Q4_K || t.type == RT_GGML_Q6_K) && t.n_cols % 256 == 0 && t.n_rows % 4 == 0;
-    };
-    for (int l = 0; l < m->cfg.n_layers; l++)
-        if (!(ok(m->wq[l]) && ok(m->wk[l]) && ok(m->wv[l]) && ok(m->wo[l]) && ok(m->wgate[l]) && ok(m->wup[l]) && ok(m->wdown[l]))) return false;
-    return m->head_dim == 64 || m->head_dim == 128;
-}
+// The batched prefill serves every block format: Q4_K / Q6_K matrices go to the matrix cores, the others run the GEMV
+// kernel with one grid slice per token (weights found in L2 / Infinity Cache after the first).
+bool prefill_batchable(const rt_hip_llama *m) { return m->head_dim == 64 || m->head_dim == 128; }
 
 int ensure_prefill_buffers(rt_hip_ctx *ctx, rt_hip_llama *m, size_t n_tok) {
     if (m->pf_cap >= n_tok) return RT_HIP_OK;
@@ -205,12 +199,19 @@ int ensure_prefill_buffers(rt_hip_ctx *ctx, rt_hip_llama *m, size_t n_tok) {
     return RT_HIP_OK;
 }
 
-// same_x: X is the matrix the previous call was given, its pre-pass is still in the workspace
-int gemm(rt_hip_ctx *ctx, const rt_hip_llama::T &t, const float *X, size_t M, float *Y, const float *res, bool same_x = false) {
-    RT_TRY_HIP(ctx, rt::launch_qgemm(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, X, M, Y, res, ctx->scratch, ctx->scratch_bytes,
-                                     same_x));
-    return RT_HIP_OK;
-}
+// The contractions of one prefill pass.  Consecutive weights that meet the same activation matrix on the matrix cores
+// share its pre-pass, which stays in the workspace until another matrix is prepared.
+struct PrefillGemm {
+    rt_hip_ctx *ctx;
+    const float *prepared = nullptr;
+    int operator()(const rt_hip_llama::T &t, const float *X, size_t M, float *Y, const float *res) {
+        const bool mc = rt::qgemm_on_matrix_cores(t.type, M, t.n_rows, t.n_cols) && res != Y;
+        RT_TRY_HIP(ctx, rt::launch_qgemm(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, X, M, Y, res, ctx->scratch, ctx->scratch_bytes,
+                                         mc && prepared == X));
+        if (mc) prepared = X;
+        return RT_HIP_OK;
+    }
+};
 
 // M tokens (already in pf_tok) at positions pos0 .. pos0+M-1 through all layers with the dense contraction:
 // per layer rmsnorm rows -> q,k,v GEMMs -> rope + cache append -> causal attention (query m over pos0+m+1 rows)
@@ -226,24 +227,28 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
     int rc = ensure_scratch(ctx, need);
     if (rc) return rc;
     float *x = m->pf_x, *x2 = m->pf_x2;
+    PrefillGemm gemm{ ctx };
     RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, m->pf_tok, M, c.vocab, x));
     for (int l = 0; l < c.n_layers; l++) {
         uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
         uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->attn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
-        if ((rc = gemm(ctx, m->wq[l], m->pf_n, M, m->pf_q, nullptr))) return rc;
-        if ((rc = gemm(ctx, m->wk[l], m->pf_n, M, m->pf_k, nullptr, true))) return rc;
-        if ((rc = gemm(ctx, m->wv[l], m->pf_n, M, m->pf_v, nullptr, true))) return rc;
+        gemm.prepared = nullptr;          // pf_n has new contents
+        if ((rc = gemm(m->wq[l], m->pf_n, M, m->pf_q, nullptr))) return rc;
+        if ((rc = gemm(m->wk[l], m->pf_n, M, m->pf_k, nullptr))) return rc;
+        if ((rc = gemm(m->wv[l], m->pf_n, M, m->pf_v, nullptr))) return rc;
         RT_TRY_HIP(ctx, rt::launch_rope_kv_batch(s, m->pf_q, m->pf_k, m->pf_v, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
         RT_TRY_HIP(ctx, rt::launch_attn_batch(s, m->pf_q, nullptr, nullptr, kc, vc, nullptr, pos0 + 1, M, c.n_heads, m->n_kv, m->head_dim,
                                               m->inv_freq, m->pf_a, nullptr, false));
-        if ((rc = gemm(ctx, m->wo[l], m->pf_a, M, x2, x))) return rc;
+        if ((rc = gemm(m->wo[l], m->pf_a, M, x2, x))) return rc;
         std::swap(x, x2);
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->ffn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
-        if ((rc = gemm(ctx, m->wgate[l], m->pf_n, M, m->pf_g, nullptr))) return rc;
-        if ((rc = gemm(ctx, m->wup[l], m->pf_n, M, m->pf_u, nullptr, true))) return rc;
+        gemm.prepared = nullptr;
+        if ((rc = gemm(m->wgate[l], m->pf_n, M, m->pf_g, nullptr))) return rc;
+        if ((rc = gemm(m->wup[l], m->pf_n, M, m->pf_u, nullptr))) return rc;
         RT_TRY_HIP(ctx, rt::launch_swiglu(s, m->pf_g, m->pf_u, m->pf_g, nullptr, M * F));
-        if ((rc = gemm(ctx, m->wdown[l], m->pf_g, M, x2, x))) return rc;
+        gemm.prepared = nullptr;          // pf_g is rewritten in place
+        if ((rc = gemm(m->wdown[l], m->pf_g, M, x2, x))) return rc;
         std::swap(x, x2);
     }
     RT_TRY_HIP(ctx, hipMemcpyAsync(m->x, x + (M - 1) * H, H * sizeof(float), hipMemcpyDeviceToDevice, s));

@@ -174,18 +174,20 @@ def test_long_context_attention_split_over_workgroups(ex, orc, n_heads, n_kv):
     assert np.median(ratios) <= 0.2
 
 
-def test_q5_k_model(ex, orc):
-    """All seven matrices of every layer in Q5_K: one row per GEMV step, gate and up as two problems of one launch
-    followed by the separate SwiGLU (the format has no gate / up pair form), prefill token by token."""
+@pytest.mark.parametrize("fmt", ["Q5_K", "Q8_0", "Q4_0"])
+def test_model_in_a_format_without_matrix_core_path(ex, orc, fmt):
+    """All seven matrices of every layer in one format that the dense contraction does not serve.  Decode: the GEMV
+    kernels (Q5_K: one row per step, gate and up as two problems of one launch followed by the separate SwiGLU).
+    Prefill of 16 tokens or more: the batched pipeline with the GEMV kernel run once per token as grid slices."""
     from rustorch_amd import llama, synth, GGMLType
     cfg = dict(n_layers=2, hidden=512, n_heads=4, ffn=1024, vocab=500, max_pos=40)
-    print("llama q5_k", cfg, flush=True)
+    print("llama uniform", fmt, cfg, flush=True)
     gm = llama.HipLlama(ex, **cfg)
     om = orc.OracleLlama(**cfg)
     head = {}
     for slot, layer, t, r, c, raw in llama.synthetic_tensors(29, cfg["n_layers"], cfg["hidden"], cfg["ffn"], cfg["vocab"]):
         if layer >= 0 and t != GGMLType.F32:
-            t = GGMLType.Q5_K
+            t = getattr(GGMLType, fmt)
             raw = synth.blocks(t, 29, synth.layer_tid(layer, slot), r, c)
         gm.upload(slot, layer, t, r, c, raw)
         om.set_tensor(slot, layer, t, r, c, raw)
@@ -195,12 +197,20 @@ def test_q5_k_model(ex, orc):
     want = om.forward(toks, 0)
     tol = logit_tol(head["wn"], cfg["hidden"])
     ratios = []
-    for p, t in enumerate(toks[:20]):
+    for p, t in enumerate(toks[:30]):
         gm.step(int(t), p)
         ratios.append(float((np.abs(gm.logits() - want[p]) / tol).max()))
+    stepped = gm.logits().copy()
     gm.reset()
-    gm.prefill(toks[:30], 0)
-    ratios.append(float((np.abs(gm.logits() - want[29]) / tol).max()))
+    gm.prefill(toks[:30], 0)                                    # batched path
+    batched = gm.logits().copy()
+    ratios.append(float((np.abs(batched - want[29]) / tol).max()))
+    assert float((np.abs(batched - stepped) / tol).max()) <= 0.1 # the two device paths agree far inside the bound
+    gm.step(int(toks[30]), 30)                                  # the cache the batched path left serves the decode step
+    ratios.append(float((np.abs(gm.logits() - want[30]) / tol).max()))
+    gm.reset()
+    gm.prefill(toks[:10], 0)                                    # under 16 tokens: token by token
+    assert float((np.abs(gm.logits() - want[9]) / tol).max()) <= 1.0
     ratios = np.array(ratios)
     print("ratio to the tolerance: median %.3f, max %.2f" % (np.median(ratios), ratios.max()), flush=True)
     assert np.median(ratios) <= 0.1 and (ratios <= 1).mean() >= 0.9
