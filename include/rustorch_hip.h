@@ -172,6 +172,12 @@ RT_HIP_API int rt_hip_kv_append_dev(rt_hip_ctx *ctx, uint16_t *cache, const floa
  * (example-cli/src/model/architectures/attention.rs:233-338 for a single query row). */
 RT_HIP_API int rt_hip_attn_decode_dev(rt_hip_ctx *ctx, const float *q, const uint16_t *kcache,
                                       const uint16_t *vcache, int n_pos, int n_heads, int head_dim, float *out);
+/* A batch of consecutive positions with the causal mask: row m of q[n_queries][n_heads * head_dim] (position
+ * pos0 + m) attends cache rows [0, pos0 + m] (the masked scores / softmax / weighted sum of
+ * example-cli/src/model/architectures/attention.rs:233-338 over the cache).  Cache rows hold n_kv_heads heads
+ * (0 = n_heads); query head h reads head h / (n_heads / n_kv_heads).  All pointers 16-byte aligned. */
+RT_HIP_API int rt_hip_attn_causal_dev(rt_hip_ctx *ctx, const float *q, const uint16_t *kcache, const uint16_t *vcache,
+                                      int pos0, int n_queries, int n_heads, int n_kv_heads, int head_dim, float *out);
 /* x += y : the residual adds of GPTBlock::forward (example-cli/src/model/architectures/gpt.rs:43-55). */
 RT_HIP_API int rt_hip_add_dev(rt_hip_ctx *ctx, float *x, const float *y, size_t n);
 /* Greedy pick (SamplingConfig::greedy, example-cli/src/model/sampling.rs:28-35); ties -> lowest index. */

@@ -544,6 +544,22 @@ int rt_hip_attn_decode_dev(rt_hip_ctx *ctx, const float *q, const uint16_t *kcac
     return RT_HIP_OK;
 }
 
+int rt_hip_attn_causal_dev(rt_hip_ctx *ctx, const float *q, const uint16_t *kcache, const uint16_t *vcache, int pos0, int n_queries,
+                           int n_heads, int n_kv_heads, int head_dim, float *out) {
+    if (!ctx || !q || !kcache || !vcache || !out) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_attn_causal_dev: NULL argument");
+    if (n_kv_heads == 0) n_kv_heads = n_heads;
+    RT_REQUIRE(ctx, head_dim == 64 || head_dim == 128, RT_HIP_ERR_SHAPE, "attn_causal: head_dim=%d (64 or 128 supported)", head_dim);
+    RT_REQUIRE(ctx, n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, RT_HIP_ERR_SHAPE, "attn_causal: n_heads=%d n_kv_heads=%d",
+               n_heads, n_kv_heads);
+    RT_REQUIRE(ctx, pos0 >= 0 && n_queries > 0 && (long long)pos0 + n_queries <= (1 << 24), RT_HIP_ERR_SHAPE, "attn_causal: pos0=%d n_queries=%d",
+               pos0, n_queries);
+    RT_REQUIRE(ctx, (((uintptr_t)q | (uintptr_t)kcache | (uintptr_t)vcache | (uintptr_t)out) & 15) == 0, RT_HIP_ERR_INVALID_ARG,
+               "attn_causal: operands must be 16-byte aligned");
+    Guard g(ctx);
+    RT_TRY_HIP(ctx, rt::launch_attn_causal(ctx->stream, q, kcache, vcache, pos0, (size_t)n_queries, n_heads, n_kv_heads, head_dim, out));
+    return RT_HIP_OK;
+}
+
 int rt_hip_add_dev(rt_hip_ctx *ctx, float *x, const float *y, size_t n) {
     if (!ctx || !x || !y) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_add_dev: NULL argument");
     Guard g(ctx);

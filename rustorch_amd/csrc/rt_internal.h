@@ -137,6 +137,9 @@ hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const f
 hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
                              const int *pos_dev, int n_pos, size_t n_queries, int n_heads, int n_kv_heads, int head_dim,
                              const float *inv_freq_dev, float *out, uint8_t *xq, bool fused);
+// rows m = 0 .. n_queries-1 of q (position pos0 + m) attend cache rows [0, pos0 + m]; matrix-core kernel, one wave per 32 queries of a head
+hipError_t launch_attn_causal(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc, int pos0, size_t n_queries,
+                              int n_heads, int n_kv_heads, int head_dim, float *out);
 hipError_t launch_embed_rows(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,
                              const int *tokens_dev, size_t n_tok, int vocab, float *out);
 hipError_t launch_add(hipStream_t s, float *x, const float *y, size_t n);

@@ -238,8 +238,7 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
         if ((rc = gemm(m->wk[l], m->pf_n, M, m->pf_k, nullptr))) return rc;
         if ((rc = gemm(m->wv[l], m->pf_n, M, m->pf_v, nullptr))) return rc;
         RT_TRY_HIP(ctx, rt::launch_rope_kv_batch(s, m->pf_q, m->pf_k, m->pf_v, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
-        RT_TRY_HIP(ctx, rt::launch_attn_batch(s, m->pf_q, nullptr, nullptr, kc, vc, nullptr, pos0 + 1, M, c.n_heads, m->n_kv, m->head_dim,
-                                              m->inv_freq, m->pf_a, nullptr, false));
+        RT_TRY_HIP(ctx, rt::launch_attn_causal(s, m->pf_q, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->pf_a));
         if ((rc = gemm(m->wo[l], m->pf_a, M, x2, x))) return rc;
         std::swap(x, x2);
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->ffn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));

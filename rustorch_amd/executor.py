@@ -308,6 +308,23 @@ class HipKernelExecutor:
         _lib.check(self.lib.rt_hip_attn_decode_dev(self.ctx, dq.ptr, dk.ptr, dv.ptr, n_pos, n_heads, head_dim, do.ptr), self.ctx)
         return do.download(np.float32)
 
+    def attn_causal(self, q, kcache_f16: np.ndarray, vcache_f16: np.ndarray, pos0: int, n_heads: int, head_dim: int,
+                    n_kv_heads: int = 0) -> np.ndarray:
+        """q[n_queries, n_heads * head_dim]: row m sits at position pos0 + m and attends cache rows [0, pos0 + m]."""
+        q = _f32(q, "q")
+        row, rowkv = n_heads * head_dim, (n_kv_heads or n_heads) * head_dim
+        if q.ndim != 2 or q.shape[1] != row or q.shape[0] == 0:
+            raise ShapeMismatch("attn_causal: q must be [n_queries, %d]" % row)
+        n_pos = pos0 + q.shape[0]
+        if kcache_f16.size < n_pos * rowkv or vcache_f16.size < n_pos * rowkv:
+            raise ShapeMismatch("attn_causal: the caches hold fewer than %d rows of %d" % (n_pos, rowkv))
+        dq = self.to_device(q)
+        dk = self.to_device(np.ascontiguousarray(kcache_f16).view(np.uint16))
+        dv = self.to_device(np.ascontiguousarray(vcache_f16).view(np.uint16))
+        do = self.buffer(q.size * 4)
+        _lib.check(self.lib.rt_hip_attn_causal_dev(self.ctx, dq.ptr, dk.ptr, dv.ptr, pos0, q.shape[0], n_heads, n_kv_heads, head_dim, do.ptr), self.ctx)
+        return do.download(np.float32).reshape(q.shape)
+
     def kv_append(self, cache: DeviceBuffer, v, pos: int) -> None:
         v = _f32(v, "v")
         dv = self.to_device(v)

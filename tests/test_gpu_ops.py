@@ -68,6 +68,42 @@ def test_kv_append_and_attention(ex, orc):
         assert not d.download(np.uint16)[:8].any()
 
 
+@pytest.mark.parametrize("nh,nkv,hd,pos0,m", [(4, 4, 64, 0, 37), (32, 32, 128, 0, 70), (8, 2, 128, 100, 45), (2, 1, 128, 1000, 33),
+                                               (6, 3, 64, 31, 1), (3, 3, 128, 0, 129)])
+def test_causal_attention_of_a_batch(ex, orc, nh, nkv, hd, pos0, m):
+    """Row i of the batch (position pos0 + i) against the single-query oracle over cache rows [0, pos0 + i]."""
+    from rustorch_amd import synth
+    print("causal attention", nh, nkv, hd, pos0, m, flush=True)
+    row, rowkv, n_pos = nh * hd, nkv * hd, pos0 + m
+    K = synth.normal(15, n_pos, n_pos * rowkv).reshape(n_pos, rowkv)
+    V = synth.normal(16, n_pos, n_pos * rowkv).reshape(n_pos, rowkv) * 10
+    q = synth.normal(17, n_pos, m * row).reshape(m, row) * 3
+    q[m // 2] *= 1e-6                                              # a query of tiny magnitude, and one of zeros
+    if m > 2:
+        q[1] = 0
+    kc = K.astype(np.float16).view(np.uint16); vc = V.astype(np.float16).view(np.uint16)
+    got = ex.attn_causal(q, kc, vc, pos0, nh, hd, nkv)
+    assert got.shape == (m, row) and np.isfinite(got).all()
+    for i in range(m):
+        want = orc.attn_decode(q[i], kc, vc, pos0 + i + 1, nh, hd, nkv)
+        assert np.allclose(got[i], want, rtol=2e-5, atol=2e-5 * np.abs(V).max()), "query %d" % i
+    # a shorter batch over caches that end at its last position: same rows, bit for bit, and nothing is read past the end
+    h = m // 2
+    got2 = ex.attn_causal(q[:h + 1], kc[:pos0 + h + 1], vc[:pos0 + h + 1], pos0, nh, hd, nkv)
+    assert np.array_equal(got2, got[:h + 1])
+
+
+def test_causal_attention_rejects_bad_shapes(ex):
+    from rustorch_amd import ShapeMismatch
+    q = np.zeros((4, 2 * 64), np.float32); c = np.zeros((4, 2 * 64), np.uint16)
+    with pytest.raises(ShapeMismatch):
+        ex.attn_causal(q, c[:3], c, 0, 2, 64)                     # cache shorter than the positions
+    with pytest.raises(ShapeMismatch):
+        ex.attn_causal(q, c, c, 0, 3, 64)                         # row width does not match
+    with pytest.raises(ShapeMismatch):
+        ex.attn_causal(np.zeros((4, 3 * 96), np.float32), np.zeros((4, 3 * 96), np.uint16), np.zeros((4, 3 * 96), np.uint16), 0, 3, 96)
+
+
 def test_attention_dominant_and_uniform_keys(ex, orc):
     nh, hd, n = 32, 128, 64
     row = nh * hd
