@@ -4,8 +4,10 @@
 // (example-cli/src/model/architectures/attention.rs:233-338: the masked scores, softmax and weighted sum of a
 // whole sequence; here the keys and values are the cache rows, as in the decode step).
 //
-// One wave per workgroup: 32 consecutive queries of one head against tiles of 32 cache rows, flash style (running
-// maximum and sum per query, accumulated output rescaled when the maximum moves).  Both products run on
+// One workgroup per 32 consecutive queries of one head, against tiles of 32 cache rows, flash style (running maximum
+// and sum per query, accumulated output rescaled when the maximum moves).  The four waves of the workgroup take the
+// tiles in turn (wave w: tiles w, w + 4, ...), each with its own running state and its own LDS tile, and never meet
+// before the end, where the four partial results {max, sum, output} are folded through LDS.  Both products run on
 // v_mfma_f32_32x32x16_f16 with the f32 operand split into two fp16 terms (value = hi + lo, both exact in the f32
 // accumulation), so the result keeps f32-level accuracy:
 //   S^T[key][query] = K . (Qhi + Qlo)^T    the lane's 16 scores belong to ONE query (lane % 32): its maximum and sum
@@ -24,17 +26,31 @@ typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+constexpr int kAttnWaves = 4;
+
+// Orders the LDS traffic of ONE wave (a tile written by all its lanes, then read across lanes).  The hardware runs a
+// wave's LDS instructions in order; this keeps the compiler from moving them across the point.  Not a workgroup
+// barrier: the waves of a workgroup run different numbers of tiles.
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 template <int HD>
-__global__ __launch_bounds__(64) void attn_causal_kernel(const float *q, const uint16_t *kc, const uint16_t *vc, int pos0, int M,
+__global__ __launch_bounds__(64 * kAttnWaves) void attn_causal_kernel(const float *q, const uint16_t *kc, const uint16_t *vc, int pos0, int M,
                                                          int n_heads, int n_kv_heads, float *out) {
     constexpr int KK = HD / 16;           // 16-wide steps of the score product
     constexpr int DB = HD / 32;           // 32-row blocks of the head dimension in the output product
     constexpr int VS = HD + 8;            // halves per value row in LDS (16-byte aligned, rows 4 apart fall on different banks)
     constexpr int CPR = HD / 8;           // 16-byte chunks per cache row of one head
     constexpr int VL = 32 * CPR / 64;     // 16-byte loads per lane for a tile of 32 value rows
-    __shared__ __align__(16) uint16_t vs[32 * VS];
+    constexpr int W = kAttnWaves;
+    constexpr int PS = 2 * 16 + 4;        // floats per lane of a fold round: two accumulator blocks, max, sum (padded to 16 bytes)
+    constexpr int kTileBytes = W * 32 * VS * 2, kPartBytes = W * 64 * PS * 4;
+    __shared__ __align__(16) uint8_t lds[kTileBytes > kPartBytes ? kTileBytes : kPartBytes];    // the partials reuse the tiles' space
 
-    const int lane = threadIdx.x, j = lane & 31, hh = lane >> 5;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), j = lane & 31, hh = lane >> 5;
+    uint16_t *vs = reinterpret_cast<uint16_t *>(lds) + wave * 32 * VS;
     const int h = blockIdx.x, qb = blockIdx.y;
     const int group = n_heads / n_kv_heads, kvh = h / group;
     const size_t row = (size_t)n_heads * HD, rowkv = (size_t)n_kv_heads * HD;
@@ -91,7 +107,7 @@ __global__ __launch_bounds__(64) void attn_causal_kernel(const float *q, const u
             vn[i] = *reinterpret_cast<const u32x4 *>(vbase + (size_t)vkey * rowkv + 8 * (c % CPR));
         }
     };
-    request(0);
+    request(min(wave, T - 1));
 
     float16v acc[DB];
 #pragma unroll
@@ -101,18 +117,18 @@ __global__ __launch_bounds__(64) void attn_causal_kernel(const float *q, const u
     float m_run = -INFINITY, l_run = 0.f;
     const _Float16 *vsh = reinterpret_cast<const _Float16 *>(vs);
 
-    for (int t = 0; t < T; t++) {
+    for (int t = wave; t < T; t += W) {
         half8v kcur[KK];
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) kcur[kk] = kn[kk];
-        __syncthreads();                                      // the previous tile's value reads are done
+        wave_lds_fence();                                     // the previous tile's value reads come first
 #pragma unroll
         for (int i = 0; i < VL; i++) {
             const int c = i * 64 + lane;
             *reinterpret_cast<u32x4 *>(vs + (c / CPR) * VS + 8 * (c % CPR)) = vn[i];
         }
-        request(min(t + 1, T - 1));                          // the last tile requests itself again: no branch around the loads
-        __syncthreads();
+        request(min(t + W, T - 1));                          // past the end a tile is requested again: no branch around the loads
+        wave_lds_fence();
 
         // scores: register r of lane (j, hh) is key 8 (r / 4) + 4 hh + r % 4 of the tile against query j
         float16v s;
@@ -165,16 +181,53 @@ __global__ __launch_bounds__(64) void attn_causal_kernel(const float *q, const u
             }
     }
 
-    // ---- register r of lane (j, hh) is element 32 db + 8 (r / 4) + 4 hh + r % 4 of query j's output
-    if (m < M) {
-        const float inv = 1.0f / (l_run * 16384.0f);
-        float *op = out + (size_t)m * row + (size_t)h * HD + 4 * hh;
+    // ---- fold the waves' partial results, two 32-element blocks of the head dimension per round; in a round wave w
+    // finishes half of block (w & 1).  Register r of lane (j, hh) is element 32 db + 8 (r / 4) + 4 hh + r % 4 of query j.
+    float *part = reinterpret_cast<float *>(lds);
+    float *mine = part + (size_t)(wave * 64 + lane) * PS;
+    float fw[W], inv = 0.f;
 #pragma unroll
-        for (int db = 0; db < DB; db++)
+    for (int c = 0; c < DB / 2; c++) {
+        __syncthreads();                                      // the tiles (first round) or the previous round's reads are done
+#pragma unroll
+        for (int b = 0; b < 2; b++)
 #pragma unroll
             for (int g = 0; g < 4; g++)
-                *reinterpret_cast<float4 *>(op + 32 * db + 8 * g) =
-                    make_float4(acc[db][4 * g] * inv, acc[db][4 * g + 1] * inv, acc[db][4 * g + 2] * inv, acc[db][4 * g + 3] * inv);
+                *reinterpret_cast<float4 *>(mine + 16 * b + 4 * g) =
+                    make_float4(acc[2 * c + b][4 * g], acc[2 * c + b][4 * g + 1], acc[2 * c + b][4 * g + 2], acc[2 * c + b][4 * g + 3]);
+        if (c == 0) *reinterpret_cast<float2 *>(mine + 32) = make_float2(m_run, l_run);
+        __syncthreads();
+        if (c == 0) {
+            float lw[W], m_all = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < W; w++) {
+                const float2 ml = *reinterpret_cast<const float2 *>(part + (size_t)(w * 64 + lane) * PS + 32);
+                fw[w] = ml.x;
+                lw[w] = ml.y;
+                m_all = fmaxf(m_all, ml.x);                   // finite: wave 0 always has tile 0
+            }
+            float l_all = 0.f;
+#pragma unroll
+            for (int w = 0; w < W; w++) {
+                fw[w] = expf(fw[w] - m_all);                  // a wave without tiles reports max = -inf: factor 0
+                l_all += lw[w] * fw[w];
+            }
+            inv = 1.0f / (l_all * 16384.0f);
+        }
+        const int b = wave & 1, db = 2 * c + b;
+#pragma unroll
+        for (int gi = 0; gi < 2; gi++) {
+            const int g = 2 * (wave >> 1) + gi;
+            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int w = 0; w < W; w++) {
+                const float4 a = *reinterpret_cast<const float4 *>(part + (size_t)(w * 64 + lane) * PS + 16 * b + 4 * g);
+                o.x += a.x * fw[w]; o.y += a.y * fw[w]; o.z += a.z * fw[w]; o.w += a.w * fw[w];
+            }
+            if (m < M)
+                *reinterpret_cast<float4 *>(out + (size_t)m * row + (size_t)h * HD + 4 * hh + 32 * db + 8 * g) =
+                    make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
+        }
     }
 }
 
@@ -190,9 +243,9 @@ hipError_t launch_attn_causal(hipStream_t s, const float *q, const uint16_t *kc,
     if (((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc | (uintptr_t)out) & 15) return hipErrorInvalidValue;
     const dim3 grid((unsigned)n_heads, (unsigned)((n_queries + 31) / 32));
     if (head_dim == 128)
-        attn_causal_kernel<128><<<grid, 64, 0, s>>>(q, kc, vc, pos0, (int)n_queries, n_heads, n_kv_heads, out);
+        attn_causal_kernel<128><<<grid, 64 * kAttnWaves, 0, s>>>(q, kc, vc, pos0, (int)n_queries, n_heads, n_kv_heads, out);
     else
-        attn_causal_kernel<64><<<grid, 64, 0, s>>>(q, kc, vc, pos0, (int)n_queries, n_heads, n_kv_heads, out);
+        attn_causal_kernel<64><<<grid, 64 * kAttnWaves, 0, s>>>(q, kc, vc, pos0, (int)n_queries, n_heads, n_kv_heads, out);
     return hipGetLastError();
 }
 
