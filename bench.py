@@ -33,7 +33,7 @@ HBM_PEAK = 8.0e12
 # HBM bytes one launch of the GEMV kernel moves on this workload, from the FETCH_SIZE and WRITE_SIZE hardware
 # counters (each scaled by what the same counter reads for a plain x += y kernel of known size); measured
 # offline with the profiler, since counters cannot be read from inside this process.
-GEMV_TRAFFIC_BYTES = 131_770_000
+GEMV_TRAFFIC_BYTES = 131_800_000
 SEED = 20250127
 H, F, V, NH, NL = 4096, 11008, 32000, 32, 32
 
