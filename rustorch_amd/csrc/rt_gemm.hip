@@ -107,6 +107,109 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float *X, size_t K, _F
     }
 }
 
+// ---- the pre-pass fused with the operation that produces the activation matrix.  A thread keeps its groups of the
+// row in registers from the first read to the conversion (rows of up to 256 * kXprepChunks * 8 elements).
+__device__ __forceinline__ void plane_load8(const PlaneSum &p, size_t off, float *v) {
+    const float4 a = *reinterpret_cast<const float4 *>(p.base + off), b = *reinterpret_cast<const float4 *>(p.base + off + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    for (int z = 1; z < p.n; z++) {
+        const float4 c = *reinterpret_cast<const float4 *>(p.base + (size_t)z * p.stride + off),
+                     d = *reinterpret_cast<const float4 *>(p.base + (size_t)z * p.stride + off + 4);
+        v[0] += c.x; v[1] += c.y; v[2] += c.z; v[3] += c.w; v[4] += d.x; v[5] += d.y; v[6] += d.z; v[7] += d.w;
+    }
+}
+
+struct RowSrc {
+    PlaneSum a, b;          // rmsnorm: a = the matrix; swiglu: a = gate, b = up
+    const float *res;       // rmsnorm: added to a (optional)
+    float *x_out;           // rmsnorm: a + res is stored here (optional)
+    const float *gamma;
+    float eps;
+};
+
+constexpr int kPrepRms = 1, kPrepSwiglu = 2;
+
+template <int MODE>
+__global__ __launch_bounds__(256) void xprep_fused_kernel(RowSrc S, size_t K, _Float16 *Xp, float *inv_scale) {
+    __shared__ float red[4];
+    const size_t m = blockIdx.x, n_chunks = K / 8;
+    auto src_of = [](size_t g) {
+        const int sh = (int)(g & 7), s = sh >> 1, h = sh & 1;
+        return 64 * (g >> 3) + 32 * (size_t)(s >> 1) + 16 * (size_t)h + 8 * (size_t)(s & 1);
+    };
+    float v[kXprepChunks][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < kXprepChunks; j++) {
+        const size_t g = threadIdx.x + 256 * (size_t)j;
+        if (g < n_chunks) {
+            const size_t off = m * K + src_of(g);
+            if (MODE == kPrepRms) {
+                plane_load8(S.a, off, v[j]);
+                if (S.res) {
+                    const float4 a = *reinterpret_cast<const float4 *>(S.res + off), b = *reinterpret_cast<const float4 *>(S.res + off + 4);
+                    v[j][0] += a.x; v[j][1] += a.y; v[j][2] += a.z; v[j][3] += a.w; v[j][4] += b.x; v[j][5] += b.y; v[j][6] += b.z; v[j][7] += b.w;
+                }
+                if (S.x_out) {
+                    *reinterpret_cast<float4 *>(S.x_out + off) = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
+                    *reinterpret_cast<float4 *>(S.x_out + off + 4) = make_float4(v[j][4], v[j][5], v[j][6], v[j][7]);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) ss += v[j][e] * v[j][e];
+            } else {
+                float gt[8], up[8];
+                plane_load8(S.a, off, gt);
+                plane_load8(S.b, off, up);
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[j][e] = up[e] * (gt[e] * (1.0f / (1.0f + expf(-gt[e]))));
+            }
+        }
+    }
+    if (MODE == kPrepRms) {
+        ss = block_sum(ss, red);
+        const float rms = sqrtf(ss / (float)K + S.eps);
+#pragma unroll
+        for (int j = 0; j < kXprepChunks; j++) {
+            const size_t g = threadIdx.x + 256 * (size_t)j;
+            if (g < n_chunks) {
+                const float *gp = S.gamma + src_of(g);
+                const float4 a = *reinterpret_cast<const float4 *>(gp), b = *reinterpret_cast<const float4 *>(gp + 4);
+                const float gm[8] = { a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w };
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[j][e] = gm[e] * (v[j][e] / rms);
+            }
+        }
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < kXprepChunks; j++) {
+        const size_t g = threadIdx.x + 256 * (size_t)j;
+        if (g < n_chunks)
+#pragma unroll
+            for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[j][e]));
+    }
+    amax = block_max(amax, red);
+    int ex = 0;
+    float scale = 1.f, inv = 1.f;
+    if (amax > 0.f && amax < INFINITY) {
+        (void)frexpf(amax, &ex);                // amax = f * 2^ex, f in [0.5, 1)
+        int se = 15 - ex;
+        se = se > 100 ? 100 : (se < -100 ? -100 : se);
+        scale = ldexpf(1.f, se);
+        inv = ldexpf(1.f, -se);
+    }
+    if (threadIdx.x == 0) inv_scale[m] = inv;
+#pragma unroll
+    for (int j = 0; j < kXprepChunks; j++) {
+        const size_t g = threadIdx.x + 256 * (size_t)j;
+        if (g < n_chunks) {
+            half8v o = { (_Float16)(v[j][0] * scale), (_Float16)(v[j][2] * scale), (_Float16)(v[j][1] * scale), (_Float16)(v[j][3] * scale),
+                         (_Float16)(v[j][4] * scale), (_Float16)(v[j][6] * scale), (_Float16)(v[j][5] * scale), (_Float16)(v[j][7] * scale) };
+            *reinterpret_cast<half8v *>(Xp + m * K + 8 * g) = o;
+        }
+    }
+}
+
 // ---- weights of one super-block (256 k) on their way to the lanes that expand them
 //
 // MFMA lane (nl, h) needs bytes of weight row nl only, and rows lie row_bytes apart: loading them lane by
@@ -686,7 +789,7 @@ GemmPlan gemm_plan(size_t M, size_t N, size_t K) {
 
 template <int TYPE, int NW, int MF>
 hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const _Float16 *Xp,
-                      const float *inv_scale, size_t M, float *Y, const float *res, float *partial) {
+                      const float *inv_scale, size_t M, float *Y, const float *res, float *partial, bool reduce) {
     constexpr int BM = 32 * MF, BN = 32 * NW;
     const size_t lds = (size_t)4 * BM * kBK * sizeof(_Float16) + (size_t)NW * WGeo<TYPE>::stage_bytes;
     auto kern = qgemm_kernel<TYPE, NW, MF>;
@@ -705,7 +808,7 @@ hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t
     kern<<<dim3((unsigned)(8 * per_xcd)), 64 * NW, lds, s>>>(w, row_bytes, (int)N, (int)K, Xp, inv_scale, (int)M, p.ksplit > 1 ? partial : Y,
                                                              plane, res, p.sb_per_split, p.ksplit, tiles_n, total, per_xcd);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || p.ksplit == 1) return e;
+    if (e != hipSuccess || p.ksplit == 1 || !reduce) return e;
     const size_t n4 = plane / 4;
     const unsigned grid = (unsigned)std::min<size_t>((n4 + 255) / 256, 2048);
     splitk_reduce_kernel<<<grid, 256, 0, s>>>(partial, plane, p.ksplit, res, Y, n4);
@@ -714,9 +817,9 @@ hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t
 
 template <int TYPE>
 hipError_t launch_type(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const _Float16 *Xp,
-                       const float *inv_scale, size_t M, float *Y, const float *res, float *partial) {
-    if (p.mf == 4) return launch_cfg<TYPE, kGemmWaves, 4>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
-    return launch_cfg<TYPE, kGemmWaves, 2>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
+                       const float *inv_scale, size_t M, float *Y, const float *res, float *partial, bool reduce = true) {
+    if (p.mf == 4) return launch_cfg<TYPE, kGemmWaves, 4>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial, reduce);
+    return launch_cfg<TYPE, kGemmWaves, 2>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial, reduce);
 }
 
 bool mfma_path(int type, size_t N, size_t K, size_t M) {
@@ -735,6 +838,51 @@ size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K) {
     if (!mfma_path(type, N, K, M)) return 0;
     GemmPlan p = gemm_plan(M, N, K);
     return align256(M * K * sizeof(_Float16)) + align256(M * sizeof(float)) + (p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0);
+}
+
+size_t qgemm_planes_bytes(int type, size_t M, size_t N, size_t K) {
+    if (!mfma_path(type, N, K, M)) return 0;
+    return (size_t)gemm_plan(M, N, K).ksplit * M * N * sizeof(float);
+}
+
+hipError_t launch_xprep(hipStream_t s, const float *X, size_t M, size_t K, _Float16 *Xp, float *inv_scale) {
+    if (M == 0 || K == 0 || K % 256 != 0) return hipErrorInvalidValue;
+    xprep_kernel<<<dim3((unsigned)M), 256, 0, s>>>(X, K, Xp, inv_scale);
+    return hipGetLastError();
+}
+
+hipError_t launch_xprep_rmsnorm(hipStream_t s, PlaneSum in, const float *res, float *x_out, const float *gamma, float eps, size_t M, size_t K,
+                                _Float16 *Xp, float *inv_scale) {
+    if (M == 0 || K == 0 || K % 256 != 0 || K > kXprepFusedMaxK || in.n < 1 || !in.base || !gamma) return hipErrorInvalidValue;
+    RowSrc S{ in, PlaneSum{ nullptr, 0, 0 }, res, x_out, gamma, eps };
+    xprep_fused_kernel<kPrepRms><<<dim3((unsigned)M), 256, 0, s>>>(S, K, Xp, inv_scale);
+    return hipGetLastError();
+}
+
+hipError_t launch_xprep_swiglu(hipStream_t s, PlaneSum gate, PlaneSum up, size_t M, size_t K, _Float16 *Xp, float *inv_scale) {
+    if (M == 0 || K == 0 || K % 256 != 0 || K > kXprepFusedMaxK || gate.n < 1 || up.n < 1 || !gate.base || !up.base) return hipErrorInvalidValue;
+    RowSrc S{ gate, up, nullptr, nullptr, nullptr, 0.f };
+    xprep_fused_kernel<kPrepSwiglu><<<dim3((unsigned)M), 256, 0, s>>>(S, K, Xp, inv_scale);
+    return hipGetLastError();
+}
+
+// The contraction alone: Xp / inv_scale come from one of the pre-pass launches above, the k splits stay as planes.
+hipError_t launch_qgemm_planes(hipStream_t s, int type, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const _Float16 *Xp,
+                               const float *inv_scale, size_t M, float *planes, size_t planes_bytes, PlaneSum *out) {
+    if (!mfma_path(type, N, K, M) || !out) return hipErrorInvalidValue;
+    const GemmPlan p = gemm_plan(M, N, K);
+    if ((size_t)p.ksplit * M * N * sizeof(float) > planes_bytes) return hipErrorInvalidValue;
+    *out = PlaneSum{ planes, M * N, p.ksplit };
+    if (type == RT_GGML_Q4_K) return launch_type<RT_GGML_Q4_K>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, planes, nullptr, planes, false);
+    return launch_type<RT_GGML_Q6_K>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, planes, nullptr, planes, false);
+}
+
+hipError_t launch_plane_sum(hipStream_t s, PlaneSum in, const float *res, float *Y, size_t n) {
+    if (n == 0 || n % 4 != 0 || in.n < 1) return hipErrorInvalidValue;
+    const size_t n4 = n / 4;
+    const unsigned grid = (unsigned)std::min<size_t>((n4 + 255) / 256, 2048);
+    splitk_reduce_kernel<<<grid, 256, 0, s>>>(in.base, in.stride, in.n, res, Y, n4);
+    return hipGetLastError();
 }
 
 // res (optional) is added to the result; it may be Y itself only on the row-by-row path.

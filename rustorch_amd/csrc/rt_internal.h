@@ -160,6 +160,32 @@ size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K);
 // true: launch_qgemm runs the matrix-core contraction (with its pre-pass of X); false: the GEMV kernel, one grid slice per row of X
 bool qgemm_on_matrix_cores(int type, size_t M, size_t N, size_t K);
 
+// A matrix held as n partial planes: element i is base[i] + base[stride + i] + ... (summed in that order).
+// What a k-split contraction leaves behind; n = 1 is an ordinary matrix.
+struct PlaneSum {
+    const float *base;
+    size_t stride;
+    int n;
+};
+// The pieces of launch_qgemm for a caller that chains contractions: the pre-pass on its own (plain, or fused with the
+// operation that produces the activation matrix), the contraction without the reduction of its k splits, and consumers
+// that read plane sums.  Xp: M x K fp16 (scaled, k-permuted), inv_scale: M floats; K a multiple of 256.
+size_t qgemm_planes_bytes(int type, size_t M, size_t N, size_t K);             // planes a contraction of this shape may write
+constexpr size_t kXprepFusedMaxK = 12288;                                       // longest row the fused producers keep in registers
+hipError_t launch_xprep(hipStream_t s, const float *X, size_t M, size_t K, _Float16 *Xp, float *inv_scale);
+// x = in (+ res), stored to x_out when given; prepared matrix = gamma * x / sqrt(mean(x^2) + eps)
+hipError_t launch_xprep_rmsnorm(hipStream_t s, PlaneSum in, const float *res, float *x_out, const float *gamma, float eps, size_t M, size_t K,
+                                _Float16 *Xp, float *inv_scale);
+// prepared matrix = up * gate * sigmoid(gate)
+hipError_t launch_xprep_swiglu(hipStream_t s, PlaneSum gate, PlaneSum up, size_t M, size_t K, _Float16 *Xp, float *inv_scale);
+hipError_t launch_qgemm_planes(hipStream_t s, int type, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const _Float16 *Xp,
+                               const float *inv_scale, size_t M, float *planes, size_t planes_bytes, PlaneSum *out);
+// Y = in (+ res), n elements (a multiple of 4)
+hipError_t launch_plane_sum(hipStream_t s, PlaneSum in, const float *res, float *Y, size_t n);
+// rope_kv_batch with q, k, v given as plane sums; the rotated q goes to q_out
+hipError_t launch_rope_kv_planes(hipStream_t s, PlaneSum q, PlaneSum k, PlaneSum v, float *q_out, uint16_t *kcache, uint16_t *vcache,
+                                 int pos0, size_t n_tok, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev);
+
 inline size_t type_block_bytes(int t) {
     switch (t) {
     case RT_GGML_F32: return 4;

@@ -189,6 +189,36 @@ __global__ void rope_kv_batch_kernel(float *q, const float *k, const float *v, u
     reinterpret_cast<uint32_t *>(vcache + (size_t)p * rowkv)[t] = (uint32_t)f2h_rne(vv.x) | ((uint32_t)f2h_rne(vv.y) << 16);
 }
 
+// The same with q, k, v given as the partial planes of k-split contractions: the planes are summed on the way in and
+// the rotated q goes to q_out.
+__device__ __forceinline__ float2 plane_pair(const PlaneSum &p, size_t pair) {
+    float2 a = reinterpret_cast<const float2 *>(p.base)[pair];
+    for (int z = 1; z < p.n; z++) {
+        const float2 b = reinterpret_cast<const float2 *>(p.base + (size_t)z * p.stride)[pair];
+        a.x += b.x;
+        a.y += b.y;
+    }
+    return a;
+}
+__global__ void rope_kv_planes_kernel(PlaneSum q, PlaneSum k, PlaneSum v, float *q_out, uint16_t *kcache, uint16_t *vcache,
+                                      int pos0, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq) {
+    int half = head_dim / 2;
+    int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_heads * half) return;
+    int i = t % half;
+    const size_t prow = (size_t)n_heads * half, prowkv = (size_t)n_kv_heads * half, m = blockIdx.y;     // float2 pairs per row
+    const int p = pos0 + (int)m;
+    float s, c;
+    sincosf((float)p * inv_freq[i], &s, &c);
+    const float2 qv = plane_pair(q, m * prow + t);
+    reinterpret_cast<float2 *>(q_out)[m * prow + t] = make_float2(qv.x * c - qv.y * s, qv.x * s + qv.y * c);
+    if (t >= n_kv_heads * half) return;          // fewer key / value heads than query heads
+    const float2 kv = plane_pair(k, m * prowkv + t), vv = plane_pair(v, m * prowkv + t);
+    float k0 = kv.x * c - kv.y * s, k1 = kv.x * s + kv.y * c;
+    reinterpret_cast<uint32_t *>(kcache + (size_t)p * 2 * prowkv)[t] = (uint32_t)f2h_rne(k0) | ((uint32_t)f2h_rne(k1) << 16);
+    reinterpret_cast<uint32_t *>(vcache + (size_t)p * 2 * prowkv)[t] = (uint32_t)f2h_rne(vv.x) | ((uint32_t)f2h_rne(vv.y) << 16);
+}
+
 // -------------------------------------------------------- decode attention
 // One block (256 threads) per query head; cache layout [pos][kv head][dim], fp16.  With fewer key / value heads
 // than query heads, query head h reads kv head h / (n_heads / n_kv_heads) and the first query head of each
@@ -724,6 +754,15 @@ hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const f
     int pairs = n_heads * head_dim / 2;
     rope_kv_batch_kernel<<<dim3((unsigned)((pairs + 255) / 256), (unsigned)n_tok), 256, 0, s>>>(q, k, v, kcache, vcache, pos0, n_heads,
                                                                                                 n_kv_heads, head_dim, inv_freq_dev);
+    return hipGetLastError();
+}
+
+hipError_t launch_rope_kv_planes(hipStream_t s, PlaneSum q, PlaneSum k, PlaneSum v, float *q_out, uint16_t *kcache, uint16_t *vcache,
+                                 int pos0, size_t n_tok, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads != 0 || n_tok == 0 || n_tok > 65535 || q.n < 1 || k.n < 1 || v.n < 1) return hipErrorInvalidValue;
+    int pairs = n_heads * head_dim / 2;
+    rope_kv_planes_kernel<<<dim3((unsigned)((pairs + 255) / 256), (unsigned)n_tok), 256, 0, s>>>(q, k, v, q_out, kcache, vcache, pos0, n_heads,
+                                                                                                 n_kv_heads, head_dim, inv_freq_dev);
     return hipGetLastError();
 }
 

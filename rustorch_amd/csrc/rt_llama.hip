@@ -64,6 +64,10 @@ struct rt_hip_llama {
     float *pf_x = nullptr, *pf_x2 = nullptr, *pf_n = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_a = nullptr;
     float *pf_g = nullptr, *pf_u = nullptr;
     int *pf_tok = nullptr;
+    // chained form of the batched prefill: prepared activation matrix, its row scales, three areas of partial planes
+    _Float16 *pf_xp = nullptr;
+    float *pf_inv = nullptr, *pf_planes[3] = { nullptr, nullptr, nullptr };
+    size_t pf_planes_bytes = 0;
     std::vector<void *> allocs;
 };
 
@@ -195,6 +199,13 @@ int ensure_prefill_buffers(rt_hip_ctx *ctx, rt_hip_llama *m, size_t n_tok) {
     if ((rc = dev_alloc(ctx, m, (void **)&m->pf_g, cap * F * sizeof(float)))) return rc;
     if ((rc = dev_alloc(ctx, m, (void **)&m->pf_u, cap * F * sizeof(float)))) return rc;
     if ((rc = dev_alloc(ctx, m, (void **)&m->pf_tok, cap * sizeof(int)))) return rc;
+    // a k-split contraction writes at most 256 tiles of 128 x 256 results; without a split, one matrix of cap rows
+    const size_t widest = std::max(std::max(H, F), m->kv_dim);
+    m->pf_planes_bytes = std::max((size_t)256 * 128 * 256, cap * widest) * sizeof(float);
+    for (float *&p : m->pf_planes)
+        if ((rc = dev_alloc(ctx, m, (void **)&p, m->pf_planes_bytes))) return rc;
+    if ((rc = dev_alloc(ctx, m, (void **)&m->pf_xp, cap * std::max(H, F) * sizeof(_Float16)))) return rc;
+    if ((rc = dev_alloc(ctx, m, (void **)&m->pf_inv, (cap + 64) * sizeof(float)))) return rc;     // read four rows at a time, past the last
     m->pf_cap = cap;
     return RT_HIP_OK;
 }
@@ -212,6 +223,62 @@ struct PrefillGemm {
         return RT_HIP_OK;
     }
 };
+
+// Every matrix of every layer goes to the matrix cores at this M, and the rows fit the fused pre-pass kernels.
+bool prefill_chainable(const rt_hip_llama *m, size_t M) {
+    const size_t H = (size_t)m->cfg.hidden, F = (size_t)m->cfg.ffn;
+    if (H > rt::kXprepFusedMaxK || F > rt::kXprepFusedMaxK || H % 256 != 0 || F % 256 != 0) return false;
+    for (int l = 0; l < m->cfg.n_layers; l++)
+        for (const auto *t : { &m->wq[l], &m->wk[l], &m->wv[l], &m->wo[l], &m->wgate[l], &m->wup[l], &m->wdown[l] })
+            if (!rt::qgemm_on_matrix_cores(t->type, M, t->n_rows, t->n_cols) ||
+                rt::qgemm_planes_bytes(t->type, M, t->n_rows, t->n_cols) > m->pf_planes_bytes)
+                return false;
+    return true;
+}
+
+// The batched prefill as a chain without stand-alone reductions or pre-passes: a k-split contraction leaves its partial
+// planes, and the kernel that consumes the result sums them on the way in; the operations that produce an activation
+// matrix (RMSNorm of the residual stream, SwiGLU) write it directly in the contraction's prepared form.
+// Per layer: [x += planes of the previous down-projection] RMSNorm -> q, k, v -> RoPE + cache append -> causal
+// attention -> pre-pass -> o-projection -> [x += its planes] RMSNorm -> gate, up -> SwiGLU -> down-projection.
+int enqueue_prefill_chain(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) {
+    hipStream_t s = ctx->stream;
+    const rt_hip_llama_config &c = m->cfg;
+    const size_t H = (size_t)c.hidden, F = (size_t)c.ffn;
+    float *x = m->pf_x;                          // the residual stream, updated in place (a thread rewrites what it has read)
+    float **P = m->pf_planes;
+    auto mm = [&](const rt_hip_llama::T &t, float *planes, rt::PlaneSum *out) {
+        return rt::launch_qgemm_planes(s, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, m->pf_xp, m->pf_inv, M, planes, m->pf_planes_bytes, out);
+    };
+    RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, m->pf_tok, M, c.vocab, x));
+    rt::PlaneSum pending{ x, 0, 1 };             // what the next RMSNorm reads: first the embeddings themselves,
+    const float *pending_res = nullptr;          // later the planes of a down-projection, to be added to x
+    for (int l = 0; l < c.n_layers; l++) {
+        uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
+        uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
+        rt::PlaneSum q, k, v, o, g, u, d;
+        RT_TRY_HIP(ctx, rt::launch_xprep_rmsnorm(s, pending, pending_res, pending_res ? x : nullptr, m->attn_norm[l], c.rms_eps, M, H, m->pf_xp, m->pf_inv));
+        RT_TRY_HIP(ctx, mm(m->wq[l], P[0], &q));
+        RT_TRY_HIP(ctx, mm(m->wk[l], P[1], &k));
+        RT_TRY_HIP(ctx, mm(m->wv[l], P[2], &v));
+        RT_TRY_HIP(ctx, rt::launch_rope_kv_planes(s, q, k, v, m->pf_q, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
+        RT_TRY_HIP(ctx, rt::launch_attn_causal(s, m->pf_q, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->pf_a));
+        RT_TRY_HIP(ctx, rt::launch_xprep(s, m->pf_a, M, H, m->pf_xp, m->pf_inv));
+        RT_TRY_HIP(ctx, mm(m->wo[l], P[0], &o));
+        RT_TRY_HIP(ctx, rt::launch_xprep_rmsnorm(s, o, x, x, m->ffn_norm[l], c.rms_eps, M, H, m->pf_xp, m->pf_inv));      // x += o
+        RT_TRY_HIP(ctx, mm(m->wgate[l], P[1], &g));
+        RT_TRY_HIP(ctx, mm(m->wup[l], P[2], &u));
+        RT_TRY_HIP(ctx, rt::launch_xprep_swiglu(s, g, u, M, F, m->pf_xp, m->pf_inv));
+        RT_TRY_HIP(ctx, mm(m->wdown[l], P[0], &d));
+        pending = d;                             // x += d happens in the next layer's RMSNorm launch
+        pending_res = x;
+    }
+    // hidden state of the last token = its row of pending_res + pending
+    const size_t last = (M - 1) * H;
+    rt::PlaneSum row{ pending.base + last, pending.stride, pending.n };
+    RT_TRY_HIP(ctx, rt::launch_plane_sum(s, row, pending_res ? pending_res + last : nullptr, m->x, H));
+    return RT_HIP_OK;
+}
 
 // M tokens (already in pf_tok) at positions pos0 .. pos0+M-1 through all layers with the dense contraction:
 // per layer rmsnorm rows -> q,k,v GEMMs -> rope + cache append -> causal attention (query m over pos0+m+1 rows)
@@ -541,7 +608,7 @@ int rt_hip_llama_prefill(rt_hip_ctx *ctx, rt_hip_llama *m, const int *tokens, in
             const size_t M = std::min(kPrefillChunk, (size_t)n_tok - t0);
             RT_TRY_HIP(ctx, hipMemcpyAsync(m->pf_tok, tokens + t0, M * sizeof(int), hipMemcpyHostToDevice, ctx->stream));
             if (M >= 16) {
-                rc = enqueue_prefill_batch(ctx, m, M, pos0 + (int)t0);
+                rc = prefill_chainable(m, M) ? enqueue_prefill_chain(ctx, m, M, pos0 + (int)t0) : enqueue_prefill_batch(ctx, m, M, pos0 + (int)t0);
                 if (rc) return rc;
             } else {
                 // a short tail goes token by token (the row form of the contraction starts at 16 rows)
