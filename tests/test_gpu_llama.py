@@ -174,6 +174,41 @@ def test_long_context_attention_split_over_workgroups(ex, orc, n_heads, n_kv):
     assert np.median(ratios) <= 0.2
 
 
+def test_prefill_in_several_passes_and_calls(ex, orc):
+    """A prompt longer than one pass of the batched prefill (512 tokens), the same prompt fed in two calls (the second
+    starts at a position above zero) and token by token: the three device paths agree far inside the tolerance, and
+    follow the oracle at the typical position."""
+    from rustorch_amd import synth
+    cfg = dict(n_layers=2, hidden=256, n_heads=2, ffn=512, vocab=300, max_pos=700)
+    print("llama prefill passes", cfg, flush=True)
+    gm, om, wn = build_pair(ex, orc, 41, **cfg)
+    toks = synth.tokens(41, synth.TID_PROMPT, 560, cfg["vocab"])
+    want = om.forward(toks, 0)
+    tol = logit_tol(wn, cfg["hidden"])
+    n = 540                                                      # 512 + 28: two passes of the chained pipeline
+    gm.prefill(toks[:n], 0)
+    one_call = gm.logits().copy()
+    gm.reset()
+    gm.prefill(toks[:300], 0)
+    gm.prefill(toks[300:n], 300)                                 # 240 tokens at positions 300 ..
+    two_calls = gm.logits().copy()
+    gm.reset()
+    for p in range(n):
+        gm.step(int(toks[p]), p)
+    stepped = gm.logits().copy()
+    d1 = float((np.abs(one_call - stepped) / tol).max()); d2 = float((np.abs(two_calls - stepped) / tol).max())
+    r = float((np.abs(one_call - want[n - 1]) / tol).max())
+    print("one call vs stepped %.3f, two calls vs stepped %.3f, vs oracle %.3f of the tolerance" % (d1, d2, r), flush=True)
+    assert d1 <= 0.1 and d2 <= 0.1
+    # the cache the passes left serves the decode steps that follow
+    ratios = []
+    gm.reset(); gm.prefill(toks[:n], 0)
+    for p in range(n, n + 12):
+        gm.step(int(toks[p]), p)
+        ratios.append(float((np.abs(gm.logits() - want[p]) / tol).max()))
+    assert np.median(ratios) <= 0.2
+
+
 @pytest.mark.parametrize("fmt", ["Q5_K", "Q8_0", "Q4_0"])
 def test_model_in_a_format_without_matrix_core_path(ex, orc, fmt):
     """All seven matrices of every layer in one format that the dense contraction does not serve.  Decode: the GEMV
