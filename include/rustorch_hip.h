@@ -52,6 +52,9 @@ typedef enum {
     RT_GGML_F32 = 0,
     RT_GGML_F16 = 1,
     RT_GGML_Q4_0 = 2,
+    RT_GGML_Q4_1 = 3,
+    RT_GGML_Q5_0 = 6,
+    RT_GGML_Q5_1 = 7,
     RT_GGML_Q8_0 = 8,
     RT_GGML_Q4_K = 12,
     RT_GGML_Q5_K = 13,

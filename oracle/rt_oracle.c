@@ -22,7 +22,7 @@
  * What the reference does NOT hold and this file therefore owns (parity with
  * the reference is unpinned for these; they are pinned by closed forms,
  * exhaustive packer round trips and an independent NumPy decoder in tests/):
- *   - the Q8_0 / Q4_0 / Q4_K / Q5_K / Q6_K block decoders.  The reference only fixes
+ *   - the Q8_0 / Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K / Q6_K block decoders.  The reference only fixes
  *     type ids and block byte sizes (example-cli/src/model/formats/gguf.rs:78-144)
  *     and decodes every quantized type with a placeholder
  *     (tensor_loader.rs:125-141,213-218).  The layouts below are the public
@@ -43,7 +43,7 @@
 
 #define ORC_API __attribute__((visibility("default")))
 
-enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };
+enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q4_1 = 3, ORC_Q5_0 = 6, ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };
 
 /* ------------------------------------------------------------------ fp16 */
 
@@ -104,7 +104,7 @@ static inline uint16_t rd_u16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1]
 
 ORC_API int orc_block_elems(int type) {
     switch (type) {
-    case ORC_Q8_0: case ORC_Q4_0: return 32;
+    case ORC_Q8_0: case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: return 32;
     case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 256;
     case ORC_F32: case ORC_F16: return 1;
     default: return 0;
@@ -116,6 +116,9 @@ ORC_API int orc_block_bytes(int type) {
     switch (type) {
     case ORC_Q8_0: return 34;
     case ORC_Q4_0: return 18;
+    case ORC_Q4_1: return 20;
+    case ORC_Q5_0: return 22;
+    case ORC_Q5_1: return 24;
     case ORC_Q4_K: return 144;
     case ORC_Q5_K: return 176;
     case ORC_Q6_K: return 210;
@@ -141,6 +144,42 @@ static void deq_q4_0(const uint8_t *b, float *y) {
     for (int j = 0; j < 16; j++) {
         y[j] = (float)((int)(qs[j] & 0x0F) - 8) * d;
         y[j + 16] = (float)((int)(qs[j] >> 4) - 8) * d;
+    }
+}
+
+/* Q4_1: { f16 d; f16 m; u8 qs[16] }   y = q * d + m, nibble order as Q4_0 */
+static void deq_q4_1(const uint8_t *b, float *y) {
+    float d = orc_h2f(rd_u16(b)), m = orc_h2f(rd_u16(b + 2));
+    const uint8_t *qs = b + 4;
+    for (int j = 0; j < 16; j++) {
+        y[j] = (float)(qs[j] & 0x0F) * d + m;
+        y[j + 16] = (float)(qs[j] >> 4) * d + m;
+    }
+}
+
+/* Q5_0: { f16 d; u8 qh[4]; u8 qs[16] }   qh read as a little-endian u32: bit j is the fifth bit of element j */
+static void deq_q5_0(const uint8_t *b, float *y) {
+    float d = orc_h2f(rd_u16(b));
+    uint32_t qh = (uint32_t)b[2] | ((uint32_t)b[3] << 8) | ((uint32_t)b[4] << 16) | ((uint32_t)b[5] << 24);
+    const uint8_t *qs = b + 6;
+    for (int j = 0; j < 16; j++) {
+        int x0 = (int)((qs[j] & 0x0F) | (((qh >> j) << 4) & 0x10)) - 16;
+        int x1 = (int)((qs[j] >> 4) | ((qh >> (j + 12)) & 0x10)) - 16;
+        y[j] = (float)x0 * d;
+        y[j + 16] = (float)x1 * d;
+    }
+}
+
+/* Q5_1: { f16 d; f16 m; u8 qh[4]; u8 qs[16] }   y = q5 * d + m */
+static void deq_q5_1(const uint8_t *b, float *y) {
+    float d = orc_h2f(rd_u16(b)), m = orc_h2f(rd_u16(b + 2));
+    uint32_t qh = (uint32_t)b[4] | ((uint32_t)b[5] << 8) | ((uint32_t)b[6] << 16) | ((uint32_t)b[7] << 24);
+    const uint8_t *qs = b + 8;
+    for (int j = 0; j < 16; j++) {
+        int x0 = (int)((qs[j] & 0x0F) | (((qh >> j) << 4) & 0x10));
+        int x1 = (int)((qs[j] >> 4) | ((qh >> (j + 12)) & 0x10));
+        y[j] = (float)x0 * d + m;
+        y[j + 16] = (float)x1 * d + m;
     }
 }
 
@@ -223,6 +262,9 @@ static void deq_row(int type, const uint8_t *row, size_t n_cols, float *y) {
     switch (type) {
     case ORC_Q8_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q8_0(row + 34 * b, y + 32 * b); break;
     case ORC_Q4_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q4_0(row + 18 * b, y + 32 * b); break;
+    case ORC_Q4_1: for (size_t b = 0; b < n_cols / 32; b++) deq_q4_1(row + 20 * b, y + 32 * b); break;
+    case ORC_Q5_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q5_0(row + 22 * b, y + 32 * b); break;
+    case ORC_Q5_1: for (size_t b = 0; b < n_cols / 32; b++) deq_q5_1(row + 24 * b, y + 32 * b); break;
     case ORC_Q4_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q4_k(row + 144 * b, y + 256 * b); break;
     case ORC_Q5_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q5_k(row + 176 * b, y + 256 * b); break;
     case ORC_Q6_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q6_k(row + 210 * b, y + 256 * b); break;

@@ -84,6 +84,27 @@ __device__ inline float deq_elem(int type, const uint8_t *row, size_t col) {
         int q = j < 16 ? (b[2 + j] & 0x0F) : (b[2 + j - 16] >> 4);
         return (float)(q - 8) * d;
     }
+    case RT_GGML_Q4_1: {       // { f16 d; f16 m; u8 qs[16] }
+        const uint8_t *b = row + 20 * (col >> 5);
+        float d = h2f(ld2u(b)), m = h2f(ld2u(b + 2));
+        int j = (int)(col & 31);
+        int q = j < 16 ? (b[4 + j] & 0x0F) : (b[4 + j - 16] >> 4);
+        return (float)q * d + m;
+    }
+    case RT_GGML_Q5_0: {       // { f16 d; u8 qh[4]; u8 qs[16] }: bit j of qh (little-endian u32) is the fifth bit of element j
+        const uint8_t *b = row + 22 * (col >> 5);
+        float d = h2f(ld2u(b));
+        int j = (int)(col & 31);
+        int q = (j < 16 ? (b[6 + j] & 0x0F) : (b[6 + j - 16] >> 4)) | (((b[2 + (j >> 3)] >> (j & 7)) & 1) << 4);
+        return (float)(q - 16) * d;
+    }
+    case RT_GGML_Q5_1: {       // { f16 d; f16 m; u8 qh[4]; u8 qs[16] }
+        const uint8_t *b = row + 24 * (col >> 5);
+        float d = h2f(ld2u(b)), m = h2f(ld2u(b + 2));
+        int j = (int)(col & 31);
+        int q = (j < 16 ? (b[8 + j] & 0x0F) : (b[8 + j - 16] >> 4)) | (((b[4 + (j >> 3)] >> (j & 7)) & 1) << 4);
+        return (float)q * d + m;
+    }
     case RT_GGML_Q4_K: {
         const uint8_t *b = row + 144 * (col >> 8);
         int e = (int)(col & 255);

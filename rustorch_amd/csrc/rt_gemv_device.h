@@ -135,6 +135,13 @@ template <> struct WRegs<RT_GGML_Q8_0> { uint4 a, b; uint32_t d; };
 template <> struct XRegs<RT_GGML_Q8_0> { uint4 h[2], l[2]; float s; };
 template <> struct WRegs<RT_GGML_Q4_0> { uint4 a; uint32_t d; };
 template <> struct XRegs<RT_GGML_Q4_0> { uint4 h[2], l[2]; float2 sv; };
+// Q4_1 / Q5_0 / Q5_1: 32-element blocks like Q4_0 (same x slice), with an offset m and / or a word of fifth bits
+template <> struct WRegs<RT_GGML_Q4_1> { uint4 a; uint32_t dm; };           // d | m << 16
+template <> struct WRegs<RT_GGML_Q5_0> { uint4 a; uint32_t d, qh; };
+template <> struct WRegs<RT_GGML_Q5_1> { uint4 a; uint32_t dm, qh; };
+template <> struct XRegs<RT_GGML_Q4_1> : XRegs<RT_GGML_Q4_0> {};
+template <> struct XRegs<RT_GGML_Q5_0> : XRegs<RT_GGML_Q4_0> {};
+template <> struct XRegs<RT_GGML_Q5_1> : XRegs<RT_GGML_Q4_0> {};
 
 // Weight loads go through a buffer resource: the matrix is the buffer, the row (wave-uniform) a scalar byte
 // offset, the lane's place in the row a 32-bit vector offset -- no 64-bit address arithmetic per load.
@@ -151,6 +158,9 @@ __device__ __forceinline__ uint4 bld16(WRow r, uint32_t off) {
 }
 __device__ __forceinline__ uint2 bld8(WRow r, uint32_t off) {
     return __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r.rsrc, off, r.soff, 0));
+}
+__device__ __forceinline__ uint32_t bld4(WRow r, uint32_t off) {
+    return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r.rsrc, off, r.soff, 0);
 }
 __device__ __forceinline__ uint32_t bld2(WRow r, uint32_t off) {
     return (uint32_t)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r.rsrc, off, r.soff, 0);
@@ -190,6 +200,24 @@ __device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_0> &w, WRow row, int u) 
     w.a = bld16(row, off + 2u);
 }
 
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_1> &w, WRow row, int u) {
+    uint32_t off = (uint32_t)u * 20u;
+    w.dm = bld4(row, off);
+    w.a = bld16(row, off + 4u);
+}
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q5_0> &w, WRow row, int u) {
+    uint32_t off = (uint32_t)u * 22u;
+    w.d = bld2(row, off);
+    w.qh = bld2(row, off + 2u) | (bld2(row, off + 4u) << 16);
+    w.a = bld16(row, off + 6u);
+}
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q5_1> &w, WRow row, int u) {
+    uint32_t off = (uint32_t)u * 24u;
+    w.dm = bld4(row, off);
+    w.qh = bld4(row, off + 4u);
+    w.a = bld16(row, off + 8u);
+}
+
 __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_K> &x, const uint32_t *lds, int u, int U, int K) {
     const uint4 *XH = reinterpret_cast<const uint4 *>(lds);
     const uint4 *XL = XH + K / 16;
@@ -220,6 +248,16 @@ __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_0> &x, const uint32_t *l
     const uint4 *XL = XH + K / 16;
     x.h[0] = XH[u]; x.h[1] = XH[U + u]; x.l[0] = XL[u]; x.l[1] = XL[U + u];
     x.sv = reinterpret_cast<const float2 *>(lds + K / 2)[u];
+}
+
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_1> &x, const uint32_t *lds, int u, int U, int K) {
+    load_x(static_cast<XRegs<RT_GGML_Q4_0> &>(x), lds, u, U, K);
+}
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q5_0> &x, const uint32_t *lds, int u, int U, int K) {
+    load_x(static_cast<XRegs<RT_GGML_Q4_0> &>(x), lds, u, U, K);
+}
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q5_1> &x, const uint32_t *lds, int u, int U, int K) {
+    load_x(static_cast<XRegs<RT_GGML_Q4_0> &>(x), lds, u, U, K);
 }
 
 #define RT_W4(v) { (v).x, (v).y, (v).z, (v).w }
@@ -357,6 +395,39 @@ __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_0> &w, const XR
         dl = sdot4(hi, (int)lhi[i], dl);
     }
     return h2f(w.d) * __builtin_fmaf(x.sv.x, (float)((dh << 7) + dl), -8.f * x.sv.y);
+}
+// The integer sums of a 32-element block against the two planes of x: nibbles of the 16 bytes, optionally with the
+// fifth bits of qh (bit j: element j; the low nibbles are elements 0..15, the high ones 16..31).  Four bits of qh
+// reach bit 4 of four bytes through one multiplication: bit k lands on 8k + 4 (and on places the mask drops).
+template <bool FIFTH>
+__device__ __forceinline__ int block32_dot(const uint4 &a, uint32_t qh, const XRegs<RT_GGML_Q4_0> &x) {
+    const uint32_t q[4] = RT_W4(a);
+    const uint32_t hlo[4] = RT_W4(x.h[0]), hhi[4] = RT_W4(x.h[1]), llo[4] = RT_W4(x.l[0]), lhi[4] = RT_W4(x.l[1]);
+    int dh = 0, dl = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint32_t lo = q[i] & 0x0f0f0f0fu, hi = (q[i] >> 4) & 0x0f0f0f0fu;
+        if (FIFTH) {
+            lo |= (((qh >> (4 * i)) & 15u) * 0x02040810u) & 0x10101010u;
+            hi |= (((qh >> (16 + 4 * i)) & 15u) * 0x02040810u) & 0x10101010u;
+        }
+        dh = sdot4(lo, (int)hlo[i], dh);
+        dl = sdot4(lo, (int)llo[i], dl);
+        dh = sdot4(hi, (int)hhi[i], dh);
+        dl = sdot4(hi, (int)lhi[i], dl);
+    }
+    return (dh << 7) + dl;      // below 2^24 in magnitude (32 elements x 31 x 127 x 128 + ...): exact as a float
+}
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_1> &w, const XRegs<RT_GGML_Q4_1> &x, int) {
+    const float t = x.sv.x * (float)block32_dot<false>(w.a, 0u, x);
+    return __builtin_fmaf(h2f(w.dm & 0xFFFFu), t, h2f(w.dm >> 16) * x.sv.y);
+}
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q5_0> &w, const XRegs<RT_GGML_Q5_0> &x, int) {
+    return h2f(w.d) * __builtin_fmaf(x.sv.x, (float)block32_dot<true>(w.a, w.qh, x), -16.f * x.sv.y);
+}
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q5_1> &w, const XRegs<RT_GGML_Q5_1> &x, int) {
+    const float t = x.sv.x * (float)block32_dot<true>(w.a, w.qh, x);
+    return __builtin_fmaf(h2f(w.dm & 0xFFFFu), t, h2f(w.dm >> 16) * x.sv.y);
 }
 #pragma clang fp contract(fast)
 
@@ -497,6 +568,9 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
         case RT_GGML_Q6_K: gemv_problem<RT_GGML_Q6_K, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q4_1: gemv_problem<RT_GGML_Q4_1, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q5_0: gemv_problem<RT_GGML_Q5_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q5_1: gemv_problem<RT_GGML_Q5_1, 2, COH>(P, wg, n_wg, m, lds, red); break;
         }
     } else {
         switch (P.type) {
@@ -505,6 +579,9 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
         case RT_GGML_Q6_K: gemv_problem<RT_GGML_Q6_K, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q4_1: gemv_problem<RT_GGML_Q4_1, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q5_0: gemv_problem<RT_GGML_Q5_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q5_1: gemv_problem<RT_GGML_Q5_1, 1, COH>(P, wg, n_wg, m, lds, red); break;
         }
     }
 }

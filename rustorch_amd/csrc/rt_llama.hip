@@ -181,7 +181,10 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
     return RT_HIP_OK;
 }
 
-bool gemv_type_ok(int t) { return t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_K || t == RT_GGML_Q5_K || t == RT_GGML_Q6_K; }
+bool gemv_type_ok(int t) {
+    return t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_1 || t == RT_GGML_Q5_0 || t == RT_GGML_Q5_1 || t == RT_GGML_Q4_K ||
+           t == RT_GGML_Q5_K || t == RT_GGML_Q6_K;
+}
 
 constexpr size_t kPrefillChunk = 512;     // tokens per pass of the batched prefill
 

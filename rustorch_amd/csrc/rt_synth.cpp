@@ -7,6 +7,8 @@
 // f16_rne((float)(lo + (hi - lo) * u))):
 //   Q8_0 : w0 -> d from u24(r);  w1..w8 -> 32 x u16 v, qs = ((v * 255) >> 16) - 127
 //   Q4_0 : w0 -> d;  w1,w2 -> the 16 qs bytes verbatim
+//   Q4_1 : w0 -> d from u24(r), m = -8 d' with d' from u24(r >> 32);  w1,w2 -> qs
+//   Q5_0 : w0 -> d, qh = bits 32..63 of r;  w1,w2 -> qs        Q5_1 : w0 -> d, m = -16 d';  w1,w2 -> qs;  w3 -> qh (low 32 bits)
 //   Q4_K : w0 -> d from u24(r), dmin from u24(r >> 32);  w1 -> 8 scales (byte & 63);
 //          w2 -> 8 mins (byte & 63), packed into the 12-byte field;  w3..w18 -> qs
 //   Q5_K : w0..w2 as Q4_K;  w3..w6 -> qh;  w7..w22 -> qs
@@ -86,6 +88,33 @@ void gen_block(int type, uint64_t key, uint64_t b, double lo, double hi, uint8_t
         put16(o, scale_f16(lo, hi, u24(mix(base))));
         put64(o + 2, mix(base + 1));
         put64(o + 10, mix(base + 2));
+        break;
+    }
+    case RT_GGML_Q4_1: {       // the offset sits where a symmetric format would put it (m of the order of -8 d)
+        uint64_t r0 = mix(base);
+        put16(o, scale_f16(lo, hi, u24(r0)));
+        put16(o + 2, scale_f16(-8.0 * lo, -8.0 * hi, u24(r0 >> 32)));
+        put64(o + 4, mix(base + 1));
+        put64(o + 12, mix(base + 2));
+        break;
+    }
+    case RT_GGML_Q5_0: {
+        uint64_t r0 = mix(base);
+        put16(o, scale_f16(lo, hi, u24(r0)));
+        uint32_t qh = (uint32_t)(r0 >> 32);
+        std::memcpy(o + 2, &qh, 4);
+        put64(o + 6, mix(base + 1));
+        put64(o + 14, mix(base + 2));
+        break;
+    }
+    case RT_GGML_Q5_1: {
+        uint64_t r0 = mix(base);
+        put16(o, scale_f16(lo, hi, u24(r0)));
+        put16(o + 2, scale_f16(-16.0 * lo, -16.0 * hi, u24(r0 >> 32)));
+        uint32_t qh = (uint32_t)mix(base + 3);
+        std::memcpy(o + 4, &qh, 4);
+        put64(o + 8, mix(base + 1));
+        put64(o + 16, mix(base + 2));
         break;
     }
     case RT_GGML_Q4_K: {

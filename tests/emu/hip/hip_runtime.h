@@ -108,10 +108,12 @@ typedef unsigned int emu_u32x2 __attribute__((ext_vector_type(2)));
 inline emu_buffer_rsrc emu_make_rsrc(const void *p) { return emu_buffer_rsrc{ (const unsigned char *)p }; }
 inline emu_u32x4 emu_bload128(emu_buffer_rsrc r, unsigned voff, unsigned soff) { emu_u32x4 v; __builtin_memcpy(&v, r.base + voff + soff, 16); return v; }
 inline emu_u32x2 emu_bload64(emu_buffer_rsrc r, unsigned voff, unsigned soff) { emu_u32x2 v; __builtin_memcpy(&v, r.base + voff + soff, 8); return v; }
+inline unsigned int emu_bload32(emu_buffer_rsrc r, unsigned voff, unsigned soff) { unsigned int v; __builtin_memcpy(&v, r.base + voff + soff, 4); return v; }
 inline short emu_bload16(emu_buffer_rsrc r, unsigned voff, unsigned soff) { short v; __builtin_memcpy(&v, r.base + voff + soff, 2); return v; }
 #define __builtin_amdgcn_make_buffer_rsrc(p, stride, num, flags) emu_make_rsrc(p)
 #define __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, aux) emu_bload128(r, voff, soff)
 #define __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, aux) emu_bload64(r, voff, soff)
+#define __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, aux) emu_bload32(r, voff, soff)
 #define __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, aux) emu_bload16(r, voff, soff)
 #define __builtin_amdgcn_s_sleep(n) emu::spin_yield()
 #define __builtin_amdgcn_s_waitcnt(n) ((void)0)

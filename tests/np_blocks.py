@@ -35,6 +35,32 @@ def decode_q4_0(blk: np.ndarray) -> np.ndarray:
     return out
 
 
+def _legacy5(blk: np.ndarray, qh_off: int, qs_off: int, e: int) -> int:
+    """Stored value of element e of a 32-element block: nibble (low for e < 16) plus, with qh_off >= 0, bit e of the
+    little-endian 32-bit word at qh_off as the fifth bit."""
+    byte = int(blk[qs_off + (e % 16)])
+    q = (byte >> 4) if e >= 16 else (byte & 15)
+    if qh_off >= 0:
+        word = int.from_bytes(bytes(blk[qh_off:qh_off + 4]), "little")
+        q |= ((word >> e) & 1) << 4
+    return q
+
+
+def decode_q4_1(blk: np.ndarray) -> np.ndarray:
+    d, m = _f16(blk, 0), _f16(blk, 2)
+    return np.array([F32(F32(F32(_legacy5(blk, -1, 4, e)) * d) + m) for e in range(32)], dtype=F32)
+
+
+def decode_q5_0(blk: np.ndarray) -> np.ndarray:
+    d = _f16(blk, 0)
+    return np.array([F32(F32(_legacy5(blk, 2, 6, e) - 16) * d) for e in range(32)], dtype=F32)
+
+
+def decode_q5_1(blk: np.ndarray) -> np.ndarray:
+    d, m = _f16(blk, 0), _f16(blk, 2)
+    return np.array([F32(F32(F32(_legacy5(blk, 4, 8, e)) * d) + m) for e in range(32)], dtype=F32)
+
+
 def q4k_scale_min(scales: np.ndarray, j: int):
     s = [int(v) for v in scales]
     if j < 4:
@@ -90,7 +116,7 @@ def decode_q6_k(blk: np.ndarray) -> np.ndarray:
 
 
 DECODERS = {8: (34, 32, decode_q8_0), 2: (18, 32, decode_q4_0), 12: (144, 256, decode_q4_k), 14: (210, 256, decode_q6_k),
-            13: (176, 256, decode_q5_k)}
+            13: (176, 256, decode_q5_k), 3: (20, 32, decode_q4_1), 6: (22, 32, decode_q5_0), 7: (24, 32, decode_q5_1)}
 
 
 def decode(ggml_type: int, raw: np.ndarray) -> np.ndarray:
@@ -118,6 +144,40 @@ def encode_q4_0(d, q) -> np.ndarray:
     _put_f16(blk, 0, d)
     q = np.asarray(q, dtype=np.uint8)
     blk[2:] = q[:16] | (q[16:] << 4)
+    return blk
+
+
+def _legacy5_fields(q):
+    """32 stored values (0..31) -> the 16 nibble bytes and the word of fifth bits."""
+    q = np.asarray(q, dtype=np.uint8)
+    qs = (q[:16] & 15) | ((q[16:] & 15) << 4)
+    word = 0
+    for e in range(32):
+        word |= ((int(q[e]) >> 4) & 1) << e
+    return qs, np.frombuffer(word.to_bytes(4, "little"), dtype=np.uint8)
+
+
+def encode_q4_1(d, m, q) -> np.ndarray:
+    """q: 32 values in 0..15; the decoded element is q * d + m."""
+    blk = np.zeros(20, dtype=np.uint8)
+    _put_f16(blk, 0, d); _put_f16(blk, 2, m)
+    blk[4:], _ = _legacy5_fields(q)
+    return blk
+
+
+def encode_q5_0(d, q) -> np.ndarray:
+    """q: 32 values in 0..31; the decoded element is (q - 16) * d."""
+    blk = np.zeros(22, dtype=np.uint8)
+    _put_f16(blk, 0, d)
+    blk[6:], blk[2:6] = _legacy5_fields(q)
+    return blk
+
+
+def encode_q5_1(d, m, q) -> np.ndarray:
+    """q: 32 values in 0..31; the decoded element is q * d + m."""
+    blk = np.zeros(24, dtype=np.uint8)
+    _put_f16(blk, 0, d); _put_f16(blk, 2, m)
+    blk[8:], blk[4:8] = _legacy5_fields(q)
     return blk
 
 

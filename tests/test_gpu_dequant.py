@@ -12,7 +12,7 @@ def bits(a):
     return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
 
 
-@pytest.mark.parametrize("t", [8, 2, 12, 13, 14])
+@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 12, 13, 14])
 def test_golden_vectors_bit_exact(ex, t):
     g = np.load(GOLDEN)
     raw, val = g["raw_%d" % t], g["val_%d" % t]
@@ -22,7 +22,8 @@ def test_golden_vectors_bit_exact(ex, t):
     assert np.array_equal(bits(got), bits(val))   # includes zero, max-finite and subnormal fp16 scales
 
 
-@pytest.mark.parametrize("t,rows,cols", [(8, 64, 4096), (2, 33, 11008), (12, 48, 4096), (12, 17, 11008), (14, 40, 4096), (14, 9, 11008), (13, 48, 4096), (13, 5, 11008)])
+@pytest.mark.parametrize("t,rows,cols", [(8, 64, 4096), (2, 33, 11008), (12, 48, 4096), (12, 17, 11008), (14, 40, 4096), (14, 9, 11008), (13, 48, 4096), (13, 5, 11008),
+                                         (3, 33, 4096), (6, 33, 11008), (7, 20, 4096)])
 def test_synthetic_tensors_bit_exact(ex, orc, t, rows, cols):
     from rustorch_amd import synth
     print("dequant synthetic", t, rows, cols, flush=True)

@@ -9,7 +9,7 @@ import pytest
 import np_blocks as nb
 
 GOLDEN = Path(__file__).resolve().parent / "golden" / "blocks_golden.npz"
-TYPES = [8, 2, 12, 13, 14]
+TYPES = [8, 2, 3, 6, 7, 12, 13, 14]
 
 
 def bits(a):
@@ -48,8 +48,8 @@ def test_f32_to_fp16_rne(orc):
 
 def test_block_geometry_matches_reference_type_size(orc):
     # example-cli/src/model/formats/gguf.rs:125-144
-    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 8, 12, 13, 14)] == [4, 2, 18, 34, 144, 176, 210]
-    assert [orc.load().orc_block_elems(t) for t in (2, 8, 12, 13, 14)] == [32, 32, 256, 256, 256]
+    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 3, 6, 7, 8, 12, 13, 14)] == [4, 2, 18, 20, 22, 24, 34, 144, 176, 210]
+    assert [orc.load().orc_block_elems(t) for t in (2, 3, 6, 7, 8, 12, 13, 14)] == [32, 32, 32, 32, 32, 256, 256, 256]
     assert orc.load().orc_row_bytes(12, 4096) == 2304 and orc.load().orc_row_bytes(14, 11008) == 9030
     assert orc.load().orc_row_bytes(12, 100) == 0
 
@@ -87,6 +87,40 @@ def test_q4_0_nibble_order_and_offset(orc):
     blk[2 + 3] = 0xA1   # low nibble 1 -> element 3, high nibble 10 -> element 19
     y = orc.dequant(2, blk, 1, 32)[0]
     want = np.full(32, -16.0, dtype=np.float32); want[3] = (1 - 8) * 2; want[19] = (10 - 8) * 2
+    assert np.array_equal(y, want)
+
+
+def test_q4_1_q5_0_q5_1_closed_forms(orc):
+    # Q4_1: q * d + m, nibble order as Q4_0
+    q4 = np.concatenate([np.arange(16), 15 - np.arange(16)]).astype(np.uint8)
+    y = orc.dequant(3, nb.encode_q4_1(1.0, 0.0, q4), 1, 32)[0]
+    assert np.array_equal(y, q4.astype(np.float32))
+    y = orc.dequant(3, nb.encode_q4_1(0.5, -3.0, q4), 1, 32)[0]
+    assert np.array_equal(y, q4.astype(np.float32) * 0.5 - 3.0)
+    # Q5_0: every stored value 0..31 at every element, one at a time (the others hold 16, which decodes to 0)
+    for e in range(32):
+        for v in (0, 1, 15, 16, 17, 30, 31):
+            q = np.full(32, 16, dtype=np.uint8); q[e] = v
+            y = orc.dequant(6, nb.encode_q5_0(2.0, q), 1, 32)[0]
+            want = np.zeros(32, dtype=np.float32); want[e] = (v - 16) * 2.0
+            assert np.array_equal(y, want), (e, v)
+    # the fifth bit of element e is bit e of the little-endian word after d: set one bit by hand
+    for e in (0, 7, 8, 15, 16, 23, 31):
+        blk = np.zeros(22, dtype=np.uint8); blk[0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+        blk[2 + e // 8] = 1 << (e % 8)
+        y = orc.dequant(6, blk, 1, 32)[0]
+        want = np.full(32, -16.0, dtype=np.float32); want[e] = 0.0
+        assert np.array_equal(y, want), e
+    # Q5_1: q5 * d + m, all 32 values at once in two arrangements
+    q5 = np.arange(32, dtype=np.uint8)
+    for q in (q5, q5[::-1].copy()):
+        y = orc.dequant(7, nb.encode_q5_1(0.25, 1.5, q), 1, 32)[0]
+        assert np.array_equal(y, q.astype(np.float32) * 0.25 + 1.5)
+    blk = np.zeros(24, dtype=np.uint8); blk[0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blk[4 + 2] = 0x20                       # bit 21 of the word: element 21
+    blk[8 + 5] = 0x93                       # low nibble 3 -> element 5, high nibble 9 -> element 21
+    y = orc.dequant(7, blk, 1, 32)[0]
+    want = np.zeros(32, dtype=np.float32); want[5] = 3; want[21] = 9 + 16
     assert np.array_equal(y, want)
 
 

@@ -38,6 +38,15 @@ def ref_block(t, seed, tid, b, lo, hi):
     if t == 2:
         w = words(seed, tid, b, 3)
         return np.concatenate([scale(lo, hi, w[0]), w[1:].view(np.uint8)])
+    if t == 3:
+        w = words(seed, tid, b, 3)
+        return np.concatenate([scale(lo, hi, w[0]), scale(-8.0 * lo, -8.0 * hi, int(w[0]) >> 32), w[1:].view(np.uint8)])
+    if t == 6:
+        w = words(seed, tid, b, 3)
+        return np.concatenate([scale(lo, hi, w[0]), w[0:1].view(np.uint8)[4:], w[1:].view(np.uint8)])
+    if t == 7:
+        w = words(seed, tid, b, 4)
+        return np.concatenate([scale(lo, hi, w[0]), scale(-16.0 * lo, -16.0 * hi, int(w[0]) >> 32), w[3:4].view(np.uint8)[:4], w[1:3].view(np.uint8)])
     if t == 12:
         w = words(seed, tid, b, 19)
         sc = w[1:2].view(np.uint8) & 63
@@ -53,7 +62,7 @@ def ref_block(t, seed, tid, b, lo, hi):
     return np.concatenate([w[:24].view(np.uint8), sc, scale(lo, hi, w[26])])
 
 
-@pytest.mark.parametrize("t", [8, 2, 12, 13, 14])
+@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 12, 13, 14])
 def test_blocks_follow_the_specification(lib, t):
     from rustorch_amd import synth, GGMLType
     lo, hi = synth.D_RANGE[GGMLType(t)]
