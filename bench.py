@@ -115,7 +115,7 @@ def bench_layer_gemv(ex, steps, warmup, n_layers):
 
 
 def bench_single_gemv(ex, reps=200):
-    """The single-matrix decode configurations: Q8_0 4096x4096 and Q4_0 at the two FFN shapes (and one Q5_K), batch 1, x resident
+    """The single-matrix decode configurations: Q8_0 4096x4096 and Q4_0 at the two FFN shapes (and one Q5_K and one unquantized F16 matrix), batch 1, x resident
     in HBM as f32 (quantized in the kernel's staging).  Eight synthetic copies of each matrix are rotated so that
     the larger ones come from HBM rather than from the Infinity Cache."""
     from rustorch_amd import synth, GGMLType
@@ -123,7 +123,8 @@ def bench_single_gemv(ex, reps=200):
     for name, t, rows, cols in (("q8_0_4096x4096", GGMLType.Q8_0, 4096, 4096),
                                 ("q4_0_11008x4096", GGMLType.Q4_0, 11008, 4096),
                                 ("q4_0_4096x11008", GGMLType.Q4_0, 4096, 11008),
-                                ("q5_k_11008x4096", GGMLType.Q5_K, 11008, 4096)):     # not a benchmark configuration: for the record
+                                ("q5_k_11008x4096", GGMLType.Q5_K, 11008, 4096),      # not benchmark configurations: for the record
+                                ("f16_4096x4096", GGMLType.F16, 4096, 4096)):
         ws = [ex.upload_qweight(t, rows, cols, synth.blocks(t, SEED, 8000 + i, rows, cols)) for i in range(8)]
         x = ex.to_device(synth.normal(SEED, 8100, cols))
         y = ex.buffer(4 * rows)

@@ -3,6 +3,8 @@
 // device code in rt_gemv_device.h.
 #include "rt_gemv_device.h"
 
+#include <algorithm>
+
 namespace rt {
 
 namespace {
@@ -36,13 +38,13 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
 hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
     if (a.n <= 0 || a.n > kMaxGemvProbs || batch <= 0) return hipErrorInvalidValue;
     double total_bytes = 0;
-    size_t maxK = 0, total_rows = 0;
+    size_t lds = 0, total_rows = 0;
     for (int i = 0; i < a.n; i++) {
         if ((double)a.p[i].N * (double)a.p[i].row_bytes >= 4294967296.0) return hipErrorInvalidValue;   // row offsets are 32-bit
         if (a.p[i].type == RT_GGML_Q5_K && a.p[i].epi == kEpiSwiglu) return hipErrorInvalidValue;         // no pair form for Q5_K
         total_bytes += (double)a.p[i].N * (double)a.p[i].row_bytes * (a.p[i].epi == kEpiSwiglu ? 2.0 : 1.0);
         total_rows += (size_t)a.p[i].N;
-        if ((size_t)a.p[i].K > maxK) maxK = (size_t)a.p[i].K;
+        lds = std::max(lds, gemv_lds_bytes(a.p[i].type, (size_t)a.p[i].K));
     }
     if (total_bytes <= 0) return hipErrorInvalidValue;
     // 16 resident waves per CU over 256 CUs, as one or two workgroups
@@ -65,7 +67,7 @@ hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
         a.p[i].rows_per_tile = n;
         wgs += n;
     }
-    size_t lds = xq_stride(maxK);
+    if (lds > 64 * 1024) return hipErrorInvalidValue;      // x of the longest row must fit the workgroup's LDS
     dim3 grid((unsigned)wgs, (unsigned)batch);
     if (threads == 512) qgemv_kernel<512><<<grid, 512, lds, s>>>(a, r2);
     else qgemv_kernel<1024><<<grid, 1024, lds, s>>>(a, r2);

@@ -25,7 +25,11 @@
 
 namespace rt {
 
+// Units of a row: 64 elements of the super-block formats, one 32-element block of the others, 16 bytes of an
+// unquantized row (8 halves or 4 floats).
 __device__ __forceinline__ int units_of(int type, int K) {
+    if (type == RT_GGML_F16) return K / 8;
+    if (type == RT_GGML_F32) return K / 4;
     return (type == RT_GGML_Q4_K || type == RT_GGML_Q5_K || type == RT_GGML_Q6_K) ? K / 64 : K / 32;
 }
 
@@ -83,6 +87,18 @@ __device__ __forceinline__ void stage_x(const GemvProb &P, int m, uint32_t *lds,
         const uint32_t *ql = reinterpret_cast<const uint32_t *>(xq + K);
         const float *xs = reinterpret_cast<const float *>(xq + 2 * (size_t)K);
         const float *xb = xs + K / 32;
+        if (gemv_float_weights(type)) {
+            // unquantized weights take x back as f32: x = s * (128 * high part + low part)
+            float4 *xf = reinterpret_cast<float4 *>(lds);
+            for (int i = threadIdx.x; i < n4; i += (int)blockDim.x) {
+                const float s = xs[i >> 3];
+                const uint32_t hi = qh[i], lo = ql[i];
+                xf[i] = make_float4(s * (float)(((int)(int8_t)(hi & 0xFF) << 7) + (int)(lo & 127)),
+                                    s * (float)(((int)(int8_t)((hi >> 8) & 0xFF) << 7) + (int)((lo >> 8) & 127)),
+                                    s * (float)(((int)(int8_t)((hi >> 16) & 0xFF) << 7) + (int)((lo >> 16) & 127)),
+                                    s * (float)(((int)(int8_t)(hi >> 24) << 7) + (int)((lo >> 24) & 127)));
+            }
+        } else
         for (int i = threadIdx.x; i < n4; i += (int)blockDim.x) {
             int e = 4 * i;
             float s = 0.f, b16 = 0.f, b32 = 0.f;
@@ -113,6 +129,10 @@ __device__ __forceinline__ void stage_x(const GemvProb &P, int m, uint32_t *lds,
                 float4 g = g4[i];
                 v = make_float4(g.x * (v.x / rms), g.y * (v.y / rms), g.z * (v.z / rms), g.w * (v.w / rms));
             }
+            if (gemv_float_weights(type)) {
+                reinterpret_cast<float4 *>(lds)[i] = v;
+                continue;
+            }
             Q4Pack p = quantize4(v);
             stage_store(type, K, U, lds, 4 * i, p.hi, p.lo, p.s, p.s * (float)p.sum16, p.s * (float)p.sum32);
         }
@@ -135,6 +155,11 @@ template <> struct WRegs<RT_GGML_Q8_0> { uint4 a, b; uint32_t d; };
 template <> struct XRegs<RT_GGML_Q8_0> { uint4 h[2], l[2]; float s; };
 template <> struct WRegs<RT_GGML_Q4_0> { uint4 a; uint32_t d; };
 template <> struct XRegs<RT_GGML_Q4_0> { uint4 h[2], l[2]; float2 sv; };
+// unquantized rows: 16 bytes of weights per unit against the f32 x in LDS
+template <> struct WRegs<RT_GGML_F16> { uint4 q; };
+template <> struct XRegs<RT_GGML_F16> { float4 a, b; };
+template <> struct WRegs<RT_GGML_F32> { uint4 q; };
+template <> struct XRegs<RT_GGML_F32> { float4 a; };
 // Q4_1 / Q5_0 / Q5_1: 32-element blocks like Q4_0 (same x slice), with an offset m and / or a word of fifth bits
 template <> struct WRegs<RT_GGML_Q4_1> { uint4 a; uint32_t dm; };           // d | m << 16
 template <> struct WRegs<RT_GGML_Q5_0> { uint4 a; uint32_t d, qh; };
@@ -200,6 +225,8 @@ __device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_0> &w, WRow row, int u) 
     w.a = bld16(row, off + 2u);
 }
 
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_F16> &w, WRow row, int u) { w.q = bld16(row, (uint32_t)u * 16u); }
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_F32> &w, WRow row, int u) { w.q = bld16(row, (uint32_t)u * 16u); }
 __device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_1> &w, WRow row, int u) {
     uint32_t off = (uint32_t)u * 20u;
     w.dm = bld4(row, off);
@@ -250,6 +277,13 @@ __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_0> &x, const uint32_t *l
     x.sv = reinterpret_cast<const float2 *>(lds + K / 2)[u];
 }
 
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_F16> &x, const uint32_t *lds, int u, int, int) {
+    x.a = reinterpret_cast<const float4 *>(lds)[2 * u];
+    x.b = reinterpret_cast<const float4 *>(lds)[2 * u + 1];
+}
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_F32> &x, const uint32_t *lds, int u, int, int) {
+    x.a = reinterpret_cast<const float4 *>(lds)[u];
+}
 __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_1> &x, const uint32_t *lds, int u, int U, int K) {
     load_x(static_cast<XRegs<RT_GGML_Q4_0> &>(x), lds, u, U, K);
 }
@@ -396,6 +430,27 @@ __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_0> &w, const XR
     }
     return h2f(w.d) * __builtin_fmaf(x.sv.x, (float)((dh << 7) + dl), -8.f * x.sv.y);
 }
+// Unquantized rows: products in element order, one fused multiply-add each.
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_F16> &w, const XRegs<RT_GGML_F16> &x, int) {
+    const uint32_t q[4] = RT_W4(w.q);
+    float a = h2f(q[0] & 0xFFFFu) * x.a.x;
+    a = __builtin_fmaf(h2f(q[0] >> 16), x.a.y, a);
+    a = __builtin_fmaf(h2f(q[1] & 0xFFFFu), x.a.z, a);
+    a = __builtin_fmaf(h2f(q[1] >> 16), x.a.w, a);
+    a = __builtin_fmaf(h2f(q[2] & 0xFFFFu), x.b.x, a);
+    a = __builtin_fmaf(h2f(q[2] >> 16), x.b.y, a);
+    a = __builtin_fmaf(h2f(q[3] & 0xFFFFu), x.b.z, a);
+    a = __builtin_fmaf(h2f(q[3] >> 16), x.b.w, a);
+    return a;
+}
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_F32> &w, const XRegs<RT_GGML_F32> &x, int) {
+    float a = __uint_as_float(w.q.x) * x.a.x;
+    a = __builtin_fmaf(__uint_as_float(w.q.y), x.a.y, a);
+    a = __builtin_fmaf(__uint_as_float(w.q.z), x.a.z, a);
+    a = __builtin_fmaf(__uint_as_float(w.q.w), x.a.w, a);
+    return a;
+}
+
 // The integer sums of a 32-element block against the two planes of x: nibbles of the 16 bytes, optionally with the
 // fifth bits of qh (bit j: element j; the low nibbles are elements 0..15, the high ones 16..31).  Four bits of qh
 // reach bit 4 of four bytes through one multiplication: bit k lands on 8k + 4 (and on places the mask drops).
@@ -569,6 +624,8 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
         case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_1: gemv_problem<RT_GGML_Q4_1, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_F16: gemv_problem<RT_GGML_F16, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_F32: gemv_problem<RT_GGML_F32, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q5_0: gemv_problem<RT_GGML_Q5_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q5_1: gemv_problem<RT_GGML_Q5_1, 2, COH>(P, wg, n_wg, m, lds, red); break;
         }
@@ -580,6 +637,8 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
         case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_1: gemv_problem<RT_GGML_Q4_1, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_F16: gemv_problem<RT_GGML_F16, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_F32: gemv_problem<RT_GGML_F32, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q5_0: gemv_problem<RT_GGML_Q5_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q5_1: gemv_problem<RT_GGML_Q5_1, 1, COH>(P, wg, n_wg, m, lds, red); break;
         }

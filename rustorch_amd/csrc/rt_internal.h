@@ -31,6 +31,9 @@ constexpr int kWave = 64;
 //   [.., +K/4)        bsum f32[K/16] = s * (sum of q over each 16-element run)  (for the -8 / -32 / -min terms)
 // padded to a multiple of 16 bytes.
 __host__ __device__ inline size_t xq_stride(size_t K) { return (2 * K + K / 8 + K / 4 + 15) & ~(size_t)15; }
+// Unquantized weight matrices (F16 / F32) meet x as plain f32 in LDS; the block formats meet the two-plane integer form.
+__host__ __device__ inline bool gemv_float_weights(int type) { return type == 0 /* F32 */ || type == 1 /* F16 */; }
+__host__ __device__ inline size_t gemv_lds_bytes(int type, size_t K) { return gemv_float_weights(type) ? 4 * K : xq_stride(K); }
 
 // How a GEMV workgroup obtains the activation vector it stages into LDS.
 enum : int {

@@ -182,8 +182,8 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
 }
 
 bool gemv_type_ok(int t) {
-    return t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_1 || t == RT_GGML_Q5_0 || t == RT_GGML_Q5_1 || t == RT_GGML_Q4_K ||
-           t == RT_GGML_Q5_K || t == RT_GGML_Q6_K;
+    return t == RT_GGML_F32 || t == RT_GGML_F16 || t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_1 || t == RT_GGML_Q5_0 ||
+           t == RT_GGML_Q5_1 || t == RT_GGML_Q4_K || t == RT_GGML_Q5_K || t == RT_GGML_Q6_K;
 }
 
 constexpr size_t kPrefillChunk = 512;     // tokens per pass of the batched prefill
@@ -415,8 +415,11 @@ int rt_hip_llama_upload_tensor(rt_hip_ctx *ctx, rt_hip_llama *m, int slot, int l
         RT_REQUIRE(ctx, n_rows == er && n_cols == ec, RT_HIP_ERR_SHAPE, "slot %d expects %zu x %zu, got %zu x %zu", slot, er, ec, n_rows, n_cols);
         size_t be = rt::type_block_elems(ggml_type), bb = rt::type_block_bytes(ggml_type);
         RT_REQUIRE(ctx, be != 0, RT_HIP_ERR_UNSUPPORTED_TYPE, "unsupported GGML type id %d", ggml_type);
-        if (slot != RT_LLAMA_TOK_EMBD)
+        if (slot != RT_LLAMA_TOK_EMBD) {
             RT_REQUIRE(ctx, gemv_type_ok(ggml_type), RT_HIP_ERR_UNSUPPORTED_TYPE, "GGML type id %d has no GEMV kernel", ggml_type);
+            RT_REQUIRE(ctx, n_cols % 32 == 0 && rt::gemv_lds_bytes(ggml_type, n_cols) <= 64 * 1024, RT_HIP_ERR_SHAPE,
+                       "rows of %zu elements of type %d do not fit the GEMV's staging", n_cols, ggml_type);
+        }
         RT_REQUIRE(ctx, n_cols % be == 0 && nbytes == n_rows * (n_cols / be) * bb, RT_HIP_ERR_SHAPE, "payload of %zu bytes does not match %zu x %zu of type %d",
                    nbytes, n_rows, n_cols, ggml_type);
     }

@@ -29,9 +29,15 @@ D_RANGE = {
 LLAMA7B = dict(n_layers=32, hidden=4096, n_heads=32, ffn=11008, vocab=32000, rms_eps=1e-5, rope_theta=10000.0)
 
 
+DENSE_STD = 0.02      # unquantized synthetic matrices: N(0, DENSE_STD^2), rounded to the storage type
+
+
 def blocks(ggml_type: int, seed: int, tensor_id: int, n_rows: int, n_cols: int, d_range=None) -> np.ndarray:
     """Raw GGUF payload (uint8) of an n_rows x n_cols tensor."""
     t = GGMLType(int(ggml_type))
+    if t in (GGMLType.F16, GGMLType.F32):
+        w = normal(seed, tensor_id, n_rows * n_cols, 0.0, DENSE_STD)
+        return np.ascontiguousarray(w.astype(np.float16 if t == GGMLType.F16 else np.float32)).view(np.uint8)
     lo, hi = d_range if d_range is not None else D_RANGE[t]
     n_blocks = n_rows * (n_cols // t.block_elems())
     out = np.empty(n_blocks * t.type_size(), dtype=np.uint8)

@@ -23,7 +23,7 @@ def test_golden_vectors_bit_exact(ex, t):
 
 
 @pytest.mark.parametrize("t,rows,cols", [(8, 64, 4096), (2, 33, 11008), (12, 48, 4096), (12, 17, 11008), (14, 40, 4096), (14, 9, 11008), (13, 48, 4096), (13, 5, 11008),
-                                         (3, 33, 4096), (6, 33, 11008), (7, 20, 4096)])
+                                         (3, 33, 4096), (6, 33, 11008), (7, 20, 4096), (1, 9, 4096), (0, 5, 1024)])
 def test_synthetic_tensors_bit_exact(ex, orc, t, rows, cols):
     from rustorch_amd import synth
     print("dequant synthetic", t, rows, cols, flush=True)

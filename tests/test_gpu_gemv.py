@@ -23,6 +23,9 @@ SHAPES = {
     "q4_1_up": (3, 11008, 4096),             # the older 32-element formats with an offset and / or a fifth bit
     "q5_0_down": (6, 4096, 11008),
     "q5_1_q": (7, 4096, 4096),
+    "f16_q": (1, 4096, 4096),                # unquantized matrices: the formats the reference decodes itself
+    "f16_down": (1, 4096, 11008),
+    "f32_up": (0, 11008, 4096),
 }
 
 
@@ -54,10 +57,10 @@ def test_gemv_config_shapes_batch1_and_8(ex, orc, name):
     check(yo, y64[:2], wn, x[:2], name + " oracle f32 vs f64")
 
 
-@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 12, 13, 14])
+@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 12, 13, 14, 1, 0])
 def test_gemv_edge_inputs(ex, orc, t):
     from rustorch_amd import synth
-    be = 32 if t in (8, 2, 3, 6, 7) else 256
+    be = 256 if t in (12, 13, 14) else 32                  # unquantized rows: any multiple of 32 columns
     rows, cols = 5, 3 * be                                  # ragged: fewer rows than a tile, odd block count
     print("gemv edge", t, rows, cols, flush=True)
     raw = synth.blocks(t, 7, 1, rows, cols)
