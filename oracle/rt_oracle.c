@@ -22,7 +22,7 @@
  * What the reference does NOT hold and this file therefore owns (parity with
  * the reference is unpinned for these; they are pinned by closed forms,
  * exhaustive packer round trips and an independent NumPy decoder in tests/):
- *   - the Q8_0 / Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K / Q6_K block decoders.  The reference only fixes
+ *   - the Q8_0 / Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q3_K / Q4_K / Q5_K / Q6_K block decoders.  The reference only fixes
  *     type ids and block byte sizes (example-cli/src/model/formats/gguf.rs:78-144)
  *     and decodes every quantized type with a placeholder
  *     (tensor_loader.rs:125-141,213-218).  The layouts below are the public
@@ -43,7 +43,7 @@
 
 #define ORC_API __attribute__((visibility("default")))
 
-enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q4_1 = 3, ORC_Q5_0 = 6, ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };
+enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q4_1 = 3, ORC_Q5_0 = 6, ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q3_K = 11, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };
 
 /* ------------------------------------------------------------------ fp16 */
 
@@ -105,7 +105,7 @@ static inline uint16_t rd_u16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1]
 ORC_API int orc_block_elems(int type) {
     switch (type) {
     case ORC_Q8_0: case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: return 32;
-    case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 256;
+    case ORC_Q3_K: case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 256;
     case ORC_F32: case ORC_F16: return 1;
     default: return 0;
     }
@@ -119,6 +119,7 @@ ORC_API int orc_block_bytes(int type) {
     case ORC_Q4_1: return 20;
     case ORC_Q5_0: return 22;
     case ORC_Q5_1: return 24;
+    case ORC_Q3_K: return 110;
     case ORC_Q4_K: return 144;
     case ORC_Q5_K: return 176;
     case ORC_Q6_K: return 210;
@@ -180,6 +181,39 @@ static void deq_q5_1(const uint8_t *b, float *y) {
         int x1 = (int)((qs[j] >> 4) | ((qh >> (j + 12)) & 0x10));
         y[j] = (float)x0 * d + m;
         y[j + 16] = (float)x1 * d + m;
+    }
+}
+
+/* Q3_K: { u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d } (110 B, type id 11, gguf.rs:89,138).
+ * Sixteen 6-bit scales (stored + 32), one per 16 elements: the low four bits of scale k sit in a nibble of
+ * scales[0..7], the high two in a 2-bit field of scales[8..11], gathered here with the word shuffle of the
+ * public ggml definition.  Element values are a 2-bit field of qs minus 4 unless its hmask bit is set. */
+static void deq_q3_k(const uint8_t *b, float *y) {
+    const uint32_t kmask1 = 0x03030303u, kmask2 = 0x0f0f0f0fu;
+    const uint8_t *hm = b, *q = b + 32;
+    float d_all = orc_h2f(rd_u16(b + 108));
+    uint32_t aux[4];
+    memcpy(aux, b + 96, 12);
+    uint32_t tmp = aux[2];
+    aux[2] = ((aux[0] >> 4) & kmask2) | (((tmp >> 4) & kmask1) << 4);
+    aux[3] = ((aux[1] >> 4) & kmask2) | (((tmp >> 6) & kmask1) << 4);
+    aux[0] = (aux[0] & kmask2) | (((tmp >> 0) & kmask1) << 4);
+    aux[1] = (aux[1] & kmask2) | (((tmp >> 2) & kmask1) << 4);
+    int8_t scales[16];
+    memcpy(scales, aux, 16);
+    int is = 0;
+    uint8_t m = 1;
+    for (int n = 0; n < 256; n += 128) {
+        int shift = 0;
+        for (int j = 0; j < 4; j++) {
+            float dl = d_all * (float)(scales[is++] - 32);
+            for (int l = 0; l < 16; l++) *y++ = dl * (float)((int)((q[l] >> shift) & 3) - ((hm[l] & m) ? 0 : 4));
+            dl = d_all * (float)(scales[is++] - 32);
+            for (int l = 0; l < 16; l++) *y++ = dl * (float)((int)((q[l + 16] >> shift) & 3) - ((hm[l + 16] & m) ? 0 : 4));
+            shift += 2;
+            m <<= 1;
+        }
+        q += 32;
     }
 }
 
@@ -265,6 +299,7 @@ static void deq_row(int type, const uint8_t *row, size_t n_cols, float *y) {
     case ORC_Q4_1: for (size_t b = 0; b < n_cols / 32; b++) deq_q4_1(row + 20 * b, y + 32 * b); break;
     case ORC_Q5_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q5_0(row + 22 * b, y + 32 * b); break;
     case ORC_Q5_1: for (size_t b = 0; b < n_cols / 32; b++) deq_q5_1(row + 24 * b, y + 32 * b); break;
+    case ORC_Q3_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q3_k(row + 110 * b, y + 256 * b); break;
     case ORC_Q4_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q4_k(row + 144 * b, y + 256 * b); break;
     case ORC_Q5_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q5_k(row + 176 * b, y + 256 * b); break;
     case ORC_Q6_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q6_k(row + 210 * b, y + 256 * b); break;

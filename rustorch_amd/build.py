@@ -46,13 +46,51 @@ def find_hipcc() -> str:
     return found
 
 
-def _run(cmd: list[str]) -> None:
+# Kernels whose speed depends on running without private (scratch) memory: the build fails if the compiler gave
+# one of them a scratch frame (register spills or an array it could not keep in registers).  One spilling variant
+# inside such a kernel slows every launch of it, also the ones that never reach the variant.
+NO_SCRATCH = {"rt_gemv.hip": ("qgemv_kernel",), "rt_gemm.hip": ("qgemm_kernel",), "rt_attn_prefill.hip": ("attn_causal_kernel",)}
+RESOURCE_FLAG = "-Rpass-analysis=kernel-resource-usage"
+
+
+def _run(cmd: list[str]) -> str:
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
         raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), proc.stdout))
-    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l and l.strip())
-    if out:
-        sys.stderr.write(out + "\n")
+    quiet = ("packed-fp32-ops", RESOURCE_FLAG)
+    keep, skip = [], 0
+    for l in proc.stdout.splitlines():
+        if skip:                         # the source line and caret that follow a remark
+            skip -= 1
+            continue
+        if "remark: Function Name" in l:
+            skip = 2
+        if l.strip() and not any(q in l for q in quiet):
+            keep.append(l)
+    if keep:
+        sys.stderr.write("\n".join(keep) + "\n")
+    return proc.stdout
+
+
+def check_no_scratch(name: str, log: str) -> None:
+    """Parse the compiler's per-kernel resource remarks of one source file."""
+    wanted = NO_SCRATCH.get(name, ())
+    current = None
+    seen = set()
+    for l in log.splitlines():
+        if "remark: Function Name:" in l:
+            current = l.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in l and current:
+            size = int(l.split("ScratchSize [bytes/lane]:")[1].split("[")[0])
+            for k in wanted:
+                if k in current:
+                    seen.add(k)
+                    if size != 0:
+                        raise RuntimeError("%s: kernel %s uses %d bytes of scratch per lane (register spills); "
+                                           "every launch of it would slow down" % (name, current, size))
+    missing = set(wanted) - seen
+    if missing:
+        raise RuntimeError("%s: no resource report for %s" % (name, ", ".join(sorted(missing))))
 
 
 def build_all(verbose: bool = True) -> Path:
@@ -63,10 +101,13 @@ def build_all(verbose: bool = True) -> Path:
     def compile_one(name: str) -> Path:
         src = CSRC / name
         obj = OBJ / (Path(name).stem + ".o")
-        cmd = [hipcc] + HIP_FLAGS + (["-x", "hip"] if name.endswith(".cpp") else []) + ["-c", str(src), "-o", str(obj)]
+        extra = [RESOURCE_FLAG] if name in NO_SCRATCH else []
+        cmd = [hipcc] + HIP_FLAGS + extra + (["-x", "hip"] if name.endswith(".cpp") else []) + ["-c", str(src), "-o", str(obj)]
         if verbose:
             print("[build]", " ".join(cmd), flush=True)
-        _run(cmd)
+        log = _run(cmd)
+        if name in NO_SCRATCH:
+            check_no_scratch(name, log)
         return obj
 
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:

@@ -105,6 +105,18 @@ __device__ inline float deq_elem(int type, const uint8_t *row, size_t col) {
         int q = (j < 16 ? (b[8 + j] & 0x0F) : (b[8 + j - 16] >> 4)) | (((b[4 + (j >> 3)] >> (j & 7)) & 1) << 4);
         return (float)q * d + m;
     }
+    case RT_GGML_Q3_K: {       // { u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d }: 2 low bits in qs, the third in hmask, 16 six-bit scales
+        const uint8_t *b = row + 110 * (col >> 8);
+        int e = (int)(col & 255);
+        int n = e >> 7, j = (e >> 5) & 3, l = e & 31;      // half, 32-run within the half, position
+        int k = 8 * n + 2 * j + (l >> 4);                  // scale of the 16 elements around e
+        const uint8_t *s = b + 96;
+        int lo4 = k < 8 ? (s[k] & 15) : (s[k - 8] >> 4);
+        int hi2 = (s[8 + (k & 3)] >> (2 * (k >> 2))) & 3;
+        float dl = h2f(ld2u(b + 108)) * (float)((lo4 | (hi2 << 4)) - 32);
+        int q = ((b[32 + 32 * n + l] >> (2 * j)) & 3) - (((b[l] >> (4 * n + j)) & 1) ? 0 : 4);
+        return dl * (float)q;
+    }
     case RT_GGML_Q4_K: {
         const uint8_t *b = row + 144 * (col >> 8);
         int e = (int)(col & 255);

@@ -61,6 +61,25 @@ def decode_q5_1(blk: np.ndarray) -> np.ndarray:
     return np.array([F32(F32(F32(_legacy5(blk, 4, 8, e)) * d) + m) for e in range(32)], dtype=F32)
 
 
+def q3k_scale(scales: np.ndarray, k: int) -> int:
+    """Stored 6-bit scale k (0..15) of a Q3_K super-block from its 12 scale bytes."""
+    lo = (int(scales[k]) & 15) if k < 8 else (int(scales[k - 8]) >> 4)
+    hi = (int(scales[8 + k % 4]) >> (2 * (k // 4))) & 3
+    return lo | (hi << 4)
+
+
+def decode_q3_k(blk: np.ndarray) -> np.ndarray:
+    hmask, qs, scales, d = blk[0:32], blk[32:96], blk[96:108], _f16(blk, 108)
+    out = np.empty(256, dtype=F32)
+    for e in range(256):
+        half, run, pos = e // 128, (e % 128) // 32, e % 32
+        field = (int(qs[32 * half + pos]) >> (2 * run)) & 3
+        third = (int(hmask[pos]) >> (4 * half + run)) & 1
+        k = e // 16
+        out[e] = F32(F32(d * F32(q3k_scale(scales, k) - 32)) * F32(field - (0 if third else 4)))
+    return out
+
+
 def q4k_scale_min(scales: np.ndarray, j: int):
     s = [int(v) for v in scales]
     if j < 4:
@@ -116,7 +135,8 @@ def decode_q6_k(blk: np.ndarray) -> np.ndarray:
 
 
 DECODERS = {8: (34, 32, decode_q8_0), 2: (18, 32, decode_q4_0), 12: (144, 256, decode_q4_k), 14: (210, 256, decode_q6_k),
-            13: (176, 256, decode_q5_k), 3: (20, 32, decode_q4_1), 6: (22, 32, decode_q5_0), 7: (24, 32, decode_q5_1)}
+            13: (176, 256, decode_q5_k), 3: (20, 32, decode_q4_1), 6: (22, 32, decode_q5_0), 7: (24, 32, decode_q5_1),
+            11: (110, 256, decode_q3_k)}
 
 
 def decode(ggml_type: int, raw: np.ndarray) -> np.ndarray:
@@ -178,6 +198,24 @@ def encode_q5_1(d, m, q) -> np.ndarray:
     blk = np.zeros(24, dtype=np.uint8)
     _put_f16(blk, 0, d); _put_f16(blk, 2, m)
     blk[8:], blk[4:8] = _legacy5_fields(q)
+    return blk
+
+
+def encode_q3_k(d, sc, q) -> np.ndarray:
+    """sc: 16 stored scales in 0..63 (the scale is sc - 32); q: 256 stored values in 0..7 (the element is q - 4)."""
+    blk = np.zeros(110, dtype=np.uint8)
+    q = np.asarray(q, dtype=np.uint8); sc = np.asarray(sc, dtype=np.uint8)
+    for e in range(256):
+        half, run, pos = e // 128, (e % 128) // 32, e % 32
+        blk[32 + 32 * half + pos] |= (int(q[e]) & 3) << (2 * run)
+        blk[pos] |= ((int(q[e]) >> 2) & 1) << (4 * half + run)
+    for k in range(16):
+        if k < 8:
+            blk[96 + k] |= int(sc[k]) & 15
+        else:
+            blk[96 + k - 8] |= (int(sc[k]) & 15) << 4
+        blk[96 + 8 + k % 4] |= ((int(sc[k]) >> 4) & 3) << (2 * (k // 4))
+    _put_f16(blk, 108, d)
     return blk
 
 

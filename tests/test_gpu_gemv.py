@@ -20,6 +20,8 @@ SHAPES = {
     "C3_down": (14, 4096, 11008),
     "q5_k_gate": (13, 11008, 4096),          # not a benchmark configuration: the Q5_K_M files' format, same shapes
     "q5_k_down": (13, 4096, 11008),
+    "q3_k_gate": (11, 11008, 4096),
+    "q3_k_down": (11, 4096, 11008),
     "q4_1_up": (3, 11008, 4096),             # the older 32-element formats with an offset and / or a fifth bit
     "q5_0_down": (6, 4096, 11008),
     "q5_1_q": (7, 4096, 4096),
@@ -57,10 +59,10 @@ def test_gemv_config_shapes_batch1_and_8(ex, orc, name):
     check(yo, y64[:2], wn, x[:2], name + " oracle f32 vs f64")
 
 
-@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 12, 13, 14, 1, 0])
+@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 11, 12, 13, 14, 1, 0])
 def test_gemv_edge_inputs(ex, orc, t):
     from rustorch_amd import synth
-    be = 256 if t in (12, 13, 14) else 32                  # unquantized rows: any multiple of 32 columns
+    be = 256 if t in (11, 12, 13, 14) else 32                  # unquantized rows: any multiple of 32 columns
     rows, cols = 5, 3 * be                                  # ragged: fewer rows than a tile, odd block count
     print("gemv edge", t, rows, cols, flush=True)
     raw = synth.blocks(t, 7, 1, rows, cols)

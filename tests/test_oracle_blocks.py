@@ -9,7 +9,7 @@ import pytest
 import np_blocks as nb
 
 GOLDEN = Path(__file__).resolve().parent / "golden" / "blocks_golden.npz"
-TYPES = [8, 2, 3, 6, 7, 12, 13, 14]
+TYPES = [8, 2, 3, 6, 7, 11, 12, 13, 14]
 
 
 def bits(a):
@@ -48,8 +48,8 @@ def test_f32_to_fp16_rne(orc):
 
 def test_block_geometry_matches_reference_type_size(orc):
     # example-cli/src/model/formats/gguf.rs:125-144
-    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 3, 6, 7, 8, 12, 13, 14)] == [4, 2, 18, 20, 22, 24, 34, 144, 176, 210]
-    assert [orc.load().orc_block_elems(t) for t in (2, 3, 6, 7, 8, 12, 13, 14)] == [32, 32, 32, 32, 32, 256, 256, 256]
+    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 3, 6, 7, 8, 11, 12, 13, 14)] == [4, 2, 18, 20, 22, 24, 34, 110, 144, 176, 210]
+    assert [orc.load().orc_block_elems(t) for t in (2, 3, 6, 7, 8, 11, 12, 13, 14)] == [32, 32, 32, 32, 32, 256, 256, 256, 256]
     assert orc.load().orc_row_bytes(12, 4096) == 2304 and orc.load().orc_row_bytes(14, 11008) == 9030
     assert orc.load().orc_row_bytes(12, 100) == 0
 
@@ -121,6 +121,33 @@ def test_q4_1_q5_0_q5_1_closed_forms(orc):
     blk[8 + 5] = 0x93                       # low nibble 3 -> element 5, high nibble 9 -> element 21
     y = orc.dequant(7, blk, 1, 32)[0]
     want = np.zeros(32, dtype=np.float32); want[5] = 3; want[21] = 9 + 16
+    assert np.array_equal(y, want)
+
+
+def test_q3_k_values_scales_and_positions(orc):
+    # every stored value 0..7 at a spread of positions, scale 33 (= +1) at the element's 16-group, 32 (= 0) elsewhere
+    for e in (0, 15, 16, 31, 32, 100, 127, 128, 143, 200, 255):
+        for v in range(8):
+            q = np.full(256, 4, dtype=np.uint8); q[e] = v            # 4 decodes to 0
+            sc = np.full(16, 32, dtype=np.uint8); sc[e // 16] = 33
+            y = orc.dequant(11, nb.encode_q3_k(2.0, sc, q), 1, 256)[0]
+            want = np.zeros(256, dtype=np.float32); want[e] = 2.0 * (v - 4)
+            assert np.array_equal(y, want), (e, v)
+    # every 6-bit scale at every one of the 16 places, with the complementary pattern next door
+    ones = np.full(256, 5, dtype=np.uint8)                           # every element +1
+    for k in range(16):
+        for s6 in range(64):
+            sc = np.full(16, 32, dtype=np.uint8); sc[k] = s6; sc[(k + 5) % 16] = 63 - s6
+            y = orc.dequant(11, nb.encode_q3_k(0.5, sc, ones), 1, 256)[0]
+            want = np.repeat((sc.astype(np.float32) - 32) * np.float32(0.5), 16)
+            assert np.array_equal(y, want), (k, s6)
+    # a hand-built block: one hmask bit, one 2-bit field, one scale nibble
+    blk = np.zeros(110, dtype=np.uint8); blk[108:110] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blk[96:108] = 0                                                  # all stored scales 0 -> scale -32
+    blk[7] = 1 << 5                                                  # third bit of element 128 + 32 + 7 (half 1, run 1)
+    blk[32 + 32 + 7] = 0b00001000                                    # its 2-bit field (run 1) = 2
+    y = orc.dequant(11, blk, 1, 256)[0]
+    want = np.full(256, -32.0 * -4.0, dtype=np.float32); want[128 + 32 + 7] = -32.0 * 2
     assert np.array_equal(y, want)
 
 
