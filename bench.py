@@ -176,10 +176,12 @@ def bench_prefill(ex, reps=20):
     from rustorch_amd import synth, GGMLType
     MFMA_PEAK = 2.5e15
     out = []
+    # the last two are not benchmark configurations: the fp16 contraction that serves the other formats, for the record
     for name, t, rows, cols in (("q4k_4096x4096", GGMLType.Q4_K, 4096, 4096), ("q4k_11008x4096", GGMLType.Q4_K, 11008, 4096),
-                                ("q6k_4096x11008", GGMLType.Q6_K, 4096, 11008)):
+                                ("q6k_4096x11008", GGMLType.Q6_K, 4096, 11008), ("q5k_4096x4096", GGMLType.Q5_K, 4096, 4096),
+                                ("f16_4096x4096", GGMLType.F16, 4096, 4096)):
         w = ex.upload_qweight(t, rows, cols, synth.blocks(t, SEED, 7000 + rows + cols, rows, cols))
-        for M in (64, 512, 2048):
+        for M in ((64, 512, 2048) if t in (GGMLType.Q4_K, GGMLType.Q6_K) else (512,)):
             x = ex.to_device(synth.normal(SEED, 7100 + M, M * cols))
             y = ex.buffer(4 * M * rows)
             for _ in range(3):

@@ -835,7 +835,7 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 bool qgemm_on_matrix_cores(int type, size_t M, size_t N, size_t K) { return mfma_path(type, N, K, M); }
 
 size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K) {
-    if (!mfma_path(type, N, K, M)) return 0;
+    if (!mfma_path(type, N, K, M)) return hgemm_serves(type, M, N, K) ? hgemm_scratch_bytes(type, M, N, K) : 0;
     GemmPlan p = gemm_plan(M, N, K);
     return align256(M * K * sizeof(_Float16)) + align256(M * sizeof(float)) + (p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0);
 }
@@ -905,7 +905,10 @@ hipError_t launch_qgemm(hipStream_t s, int type, const uint8_t *w, size_t N, siz
         if (type == RT_GGML_Q4_K) return launch_type<RT_GGML_Q4_K>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
         return launch_type<RT_GGML_Q6_K>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial);
     }
-    // Row-by-row form (small M, Q8_0 / Q4_0, in-place residual): the GEMV kernel, one grid slice per row of X.
+    // formats without a fused contraction: the fp16 matrix-core kernel over an fp16 copy of the weights
+    if (hgemm_serves(type, M, N, K) && scratch_bytes >= hgemm_scratch_bytes(type, M, N, K))
+        return launch_hgemm(s, type, w, N, K, row_bytes, X, M, Y, res, scratch, scratch_bytes);
+    // Row-by-row form (few rows, in-place residual of the fused contraction): the GEMV kernel, one grid slice per row of X.
     GemvArgs a;
     memset(&a, 0, sizeof a);
     a.n = 1;

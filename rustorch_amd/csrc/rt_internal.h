@@ -163,6 +163,13 @@ size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K);
 // true: launch_qgemm runs the matrix-core contraction (with its pre-pass of X); false: the GEMV kernel, one grid slice per row of X
 bool qgemm_on_matrix_cores(int type, size_t M, size_t N, size_t K);
 
+// fp16 contraction for the formats without a fused dequantizing kernel (rt_hgemm.hip): unquantized F16 weights as they
+// are, the others through an fp16 copy in the workspace.  res may be Y.
+bool hgemm_serves(int type, size_t M, size_t N, size_t K);
+size_t hgemm_scratch_bytes(int type, size_t M, size_t N, size_t K);
+hipError_t launch_hgemm(hipStream_t s, int type, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const float *X, size_t M, float *Y,
+                        const float *res, void *scratch, size_t scratch_bytes);
+
 // A matrix held as n partial planes: element i is base[i] + base[stride + i] + ... (summed in that order).
 // What a k-split contraction leaves behind; n = 1 is an ordinary matrix.
 struct PlaneSum {

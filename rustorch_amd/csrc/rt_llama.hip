@@ -291,9 +291,10 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
     hipStream_t s = ctx->stream;
     const rt_hip_llama_config &c = m->cfg;
     const size_t H = (size_t)c.hidden, F = (size_t)c.ffn;
-    size_t need = 0;
-    for (const auto *t : { &m->wq[0], &m->wo[0], &m->wgate[0], &m->wdown[0], &m->wv[0] })
-        need = std::max(need, rt::qgemm_scratch_bytes(t->type, M, t->n_rows, t->n_cols));
+    size_t need = 0;      // formats may differ from layer to layer (the common 4-bit files alternate Q4_K and Q6_K for v and down)
+    for (int l = 0; l < c.n_layers; l++)
+        for (const auto *t : { &m->wq[l], &m->wk[l], &m->wv[l], &m->wo[l], &m->wgate[l], &m->wup[l], &m->wdown[l] })
+            need = std::max(need, rt::qgemm_scratch_bytes(t->type, M, t->n_rows, t->n_cols));
     int rc = ensure_scratch(ctx, need);
     if (rc) return rc;
     float *x = m->pf_x, *x2 = m->pf_x2;

@@ -88,6 +88,38 @@ def test_other_formats_and_small_m_use_the_row_form(ex, orc):
             assert (np.abs(ex.qgemm(w, X) - y64) / (wn[None, :] * xn)).max() <= HELD * np.sqrt(4096 / cols)
 
 
+@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 11, 13, 1, 0])
+def test_formats_without_a_fused_contraction(ex, orc, t):
+    """From 32 rows of X on these formats go through the fp16 matrix-core kernel (F16 weights as they are, the others
+    through an fp16 copy of the exact block decode): the benchmark's FFN shape, then ragged shapes with extreme rows."""
+    from rustorch_amd import synth
+    rows, cols, M = 4096, 11008 if t in (11, 13) else 4096, 160
+    print("hgemm type", t, rows, cols, "M", M, flush=True)
+    raw = synth.blocks(t, 35, 7, rows, cols)
+    w = ex.upload_qweight(t, rows, cols, raw)
+    X = synth.normal(35, 100 + M, M * cols).reshape(M, cols)
+    Y = ex.qgemm(w, X)
+    rng = np.random.default_rng(t)
+    toks = np.sort(rng.choice(M, size=40, replace=False))
+    starts = sorted(set([0, rows - 64] + [int(v) for v in rng.integers(0, rows - 64, 3)]))
+    check(Y, [(s0, s0 + 64) for s0 in starts], toks, raw, t, rows, cols, X, orc, "type %d M=%d" % (t, M))
+    rows, cols = 1000, 1024 if t not in (1, 0) else 960          # N not a multiple of the wave tile; K = 15 * 64 for plain rows
+    raw = synth.blocks(t, 36, 1, rows, cols)
+    w = ex.upload_qweight(t, rows, cols, raw)
+    y_ref = None
+    for M in (32, 33, 100, 300):
+        X = synth.normal(36, M, M * cols).reshape(M, cols).copy()
+        X[0] *= 3e5; X[1] *= 1e-20; X[2] = 0; X[3, 5:] = 0
+        Y = ex.qgemm(w, X)
+        y64, wn = orc.qgemv_f64(t, raw, rows, cols, X)
+        xn = np.linalg.norm(X.astype(np.float64), axis=1)[:, None]
+        xn[xn == 0] = 1
+        ratio = np.abs(Y - y64) / (wn[None, :] * xn)
+        held = HELD * np.sqrt(4096 / cols)
+        assert np.isfinite(Y).all() and ratio.max() <= held, (M, ratio.max())
+        assert not Y[2].any()
+
+
 @pytest.mark.parametrize("t", [12, 14])
 @pytest.mark.parametrize("rows,cols,M", [(36, 256, 40), (4, 512, 130), (260, 768, 65), (512, 2816, 96)])
 def test_single_superblock_odd_counts_and_tiny_matrices(ex, orc, t, rows, cols, M):
