@@ -168,7 +168,8 @@ bool qgemm_on_matrix_cores(int type, size_t M, size_t N, size_t K);
 bool hgemm_serves(int type, size_t M, size_t N, size_t K);
 size_t hgemm_scratch_bytes(int type, size_t M, size_t N, size_t K);
 hipError_t launch_hgemm(hipStream_t s, int type, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const float *X, size_t M, float *Y,
-                        const float *res, void *scratch, size_t scratch_bytes);
+                        const float *res, void *scratch, size_t scratch_bytes, const _Float16 *w_f16 = nullptr);
+hipError_t launch_weights_f16(hipStream_t s, int type, const uint8_t *w, size_t N, size_t K, size_t row_bytes, _Float16 *out);
 
 // A matrix held as n partial planes: element i is base[i] + base[stride + i] + ... (summed in that order).
 // What a k-split contraction leaves behind; n = 1 is an ordinary matrix.

@@ -27,6 +27,7 @@ struct rt_hip_llama {
         int type = -1;
         size_t n_rows = 0, n_cols = 0, row_bytes = 0, nbytes = 0;
         uint8_t *dev = nullptr;
+        _Float16 *f16 = nullptr;    // fp16 copy, made when a batched prefill first meets a matrix whose format has no fused contraction
     };
     rt_hip_llama_config cfg{};
     int head_dim = 0;
@@ -217,8 +218,23 @@ int ensure_prefill_buffers(rt_hip_ctx *ctx, rt_hip_llama *m, size_t n_tok) {
 // share its pre-pass, which stays in the workspace until another matrix is prepared.
 struct PrefillGemm {
     rt_hip_ctx *ctx;
+    rt_hip_llama *m;
     const float *prepared = nullptr;
-    int operator()(const rt_hip_llama::T &t, const float *X, size_t M, float *Y, const float *res) {
+    int operator()(rt_hip_llama::T &t, const float *X, size_t M, float *Y, const float *res) {
+        if (rt::hgemm_serves(t.type, M, t.n_rows, t.n_cols)) {
+            // 288 GB of HBM: the fp16 copy (2 bytes per weight) is made once and stays beside the blocks, so later
+            // prompts skip the conversion
+            if (t.type != RT_GGML_F16 && !t.f16) {
+                void *p = nullptr;
+                int rc = dev_alloc(ctx, m, &p, t.n_rows * t.n_cols * sizeof(_Float16));
+                if (rc) return rc;
+                RT_TRY_HIP(ctx, rt::launch_weights_f16(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, (_Float16 *)p));
+                t.f16 = (_Float16 *)p;
+            }
+            RT_TRY_HIP(ctx, rt::launch_hgemm(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, X, M, Y, res, ctx->scratch,
+                                             ctx->scratch_bytes, t.f16));
+            return RT_HIP_OK;
+        }
         const bool mc = rt::qgemm_on_matrix_cores(t.type, M, t.n_rows, t.n_cols) && res != Y;
         RT_TRY_HIP(ctx, rt::launch_qgemm(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, X, M, Y, res, ctx->scratch, ctx->scratch_bytes,
                                          mc && prepared == X));
@@ -298,7 +314,7 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
     int rc = ensure_scratch(ctx, need);
     if (rc) return rc;
     float *x = m->pf_x, *x2 = m->pf_x2;
-    PrefillGemm gemm{ ctx };
+    PrefillGemm gemm{ ctx, m };
     RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, m->pf_tok, M, c.vocab, x));
     for (int l = 0; l < c.n_layers; l++) {
         uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
