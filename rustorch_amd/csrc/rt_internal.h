@@ -147,6 +147,9 @@ hipError_t launch_embed_rows(hipStream_t s, int type, const uint8_t *w, size_t r
                              const int *tokens_dev, size_t n_tok, int vocab, float *out);
 hipError_t launch_add(hipStream_t s, float *x, const float *y, size_t n);
 hipError_t launch_argmax(hipStream_t s, const float *v, size_t n, int *out_dev);
+// the greedy pick and the end of the decode step (as launch_step_advance) in one launch
+hipError_t launch_argmax_advance(hipStream_t s, const float *v, size_t n, int *pick_dev, int *pos_dev, int *token_dev, const int *forced_dev,
+                                 int *out_tokens_dev, int *step_dev);
 hipError_t launch_embed_row(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,
                             const int *token_dev, int vocab, float *out);
 hipError_t launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *c, size_t m, size_t n, size_t k);

@@ -553,14 +553,28 @@ __global__ void add_kernel(float *x, const float *y, size_t n) {
 }
 
 // Greedy pick; ties resolve to the lowest index.
-__global__ __launch_bounds__(1024) void argmax_kernel(const float *v, size_t n, int *out) {
+// A thread's candidates are loaded eight at a time before they are compared (independent loads, one round trip per
+// eight).  With `adv` the same launch ends the decode step: record the pick, choose the next input token, advance.
+struct StepAdvance {
+    int *pos_dev, *token_dev, *out_tokens_dev, *step_dev;
+    const int *forced_dev;
+    int enabled;
+};
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *v, size_t n, int *out, StepAdvance adv) {
     __shared__ float bv[1024];
     __shared__ int bi[1024];
     float best = -INFINITY;
     int idx = 0x7fffffff;
-    for (size_t i = threadIdx.x; i < n; i += blockDim.x) {
-        float f = v[i];
-        if (f > best) { best = f; idx = (int)i; }
+    for (size_t i0 = threadIdx.x; i0 < n; i0 += 8 * (size_t)blockDim.x) {
+        float f[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const size_t i = i0 + (size_t)u * blockDim.x;
+            f[u] = i < n ? v[i] : -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (f[u] > best) { best = f[u]; idx = (int)(i0 + (size_t)u * blockDim.x); }      // ascending index: the first of equals stays
     }
     bv[threadIdx.x] = best;
     bi[threadIdx.x] = idx;
@@ -576,7 +590,17 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *v, size_t n, 
         }
         __syncthreads();
     }
-    if (threadIdx.x == 0) *out = bi[0] == 0x7fffffff ? 0 : bi[0];
+    if (threadIdx.x == 0) {
+        const int pick = bi[0] == 0x7fffffff ? 0 : bi[0];
+        *out = pick;
+        if (adv.enabled) {
+            const int step = *adv.step_dev;
+            if (adv.out_tokens_dev) adv.out_tokens_dev[step] = pick;
+            *adv.token_dev = adv.forced_dev ? adv.forced_dev[step] : pick;
+            *adv.pos_dev = *adv.pos_dev + 1;
+            *adv.step_dev = step + 1;
+        }
+    }
 }
 
 __global__ void set_int_kernel(int *dst, int value) { *dst = value; }
@@ -826,7 +850,13 @@ hipError_t launch_add(hipStream_t s, float *x, const float *y, size_t n) {
 }
 
 hipError_t launch_argmax(hipStream_t s, const float *v, size_t n, int *out_dev) {
-    argmax_kernel<<<1, 1024, 0, s>>>(v, n, out_dev);
+    argmax_kernel<<<1, 1024, 0, s>>>(v, n, out_dev, StepAdvance{ nullptr, nullptr, nullptr, nullptr, nullptr, 0 });
+    return hipGetLastError();
+}
+
+hipError_t launch_argmax_advance(hipStream_t s, const float *v, size_t n, int *pick_dev, int *pos_dev, int *token_dev, const int *forced_dev,
+                                 int *out_tokens_dev, int *step_dev) {
+    argmax_kernel<<<1, 1024, 0, s>>>(v, n, pick_dev, StepAdvance{ pos_dev, token_dev, out_tokens_dev, step_dev, forced_dev, 1 });
     return hipGetLastError();
 }
 

@@ -541,8 +541,12 @@ static int enqueue_token(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits, boo
     auto enqueue = [&]() -> int {
         int rc = enqueue_step(ctx, m, want_logits);
         if (rc) return rc;
-        if (want_logits) RT_TRY_HIP(ctx, rt::launch_argmax(ctx->stream, m->logits, (size_t)m->cfg.vocab, m->state + 2));
-        if (advance)
+        if (want_logits && advance)
+            RT_TRY_HIP(ctx, rt::launch_argmax_advance(ctx->stream, m->logits, (size_t)m->cfg.vocab, m->state + 2, m->state + 0, m->state + 1,
+                                                      use_forced ? m->forced_dev : nullptr, m->out_tokens_dev, m->state + 3));
+        else if (want_logits)
+            RT_TRY_HIP(ctx, rt::launch_argmax(ctx->stream, m->logits, (size_t)m->cfg.vocab, m->state + 2));
+        else if (advance)
             RT_TRY_HIP(ctx, rt::launch_step_advance(ctx->stream, m->state + 0, m->state + 1, m->state + 2, use_forced ? m->forced_dev : nullptr,
                                                     m->out_tokens_dev, m->state + 3));
         return RT_HIP_OK;
