@@ -375,8 +375,9 @@ int rt_hip_llama_create(rt_hip_ctx *ctx, const rt_hip_llama_config *cfg, rt_hip_
     int rc = RT_HIP_OK;
     auto A = [&](void **p, size_t b) { if (rc == RT_HIP_OK) rc = dev_alloc(ctx, m, p, b); };
     // One workgroup per head serves a short cache; from RT_ATTN_SPLIT_MIN positions on, a head's positions are spread over
-    // up to eight workgroups of at least half that many each (a fixed shape per model, so a captured step stays valid).
-    m->attn_splits = cfg->max_pos >= RT_ATTN_SPLIT_MIN ? std::min(8, (cfg->max_pos + RT_ATTN_SPLIT_MIN / 2 - 1) / (RT_ATTN_SPLIT_MIN / 2)) : 1;
+    // up to sixteen workgroups of 128 positions or more each (a fixed shape per model, so a captured step stays valid;
+    // 64 positions per workgroup measured slower, 256 slower too).
+    m->attn_splits = cfg->max_pos >= RT_ATTN_SPLIT_MIN ? std::min(16, (cfg->max_pos + RT_ATTN_SPLIT_MIN / 4 - 1) / (RT_ATTN_SPLIT_MIN / 4)) : 1;
     A((void **)&m->attn_part, (size_t)cfg->n_heads * (size_t)m->attn_splits * (size_t)(hd + 2) * sizeof(float));
     A((void **)&m->kcache, L * P * m->kv_dim * 2); A((void **)&m->vcache, L * P * m->kv_dim * 2);
     A((void **)&m->x, H * 4); A((void **)&m->q, H * 4); A((void **)&m->k, H * 4); A((void **)&m->v, H * 4);
