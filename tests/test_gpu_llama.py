@@ -152,14 +152,14 @@ def test_long_context_attention_split_over_workgroups(ex, orc, n_heads, n_kv):
     from rustorch_amd import llama, synth
     base = dict(n_layers=2, hidden=256, n_heads=n_heads, ffn=512, vocab=300)
     print("llama long context", base, "n_kv", n_kv, flush=True)
-    split, om, wn = build_pair(ex, orc, 37, max_pos=600, n_kv_heads=n_kv, **base)       # 3 workgroups per head, 200 positions each
+    split, om, wn = build_pair(ex, orc, 37, max_pos=600, n_kv_heads=n_kv, **base)       # 5 workgroups per head, 120 positions each
     single = llama.HipLlama(ex, max_pos=500, n_kv_heads=n_kv, **base)
     llama.load_synthetic(single, 37)
     toks = synth.tokens(37, synth.TID_PROMPT, 420, base["vocab"])
     want = om.forward(toks, 0)
     tol = logit_tol(wn, base["hidden"])
     ratios, between = [], []
-    for n0 in (1, 192, 392):                      # the first steps, then across the chunk boundaries at 200 and 400
+    for n0 in (1, 112, 352):                      # the first steps, then across the chunk boundaries at 120 and 360
         split.reset(); single.reset()
         split.prefill(toks[:n0], 0); single.prefill(toks[:n0], 0)
         for p in range(n0, n0 + 14):
