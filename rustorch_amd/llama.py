@@ -168,7 +168,8 @@ def load_gguf(ex: HipKernelExecutor, path, max_pos: int | None = None) -> HipLla
         vocab = emb.dims[1]
         ctx = g.get_metadata("llama.context_length")
         if max_pos is None:
-            max_pos = ctx.as_u32() if ctx is not None and ctx.as_u32() else 2048
+            # the file's training context, capped at what the attention kernels hold per head (16 000 positions)
+            max_pos = min(ctx.as_u32() if ctx is not None and ctx.as_u32() else 2048, 16000)
         model = HipLlama(ex, n_layers, hidden, n_heads, ffn, vocab, max_pos, opt_f32("llama.attention.layer_norm_rms_epsilon", 1e-5),
                          opt_f32("llama.rope.freq_base", 10000.0), n_kv)
         try:

@@ -332,6 +332,14 @@ def test_model_from_gguf_file_equals_direct_upload(ex, orc, tmp_path):
         la, lb = gf.logits(), gm.logits()
         assert a == b and np.array_equal(la, lb)
         assert np.all(np.abs(la - want[pos]) <= tol)
+    # a training context beyond what the attention kernels hold is capped, an explicit one is taken as given
+    llama.write_synthetic_gguf(tmp_path / "long.gguf", 31, context=131072, **cfg)
+    gl = llama.load_gguf(ex, tmp_path / "long.gguf")
+    assert gl.cfg.max_pos == 16000
+    gl.close()
+    gl = llama.load_gguf(ex, tmp_path / "long.gguf", max_pos=600)
+    assert gl.cfg.max_pos == 600
+    gl.close()
     # a file without the block count is an error, not a guess
     from rustorch_amd import gguf
     w = gguf.GGUFWriter()
