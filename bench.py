@@ -147,12 +147,18 @@ def bench_single_gemv(ex, reps=200):
     return out
 
 
-def bench_decode(ex, n_prompt, n_gen):
+# A 70B-class shape for the record (--decode-shape 70b): 43 GB of blocks resident on the one GPU, grouped-query attention.
+SHAPES = {"7b": dict(NL=NL, H=H, NH=NH, NKV=NH, F=F, V=V), "70b": dict(NL=80, H=8192, NH=64, NKV=8, F=28672, V=32000)}
+
+
+def bench_decode(ex, n_prompt, n_gen, shape="7b"):
     from rustorch_amd import llama, synth
+    sh = SHAPES[shape]
+    NL, H, NH, NKV, F, V = sh["NL"], sh["H"], sh["NH"], sh["NKV"], sh["F"], sh["V"]
     t0 = time.time()
-    gm = llama.HipLlama(ex, NL, H, NH, F, V, n_prompt + n_gen)
+    gm = llama.HipLlama(ex, NL, H, NH, F, V, n_prompt + n_gen, n_kv_heads=NKV)
     wbytes = llama.load_synthetic(gm, SEED)
-    log("[bench] 7B-shaped model (%.2f GB of blocks) generated and uploaded in %.1f s" % (wbytes / 1e9, time.time() - t0))
+    log("[bench] %s-shaped model (%.2f GB of blocks) generated and uploaded in %.1f s" % (shape.upper(), wbytes / 1e9, time.time() - t0))
     prompt = synth.tokens(SEED, synth.TID_PROMPT, n_prompt, V)
     t0 = time.perf_counter()
     gm.prefill(prompt[:-1], 0)
@@ -163,10 +169,11 @@ def bench_decode(ex, n_prompt, n_gen):
     toks = gm.decode(int(prompt[-1]), n_prompt - 1, n_gen)
     t_dec = time.perf_counter() - t0
     gm.close()
-    per_layer = synth.layer_weight_bytes(H, F)
+    kv_dim = NKV * (H // NH)
+    per_layer = sum(t.row_bytes(c) * r for _, t, r, c in synth.layer_tensor_specs(H, F, kv_dim))
     tok_bytes = NL * per_layer + 210 * (H // 256) * V       # weights streamed per token (output head is Q6_K)
-    kv_avg = 2 * NL * H * 2 * (n_prompt + n_gen / 2)           # fp16 K and V rows read per token, averaged over the run
-    return dict(tokens_per_s=n_gen / t_dec, ms_per_token=1e3 * t_dec / n_gen, prefill_tokens_per_s=(n_prompt - 1) / t_prefill,
+    kv_avg = 2 * NL * kv_dim * 2 * (n_prompt + n_gen / 2)      # fp16 K and V rows read per token, averaged over the run
+    return dict(shape=shape, tokens_per_s=n_gen / t_dec, ms_per_token=1e3 * t_dec / n_gen, prefill_tokens_per_s=(n_prompt - 1) / t_prefill,
                 bytes_per_token=int(tok_bytes + kv_avg), hbm_frac=(tok_bytes + kv_avg) * n_gen / t_dec / HBM_PEAK,
                 n_prompt=n_prompt, n_generated=n_gen, first_tokens=[int(t) for t in toks[:8]])
 
@@ -236,6 +243,7 @@ def main():
     ap.add_argument("--prefill-only", action="store_true", help="run only the prefill contraction shapes (for kernel traces)")
     ap.add_argument("--decode-prompt", type=int, default=128)
     ap.add_argument("--decode-gen", type=int, default=128)
+    ap.add_argument("--decode-shape", choices=sorted(SHAPES), default="7b", help="model shape of the decode measurement (the benchmark's is 7b)")
     ap.add_argument("--calibrate", action="store_true",
                     help="run only a plain x += y kernel over 2 x 128 MiB (reads 256 MiB, writes 128 MiB per launch): "
                          "the known-size launch that hardware traffic counters are scaled by")
@@ -286,7 +294,7 @@ def main():
     if not args.no_prefill:
         out["prefill"] = bench_prefill(ex)
     if not args.no_decode:
-        out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen)
+        out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen, args.decode_shape)
     ex.close()
     if not args.no_cpu:
         wbytes, t1, tn, ncores = cpu_baseline(3)

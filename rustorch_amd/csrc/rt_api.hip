@@ -374,7 +374,7 @@ static int qgemv_check(rt_hip_ctx *ctx, const rt_hip_qweight *w, int batch) {
     RT_REQUIRE(ctx, w->n_cols % 32 == 0, RT_HIP_ERR_SHAPE, "qgemv: n_cols=%zu is not a multiple of 32", w->n_cols);
     RT_REQUIRE(ctx, batch >= 1 && batch <= 8, RT_HIP_ERR_INVALID_ARG, "qgemv: batch=%d outside 1..8 (use rt_hip_qgemm)", batch);
     RT_REQUIRE(ctx, w->n_rows < ((size_t)1 << 31) && w->n_cols < ((size_t)1 << 24), RT_HIP_ERR_SHAPE, "qgemv: tensor too large");
-    RT_REQUIRE(ctx, rt::gemv_lds_bytes(w->type, w->n_cols) <= 64 * 1024, RT_HIP_ERR_SHAPE, "qgemv: n_cols=%zu exceeds the LDS staging limit", w->n_cols);
+    RT_REQUIRE(ctx, rt::gemv_lds_bytes(w->type, w->n_cols) <= rt::kGemvLdsMax, RT_HIP_ERR_SHAPE, "qgemv: n_cols=%zu exceeds the LDS staging limit", w->n_cols);
     return RT_HIP_OK;
 }
 
@@ -474,7 +474,7 @@ int rt_hip_qgemm_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *X_de
     RT_REQUIRE(ctx, gemv_type_ok(w->type), RT_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: GGML type id %d has no kernel", w->type);
     RT_REQUIRE(ctx, w->n_cols % 32 == 0, RT_HIP_ERR_SHAPE, "qgemm: n_cols=%zu is not a multiple of 32", w->n_cols);
     RT_REQUIRE(ctx, M >= 1 && M <= 65535, RT_HIP_ERR_SHAPE, "qgemm: M=%zu outside 1..65535", M);
-    RT_REQUIRE(ctx, rt::gemv_lds_bytes(w->type, w->n_cols) <= 64 * 1024, RT_HIP_ERR_SHAPE, "qgemm: n_cols=%zu too large", w->n_cols);
+    RT_REQUIRE(ctx, rt::gemv_lds_bytes(w->type, w->n_cols) <= rt::kGemvLdsMax, RT_HIP_ERR_SHAPE, "qgemm: n_cols=%zu too large", w->n_cols);
     Guard g(ctx);
     size_t sb = rt::qgemm_scratch_bytes(w->type, M, w->n_rows, w->n_cols);
     int rc = ensure_scratch(ctx, sb);
@@ -489,7 +489,7 @@ int rt_hip_qgemm(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *X, size_
     RT_REQUIRE(ctx, gemv_type_ok(w->type), RT_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: GGML type id %d has no kernel", w->type);
     RT_REQUIRE(ctx, w->n_cols % 32 == 0, RT_HIP_ERR_SHAPE, "qgemm: n_cols=%zu is not a multiple of 32", w->n_cols);
     RT_REQUIRE(ctx, M >= 1 && M <= 65535, RT_HIP_ERR_SHAPE, "qgemm: M=%zu outside 1..65535", M);
-    RT_REQUIRE(ctx, rt::gemv_lds_bytes(w->type, w->n_cols) <= 64 * 1024, RT_HIP_ERR_SHAPE, "qgemm: n_cols=%zu too large", w->n_cols);
+    RT_REQUIRE(ctx, rt::gemv_lds_bytes(w->type, w->n_cols) <= rt::kGemvLdsMax, RT_HIP_ERR_SHAPE, "qgemm: n_cols=%zu too large", w->n_cols);
     Guard g(ctx);
     size_t xb = align_up(M * w->n_cols * 4, 256), yb = align_up(M * w->n_rows * 4, 256);
     size_t sb = rt::qgemm_scratch_bytes(w->type, M, w->n_rows, w->n_cols);

@@ -67,8 +67,22 @@ hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
         a.p[i].rows_per_tile = n;
         wgs += n;
     }
-    if (lds > 64 * 1024) return hipErrorInvalidValue;      // x of the longest row must fit the workgroup's LDS
+    if (lds > kGemvLdsMax) return hipErrorInvalidValue;    // x of the longest row must fit the workgroup's LDS
     dim3 grid((unsigned)wgs, (unsigned)batch);
+    if (lds > 64 * 1024) {
+        // rows longer than 27 000 elements (the 70B-class FFN): more than the default 64 KB of dynamic LDS, granted per
+        // kernel and device on request
+        static bool attr_set[2][64] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+        const int which = threads == 512 ? 0 : 1;
+        if (!attr_set[which][dev]) {
+            const void *fn = which == 0 ? (const void *)qgemv_kernel<512> : (const void *)qgemv_kernel<1024>;
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvLdsMax);
+            if (e != hipSuccess) return e;
+            attr_set[which][dev] = true;
+        }
+    }
     if (threads == 512) qgemv_kernel<512><<<grid, 512, lds, s>>>(a, r2);
     else qgemv_kernel<1024><<<grid, 1024, lds, s>>>(a, r2);
     return hipGetLastError();

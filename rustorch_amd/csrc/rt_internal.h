@@ -34,6 +34,8 @@ __host__ __device__ inline size_t xq_stride(size_t K) { return (2 * K + K / 8 + 
 // Unquantized weight matrices (F16 / F32) meet x as plain f32 in LDS; the block formats meet the two-plane integer form.
 __host__ __device__ inline bool gemv_float_weights(int type) { return type == 0 /* F32 */ || type == 1 /* F16 */; }
 __host__ __device__ inline size_t gemv_lds_bytes(int type, size_t K) { return gemv_float_weights(type) ? 4 * K : xq_stride(K); }
+// most LDS a GEMV workgroup may ask for x: the CU's 160 KB less the kernel's own few static bytes, with room to spare
+constexpr size_t kGemvLdsMax = 144 * 1024;
 
 // How a GEMV workgroup obtains the activation vector it stages into LDS.
 enum : int {

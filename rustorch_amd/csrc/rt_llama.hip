@@ -357,7 +357,7 @@ int rt_hip_llama_create(rt_hip_ctx *ctx, const rt_hip_llama_config *cfg, rt_hip_
     RT_REQUIRE(ctx, n_kv > 0 && cfg->n_heads % n_kv == 0, RT_HIP_ERR_SHAPE, "n_kv_heads=%d does not divide n_heads=%d", cfg->n_kv_heads, cfg->n_heads);
     RT_REQUIRE(ctx, cfg->hidden % 256 == 0 && cfg->ffn % 256 == 0, RT_HIP_ERR_SHAPE, "hidden=%d and ffn=%d must be multiples of 256", cfg->hidden, cfg->ffn);
     RT_REQUIRE(ctx, cfg->max_pos <= 16000, RT_HIP_ERR_SHAPE, "max_pos=%d exceeds 16000", cfg->max_pos);
-    RT_REQUIRE(ctx, rt::xq_stride((size_t)cfg->ffn) <= 64 * 1024 && rt::xq_stride((size_t)cfg->hidden) <= 64 * 1024, RT_HIP_ERR_SHAPE,
+    RT_REQUIRE(ctx, rt::xq_stride((size_t)cfg->ffn) <= rt::kGemvLdsMax && rt::xq_stride((size_t)cfg->hidden) <= rt::kGemvLdsMax, RT_HIP_ERR_SHAPE,
                "hidden / ffn exceed the GEMV staging limit");
     RT_REQUIRE(ctx, cfg->rms_eps >= 0.f && cfg->rope_theta > 0.f, RT_HIP_ERR_INVALID_ARG, "rms_eps=%g rope_theta=%g", (double)cfg->rms_eps,
                (double)cfg->rope_theta);
@@ -435,7 +435,7 @@ int rt_hip_llama_upload_tensor(rt_hip_ctx *ctx, rt_hip_llama *m, int slot, int l
         RT_REQUIRE(ctx, be != 0, RT_HIP_ERR_UNSUPPORTED_TYPE, "unsupported GGML type id %d", ggml_type);
         if (slot != RT_LLAMA_TOK_EMBD) {
             RT_REQUIRE(ctx, gemv_type_ok(ggml_type), RT_HIP_ERR_UNSUPPORTED_TYPE, "GGML type id %d has no GEMV kernel", ggml_type);
-            RT_REQUIRE(ctx, n_cols % 32 == 0 && rt::gemv_lds_bytes(ggml_type, n_cols) <= 64 * 1024, RT_HIP_ERR_SHAPE,
+            RT_REQUIRE(ctx, n_cols % 32 == 0 && rt::gemv_lds_bytes(ggml_type, n_cols) <= rt::kGemvLdsMax, RT_HIP_ERR_SHAPE,
                        "rows of %zu elements of type %d do not fit the GEMV's staging", n_cols, ggml_type);
         }
         RT_REQUIRE(ctx, n_cols % be == 0 && nbytes == n_rows * (n_cols / be) * bb, RT_HIP_ERR_SHAPE, "payload of %zu bytes does not match %zu x %zu of type %d",

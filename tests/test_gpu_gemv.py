@@ -83,6 +83,20 @@ def test_gemv_edge_inputs(ex, orc, t):
     assert np.all(np.abs(ex.qgemv(w, x2) - y64) <= TIGHT * np.linalg.norm(W, axis=1) * np.linalg.norm(x2))
 
 
+@pytest.mark.parametrize("t", [12, 14, 8])
+def test_rows_longer_than_the_default_lds(ex, orc, t):
+    """K = 28 672 (the feed-forward width of a 70B-class model): the staged x is 68 KB, beyond the 64 KB a kernel gets
+    without asking."""
+    from rustorch_amd import synth
+    rows, cols = 768, 28672
+    print("gemv long rows", t, rows, cols, flush=True)
+    raw = synth.blocks(t, 77, 3, rows, cols)
+    w = ex.upload_qweight(t, rows, cols, raw)
+    x = synth.normal(77, 4, 2 * cols).reshape(2, cols)
+    y64, wn = orc.qgemv_f64(t, raw, rows, cols, x)
+    check(ex.qgemv(w, x), y64, wn, x, "type %d K=%d" % (t, cols))
+
+
 def test_grouped_launch_equals_single_launches(ex, orc):
     from rustorch_amd import synth
     specs = [(12, 4096, 4096), (12, 512, 4096), (14, 4096, 4096), (14, 256, 11008), (8, 100, 4096)]

@@ -174,6 +174,30 @@ def test_long_context_attention_split_over_workgroups(ex, orc, n_heads, n_kv):
     assert np.median(ratios) <= 0.2
 
 
+def test_70b_class_widths(ex, orc):
+    """One layer with the widths of a 70B-class model (hidden 8192, 64 heads over 8 key / value heads, feed-forward
+    28 672): rows whose staged activations exceed the default 64 KB of LDS, and a feed-forward too wide for the fused
+    pre-pass of the chained prefill (it takes the general pass)."""
+    from rustorch_amd import synth
+    cfg = dict(n_layers=1, hidden=8192, n_heads=64, ffn=28672, vocab=256, max_pos=48)
+    print("llama 70b-class widths", cfg, flush=True)
+    gm, om, wn = build_pair(ex, orc, 43, n_kv_heads=8, **cfg)
+    toks = synth.tokens(43, synth.TID_PROMPT, 40, cfg["vocab"])
+    want = om.forward(toks, 0)
+    tol = logit_tol(wn, cfg["hidden"])
+    ratios = []
+    for p in range(8):
+        gm.step(int(toks[p]), p)
+        ratios.append(float((np.abs(gm.logits() - want[p]) / tol).max()))
+    gm.reset()
+    gm.prefill(toks[:36], 0)
+    ratios.append(float((np.abs(gm.logits() - want[35]) / tol).max()))
+    gm.step(int(toks[36]), 36)
+    ratios.append(float((np.abs(gm.logits() - want[36]) / tol).max()))
+    print("ratio to the tolerance: median %.3f, max %.2f" % (np.median(ratios), max(ratios)), flush=True)
+    assert np.median(ratios) <= 0.1 and max(ratios) <= 1.0
+
+
 def test_prefill_in_several_passes_and_calls(ex, orc):
     """A prompt longer than one pass of the batched prefill (512 tokens), the same prompt fed in two calls (the second
     starts at a position above zero) and token by token: the three device paths agree far inside the tolerance, and
