@@ -108,7 +108,8 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float *X, size_t K, _F
 }
 
 // ---- the pre-pass fused with the operation that produces the activation matrix.  A thread keeps its groups of the
-// row in registers from the first read to the conversion (rows of up to 256 * kXprepChunks * 8 elements).
+// row in registers from the first read to the conversion: rows of up to THREADS * kXprepChunks * 8 elements
+// (12 288 with 256 threads, 49 152 with 1024).
 __device__ __forceinline__ void plane_load8(const PlaneSum &p, size_t off, float *v) {
     const float4 a = *reinterpret_cast<const float4 *>(p.base + off), b = *reinterpret_cast<const float4 *>(p.base + off + 4);
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
@@ -129,9 +130,9 @@ struct RowSrc {
 
 constexpr int kPrepRms = 1, kPrepSwiglu = 2;
 
-template <int MODE>
-__global__ __launch_bounds__(256) void xprep_fused_kernel(RowSrc S, size_t K, _Float16 *Xp, float *inv_scale) {
-    __shared__ float red[4];
+template <int MODE, int THREADS>
+__global__ __launch_bounds__(THREADS) void xprep_fused_kernel(RowSrc S, size_t K, _Float16 *Xp, float *inv_scale) {
+    __shared__ float red[THREADS / 64];
     const size_t m = blockIdx.x, n_chunks = K / 8;
     auto src_of = [](size_t g) {
         const int sh = (int)(g & 7), s = sh >> 1, h = sh & 1;
@@ -141,7 +142,7 @@ __global__ __launch_bounds__(256) void xprep_fused_kernel(RowSrc S, size_t K, _F
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < kXprepChunks; j++) {
-        const size_t g = threadIdx.x + 256 * (size_t)j;
+        const size_t g = threadIdx.x + THREADS * (size_t)j;
         if (g < n_chunks) {
             const size_t off = m * K + src_of(g);
             if (MODE == kPrepRms) {
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(256) void xprep_fused_kernel(RowSrc S, size_t K, _F
         const float rms = sqrtf(ss / (float)K + S.eps);
 #pragma unroll
         for (int j = 0; j < kXprepChunks; j++) {
-            const size_t g = threadIdx.x + 256 * (size_t)j;
+            const size_t g = threadIdx.x + THREADS * (size_t)j;
             if (g < n_chunks) {
                 const float *gp = S.gamma + src_of(g);
                 const float4 a = *reinterpret_cast<const float4 *>(gp), b = *reinterpret_cast<const float4 *>(gp + 4);
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(256) void xprep_fused_kernel(RowSrc S, size_t K, _F
     float amax = 0.f;
 #pragma unroll
     for (int j = 0; j < kXprepChunks; j++) {
-        const size_t g = threadIdx.x + 256 * (size_t)j;
+        const size_t g = threadIdx.x + THREADS * (size_t)j;
         if (g < n_chunks)
 #pragma unroll
             for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[j][e]));
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(256) void xprep_fused_kernel(RowSrc S, size_t K, _F
     if (threadIdx.x == 0) inv_scale[m] = inv;
 #pragma unroll
     for (int j = 0; j < kXprepChunks; j++) {
-        const size_t g = threadIdx.x + 256 * (size_t)j;
+        const size_t g = threadIdx.x + THREADS * (size_t)j;
         if (g < n_chunks) {
             half8v o = { (_Float16)(v[j][0] * scale), (_Float16)(v[j][2] * scale), (_Float16)(v[j][1] * scale), (_Float16)(v[j][3] * scale),
                          (_Float16)(v[j][4] * scale), (_Float16)(v[j][6] * scale), (_Float16)(v[j][5] * scale), (_Float16)(v[j][7] * scale) };
@@ -855,14 +856,16 @@ hipError_t launch_xprep_rmsnorm(hipStream_t s, PlaneSum in, const float *res, fl
                                 _Float16 *Xp, float *inv_scale) {
     if (M == 0 || K == 0 || K % 256 != 0 || K > kXprepFusedMaxK || in.n < 1 || !in.base || !gamma) return hipErrorInvalidValue;
     RowSrc S{ in, PlaneSum{ nullptr, 0, 0 }, res, x_out, gamma, eps };
-    xprep_fused_kernel<kPrepRms><<<dim3((unsigned)M), 256, 0, s>>>(S, K, Xp, inv_scale);
+    if (K <= 256 * kXprepChunks * 8) xprep_fused_kernel<kPrepRms, 256><<<dim3((unsigned)M), 256, 0, s>>>(S, K, Xp, inv_scale);
+    else xprep_fused_kernel<kPrepRms, 1024><<<dim3((unsigned)M), 1024, 0, s>>>(S, K, Xp, inv_scale);
     return hipGetLastError();
 }
 
 hipError_t launch_xprep_swiglu(hipStream_t s, PlaneSum gate, PlaneSum up, size_t M, size_t K, _Float16 *Xp, float *inv_scale) {
     if (M == 0 || K == 0 || K % 256 != 0 || K > kXprepFusedMaxK || gate.n < 1 || up.n < 1 || !gate.base || !up.base) return hipErrorInvalidValue;
     RowSrc S{ gate, up, nullptr, nullptr, nullptr, 0.f };
-    xprep_fused_kernel<kPrepSwiglu><<<dim3((unsigned)M), 256, 0, s>>>(S, K, Xp, inv_scale);
+    if (K <= 256 * kXprepChunks * 8) xprep_fused_kernel<kPrepSwiglu, 256><<<dim3((unsigned)M), 256, 0, s>>>(S, K, Xp, inv_scale);
+    else xprep_fused_kernel<kPrepSwiglu, 1024><<<dim3((unsigned)M), 1024, 0, s>>>(S, K, Xp, inv_scale);
     return hipGetLastError();
 }
 

@@ -187,7 +187,7 @@ struct PlaneSum {
 // operation that produces the activation matrix), the contraction without the reduction of its k splits, and consumers
 // that read plane sums.  Xp: M x K fp16 (scaled, k-permuted), inv_scale: M floats; K a multiple of 256.
 size_t qgemm_planes_bytes(int type, size_t M, size_t N, size_t K);             // planes a contraction of this shape may write
-constexpr size_t kXprepFusedMaxK = 12288;                                       // longest row the fused producers keep in registers
+constexpr size_t kXprepFusedMaxK = 49152;                                       // longest row the fused producers keep in registers
 hipError_t launch_xprep(hipStream_t s, const float *X, size_t M, size_t K, _Float16 *Xp, float *inv_scale);
 // x = in (+ res), stored to x_out when given; prepared matrix = gamma * x / sqrt(mean(x^2) + eps)
 hipError_t launch_xprep_rmsnorm(hipStream_t s, PlaneSum in, const float *res, float *x_out, const float *gamma, float eps, size_t M, size_t K,

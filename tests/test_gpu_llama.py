@@ -176,8 +176,8 @@ def test_long_context_attention_split_over_workgroups(ex, orc, n_heads, n_kv):
 
 def test_70b_class_widths(ex, orc):
     """One layer with the widths of a 70B-class model (hidden 8192, 64 heads over 8 key / value heads, feed-forward
-    28 672): rows whose staged activations exceed the default 64 KB of LDS, and a feed-forward too wide for the fused
-    pre-pass of the chained prefill (it takes the general pass)."""
+    28 672): rows whose staged activations exceed the default 64 KB of LDS, and a feed-forward wide enough for the
+    1024-thread form of the fused pre-pass in the chained prefill."""
     from rustorch_amd import synth
     cfg = dict(n_layers=1, hidden=8192, n_heads=64, ffn=28672, vocab=256, max_pos=48)
     print("llama 70b-class widths", cfg, flush=True)
