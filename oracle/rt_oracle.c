@@ -22,7 +22,7 @@
  * What the reference does NOT hold and this file therefore owns (parity with
  * the reference is unpinned for these; they are pinned by closed forms,
  * exhaustive packer round trips and an independent NumPy decoder in tests/):
- *   - the Q8_0 / Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q3_K / Q4_K / Q5_K / Q6_K block decoders.  The reference only fixes
+ *   - the Q8_0 / Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q2_K / Q3_K / Q4_K / Q5_K / Q6_K block decoders.  The reference only fixes
  *     type ids and block byte sizes (example-cli/src/model/formats/gguf.rs:78-144)
  *     and decodes every quantized type with a placeholder
  *     (tensor_loader.rs:125-141,213-218).  The layouts below are the public
@@ -43,7 +43,7 @@
 
 #define ORC_API __attribute__((visibility("default")))
 
-enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q4_1 = 3, ORC_Q5_0 = 6, ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q3_K = 11, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };
+enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q4_1 = 3, ORC_Q5_0 = 6, ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q2_K = 10, ORC_Q3_K = 11, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };
 
 /* ------------------------------------------------------------------ fp16 */
 
@@ -105,7 +105,7 @@ static inline uint16_t rd_u16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1]
 ORC_API int orc_block_elems(int type) {
     switch (type) {
     case ORC_Q8_0: case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: return 32;
-    case ORC_Q3_K: case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 256;
+    case ORC_Q2_K: case ORC_Q3_K: case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 256;
     case ORC_F32: case ORC_F16: return 1;
     default: return 0;
     }
@@ -119,6 +119,7 @@ ORC_API int orc_block_bytes(int type) {
     case ORC_Q4_1: return 20;
     case ORC_Q5_0: return 22;
     case ORC_Q5_1: return 24;
+    case ORC_Q2_K: return 84;   /* the public ggml block; the table at gguf.rs:137 lists 82 */
     case ORC_Q3_K: return 110;
     case ORC_Q4_K: return 144;
     case ORC_Q5_K: return 176;
@@ -181,6 +182,27 @@ static void deq_q5_1(const uint8_t *b, float *y) {
         int x1 = (int)((qs[j] >> 4) | ((qh >> (j + 12)) & 0x10));
         y[j] = (float)x0 * d + m;
         y[j + 16] = (float)x1 * d + m;
+    }
+}
+
+/* Q2_K: { u8 scales[16]; u8 qs[64]; f16 d; f16 dmin } (84 B, type id 10, gguf.rs:88): per 16 elements a scale byte whose
+ * low nibble scales d and whose high nibble scales dmin; values are 2-bit fields of qs. */
+static void deq_q2_k(const uint8_t *b, float *y) {
+    const uint8_t *sc = b, *q = b + 16;
+    float d = orc_h2f(rd_u16(b + 80)), mn = orc_h2f(rd_u16(b + 82));
+    int is = 0;
+    for (int n = 0; n < 256; n += 128) {
+        int shift = 0;
+        for (int j = 0; j < 4; j++) {
+            uint8_t s = sc[is++];
+            float dl = d * (float)(s & 0xF), ml = mn * (float)(s >> 4);
+            for (int l = 0; l < 16; l++) *y++ = dl * (float)((q[l] >> shift) & 3) - ml;
+            s = sc[is++];
+            dl = d * (float)(s & 0xF); ml = mn * (float)(s >> 4);
+            for (int l = 0; l < 16; l++) *y++ = dl * (float)((q[l + 16] >> shift) & 3) - ml;
+            shift += 2;
+        }
+        q += 32;
     }
 }
 
@@ -299,6 +321,7 @@ static void deq_row(int type, const uint8_t *row, size_t n_cols, float *y) {
     case ORC_Q4_1: for (size_t b = 0; b < n_cols / 32; b++) deq_q4_1(row + 20 * b, y + 32 * b); break;
     case ORC_Q5_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q5_0(row + 22 * b, y + 32 * b); break;
     case ORC_Q5_1: for (size_t b = 0; b < n_cols / 32; b++) deq_q5_1(row + 24 * b, y + 32 * b); break;
+    case ORC_Q2_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q2_k(row + 84 * b, y + 256 * b); break;
     case ORC_Q3_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q3_k(row + 110 * b, y + 256 * b); break;
     case ORC_Q4_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q4_k(row + 144 * b, y + 256 * b); break;
     case ORC_Q5_K: for (size_t b = 0; b < n_cols / 256; b++) deq_q5_k(row + 176 * b, y + 256 * b); break;

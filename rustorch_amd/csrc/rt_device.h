@@ -105,6 +105,15 @@ __device__ inline float deq_elem(int type, const uint8_t *row, size_t col) {
         int q = (j < 16 ? (b[8 + j] & 0x0F) : (b[8 + j - 16] >> 4)) | (((b[4 + (j >> 3)] >> (j & 7)) & 1) << 4);
         return (float)q * d + m;
     }
+    case RT_GGML_Q2_K: {       // { u8 scales[16]; u8 qs[64]; f16 d; f16 dmin }: 2-bit values, per 16 elements a 4-bit scale and a 4-bit minimum
+        const uint8_t *b = row + 84 * (col >> 8);
+        int e = (int)(col & 255);
+        int n = e >> 7, j = (e >> 5) & 3, l = e & 31;
+        uint8_t sc = b[8 * n + 2 * j + (l >> 4)];
+        float dl = h2f(ld2u(b + 80)) * (float)(sc & 0xF), ml = h2f(ld2u(b + 82)) * (float)(sc >> 4);
+        int q = (b[16 + 32 * n + l] >> (2 * j)) & 3;
+        return dl * (float)q - ml;
+    }
     case RT_GGML_Q3_K: {       // { u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d }: 2 low bits in qs, the third in hmask, 16 six-bit scales
         const uint8_t *b = row + 110 * (col >> 8);
         int e = (int)(col & 255);

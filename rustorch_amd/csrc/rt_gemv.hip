@@ -41,7 +41,8 @@ hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
     size_t lds = 0, total_rows = 0;
     for (int i = 0; i < a.n; i++) {
         if ((double)a.p[i].N * (double)a.p[i].row_bytes >= 4294967296.0) return hipErrorInvalidValue;   // row offsets are 32-bit
-        if ((a.p[i].type == RT_GGML_Q5_K || a.p[i].type == RT_GGML_Q3_K) && a.p[i].epi == kEpiSwiglu) return hipErrorInvalidValue;   // no pair form for these
+        if ((a.p[i].type == RT_GGML_Q5_K || a.p[i].type == RT_GGML_Q3_K || a.p[i].type == RT_GGML_Q2_K) && a.p[i].epi == kEpiSwiglu)
+            return hipErrorInvalidValue;   // no pair form for these
         total_bytes += (double)a.p[i].N * (double)a.p[i].row_bytes * (a.p[i].epi == kEpiSwiglu ? 2.0 : 1.0);
         total_rows += (size_t)a.p[i].N;
         lds = std::max(lds, gemv_lds_bytes(a.p[i].type, (size_t)a.p[i].K));

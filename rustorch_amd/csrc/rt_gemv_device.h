@@ -30,7 +30,7 @@ namespace rt {
 __device__ __forceinline__ int units_of(int type, int K) {
     if (type == RT_GGML_F16) return K / 8;
     if (type == RT_GGML_F32) return K / 4;
-    return (type == RT_GGML_Q3_K || type == RT_GGML_Q4_K || type == RT_GGML_Q5_K || type == RT_GGML_Q6_K) ? K / 64 : K / 32;
+    return (type == RT_GGML_Q2_K || type == RT_GGML_Q3_K || type == RT_GGML_Q4_K || type == RT_GGML_Q5_K || type == RT_GGML_Q6_K) ? K / 64 : K / 32;
 }
 
 // dword index inside a plane (xh or xl) of the 4 elements starting at e (e % 4 == 0)
@@ -38,7 +38,7 @@ __device__ __forceinline__ int x_slot_dword(int type, int e, int U) {
     int j = e >> 4, w = (e >> 2) & 3;
     int slot;
     if (type == RT_GGML_Q4_K || type == RT_GGML_Q5_K) slot = (j & 3) * U + (j >> 2);
-    else if (type == RT_GGML_Q6_K || type == RT_GGML_Q3_K) slot = ((j >> 1) & 3) * U + (2 * (j >> 3) + (j & 1));
+    else if (type == RT_GGML_Q6_K || type == RT_GGML_Q3_K || type == RT_GGML_Q2_K) slot = ((j >> 1) & 3) * U + (2 * (j >> 3) + (j & 1));
     else slot = (j & 1) * U + (j >> 1);
     return slot * 4 + w;
 }
@@ -46,7 +46,7 @@ __device__ __forceinline__ int x_slot_dword(int type, int e, int U) {
 // Place 4 quantized elements and the block metadata they carry into the per-type LDS layout.
 //   planes: xh at dword 0, xl at dword K/4; floats S from dword K/2:
 //   Q4_K, Q5_K : S[4u + {0,1}] = scale of the unit's two 32-blocks, S[4u + {2,3}] = scale * sum of each block
-//   Q6_K, Q3_K : S[b] = scale of 32-block b (= 4 * half + run);  S[2U + 4u + r] = scale * sum of the unit's run r
+//   Q6_K, Q3_K, Q2_K : S[b] = scale of 32-block b (= 4 * half + run);  S[2U + 4u + r] = scale * sum of the unit's run r
 //   Q8_0 : S[u] = scale;   Q4_0 : S[2u] = scale, S[2u+1] = scale * sum of the block
 __device__ __forceinline__ void stage_store(int type, int K, int U, uint32_t *lds, int e, uint32_t hi, uint32_t lo,
                                             float s, float bsum16, float bsum32) {
@@ -60,7 +60,7 @@ __device__ __forceinline__ void stage_store(int type, int K, int U, uint32_t *ld
             S[4 * u + half] = s;
             S[4 * u + 2 + half] = bsum32;
         }
-    } else if (type == RT_GGML_Q6_K || type == RT_GGML_Q3_K) {
+    } else if (type == RT_GGML_Q6_K || type == RT_GGML_Q3_K || type == RT_GGML_Q2_K) {
         if ((e & 31) == 0) S[e >> 5] = s;
         if ((e & 15) == 0) {
             int i16 = e >> 4;
@@ -159,6 +159,9 @@ template <> struct XRegs<RT_GGML_Q4_0> { uint4 h[2], l[2]; float2 sv; };
 // the same x slice; 16 bytes of 2-bit fields, 16 bytes of third bits, the 12 scale bytes, d
 template <> struct WRegs<RT_GGML_Q3_K> { uint4 Q, H; uint2 s01; uint32_t s2, d; };
 template <> struct XRegs<RT_GGML_Q3_K> : XRegs<RT_GGML_Q6_K> {};
+// Q2_K: the same unit and x slice again; 16 bytes of 2-bit fields, the eight scale bytes of the half, d | dmin << 16
+template <> struct WRegs<RT_GGML_Q2_K> { uint4 Q; uint2 sc; uint32_t dm; };
+template <> struct XRegs<RT_GGML_Q2_K> : XRegs<RT_GGML_Q6_K> {};
 // unquantized rows: 16 bytes of weights per unit against the f32 x in LDS
 template <> struct WRegs<RT_GGML_F16> { uint4 q; };
 template <> struct XRegs<RT_GGML_F16> { float4 a, b; };
@@ -216,6 +219,12 @@ __device__ __forceinline__ void load_w(WRegs<RT_GGML_Q6_K> &w, WRow row, int u) 
     w.H = bld16(row, off + 128u + 32u * h + 16u * c);
     w.sc = bld8(row, off + 192u + 8u * h);
     w.d = bld2(row, off + 208u);
+}
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q2_K> &w, WRow row, int u) {
+    uint32_t off = (uint32_t)(u >> 2) * 84u, n = (uint32_t)((u >> 1) & 1), c = (uint32_t)(u & 1);
+    w.sc = bld8(row, off + 8u * n);
+    w.Q = bld16(row, off + 16u + 32u * n + 16u * c);
+    w.dm = bld4(row, off + 80u);
 }
 __device__ __forceinline__ void load_w(WRegs<RT_GGML_Q3_K> &w, WRow row, int u) {
     uint32_t off = (uint32_t)(u >> 2) * 110u, n = (uint32_t)((u >> 1) & 1), c = (uint32_t)(u & 1);
@@ -275,6 +284,9 @@ __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q6_K> &x, const uint32_t *l
     const float *S = reinterpret_cast<const float *>(lds + K / 2);
     x.xs = reinterpret_cast<const float4 *>(S)[u >> 1];
     x.xb = reinterpret_cast<const float4 *>(S + 2 * U)[u];
+}
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q2_K> &x, const uint32_t *lds, int u, int U, int K) {
+    load_x(static_cast<XRegs<RT_GGML_Q6_K> &>(x), lds, u, U, K);
 }
 __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q3_K> &x, const uint32_t *lds, int u, int U, int K) {
     load_x(static_cast<XRegs<RT_GGML_Q6_K> &>(x), lds, u, U, K);
@@ -416,6 +428,36 @@ __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q6_K> &w, const XR
     a = __builtin_fmaf(sc2, __builtin_fmaf(x.xs.z, (float)((dh[2] << 7) + dl[2]), -32.f * x.xb.z), a);
     a = __builtin_fmaf(sc3, __builtin_fmaf(x.xs.w, (float)((dh[3] << 7) + dl[3]), -32.f * x.xb.w), a);
     return h2f(w.d) * a;
+}
+
+// Q2_K: run j of the unit holds the 2-bit fields j of 16 bytes; its scale byte is number 2 j + c of the half's eight
+// (low nibble: scale, high nibble: minimum).  y = d * scale * q - dmin * minimum.
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q2_K> &w, const XRegs<RT_GGML_Q2_K> &x, int u) {
+    const int c = u & 1;
+    const uint32_t Q[4] = RT_W4(w.Q);
+    const uint32_t h0[4] = RT_W4(x.h[0]), h1[4] = RT_W4(x.h[1]), h2[4] = RT_W4(x.h[2]), h3[4] = RT_W4(x.h[3]);
+    const uint32_t l0[4] = RT_W4(x.l[0]), l1[4] = RT_W4(x.l[1]), l2[4] = RT_W4(x.l[2]), l3[4] = RT_W4(x.l[3]);
+    int dh[4] = { 0, 0, 0, 0 }, dl[4] = { 0, 0, 0, 0 };
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t q0 = Q[i] & 0x03030303u, q1 = (Q[i] >> 2) & 0x03030303u, q2 = (Q[i] >> 4) & 0x03030303u, q3 = (Q[i] >> 6) & 0x03030303u;
+        dh[0] = sdot4(q0, (int)h0[i], dh[0]);  dl[0] = sdot4(q0, (int)l0[i], dl[0]);
+        dh[1] = sdot4(q1, (int)h1[i], dh[1]);  dl[1] = sdot4(q1, (int)l1[i], dl[1]);
+        dh[2] = sdot4(q2, (int)h2[i], dh[2]);  dl[2] = sdot4(q2, (int)l2[i], dl[2]);
+        dh[3] = sdot4(q3, (int)h3[i], dh[3]);  dl[3] = sdot4(q3, (int)l3[i], dl[3]);
+    }
+    const uint32_t b01 = w.sc.x >> (8 * c), b23 = w.sc.y >> (8 * c);      // bytes c, c + 2 of each word: runs 0, 1 | 2, 3
+    const float s0 = (float)(b01 & 0xFu), s1 = (float)((b01 >> 16) & 0xFu), s2 = (float)(b23 & 0xFu), s3 = (float)((b23 >> 16) & 0xFu);
+    const float m0 = (float)((b01 >> 4) & 0xFu), m1 = (float)((b01 >> 20) & 0xFu), m2 = (float)((b23 >> 4) & 0xFu), m3 = (float)((b23 >> 20) & 0xFu);
+    float pos = s0 * (x.xs.x * (float)((dh[0] << 7) + dl[0]));
+    pos = __builtin_fmaf(s1, x.xs.y * (float)((dh[1] << 7) + dl[1]), pos);
+    pos = __builtin_fmaf(s2, x.xs.z * (float)((dh[2] << 7) + dl[2]), pos);
+    pos = __builtin_fmaf(s3, x.xs.w * (float)((dh[3] << 7) + dl[3]), pos);
+    float neg = m0 * x.xb.x;
+    neg = __builtin_fmaf(m1, x.xb.y, neg);
+    neg = __builtin_fmaf(m2, x.xb.z, neg);
+    neg = __builtin_fmaf(m3, x.xb.w, neg);
+    return __builtin_fmaf(h2f(w.dm & 0xFFFFu), pos, -(h2f(w.dm >> 16) * neg));
 }
 
 // Run j of the unit: stored value v = 2-bit field j of the byte | third bit (bit 4 n + j of the hmask byte) << 2, element = v - 4;
@@ -665,12 +707,14 @@ __device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg
 // Dispatch on the block format.  R2 picks two rows per wave step (always used by the SwiGLU epilogue).
 template <bool COH, bool ALLOW_R2>
 __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_wg, int m, bool r2, uint32_t *lds, float *red) {
-    // 80 / 48 bytes of registers per row and unit: Q5_K and Q3_K run one row per step (two would spill); the launcher
+    // Q5_K, Q3_K and Q2_K run one row per step (with a two-row form of any of them the kernel as a whole spills); the launcher
     // refuses the gate / up pair form for them, the caller issues gate and up as two problems and a separate SwiGLU
     if (P.type == RT_GGML_Q5_K) {
         gemv_problem<RT_GGML_Q5_K, 1, COH>(P, wg, n_wg, m, lds, red);
     } else if (P.type == RT_GGML_Q3_K) {
         gemv_problem<RT_GGML_Q3_K, 1, COH>(P, wg, n_wg, m, lds, red);
+    } else if (P.type == RT_GGML_Q2_K) {
+        gemv_problem<RT_GGML_Q2_K, 1, COH>(P, wg, n_wg, m, lds, red);
     } else if ((ALLOW_R2 && r2) || P.epi == kEpiSwiglu) {
         switch (P.type) {
         case RT_GGML_Q4_K: gemv_problem<RT_GGML_Q4_K, 2, COH>(P, wg, n_wg, m, lds, red); break;

@@ -9,6 +9,7 @@
 //   Q4_1 20 B / 32 el : f16 d; f16 m; u8 qs[16]                 (q * d + m)
 //   Q5_0 22 B / 32 el : f16 d; u8 qh[4]; u8 qs[16]              (bit j of qh = fifth bit of element j; (q - 16) * d)
 //   Q5_1 24 B / 32 el : f16 d; f16 m; u8 qh[4]; u8 qs[16]
+//   Q2_K 84 B / 256   : u8 scales[16]; u8 qs[64]; f16 d; f16 dmin
 //   Q3_K 110 B / 256  : u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d
 //   Q4_K 144 B / 256  : f16 d; f16 dmin; u8 scales[12]; u8 qs[128]
 //   Q5_K 176 B / 256  : f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]

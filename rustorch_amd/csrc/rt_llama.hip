@@ -152,7 +152,8 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
         a.p[0] = make_prob(m->wo[l], m->xq_a, rt::kStageXq, m->x, m->x);
         RT_TRY_HIP(ctx, rt::launch_qgemv(s, a, 1));
         memset(&a, 0, sizeof a);
-        if (m->wgate[l].type == m->wup[l].type && m->wgate[l].type != RT_GGML_Q5_K && m->wgate[l].type != RT_GGML_Q3_K) {
+        if (m->wgate[l].type == m->wup[l].type && m->wgate[l].type != RT_GGML_Q5_K && m->wgate[l].type != RT_GGML_Q3_K &&
+            m->wgate[l].type != RT_GGML_Q2_K) {
             a.n = 1;
             a.p[0] = make_prob(m->wgate[l], m->x, rt::kStageRms, m->g, nullptr);
             a.p[0].w2 = m->wup[l].dev; a.p[0].epi = rt::kEpiSwiglu; a.p[0].gamma = m->ffn_norm[l]; a.p[0].eps = c.rms_eps;
@@ -184,7 +185,7 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
 
 bool gemv_type_ok(int t) {
     return t == RT_GGML_F32 || t == RT_GGML_F16 || t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_1 || t == RT_GGML_Q5_0 ||
-           t == RT_GGML_Q5_1 || t == RT_GGML_Q3_K || t == RT_GGML_Q4_K || t == RT_GGML_Q5_K || t == RT_GGML_Q6_K;
+           t == RT_GGML_Q5_1 || t == RT_GGML_Q2_K || t == RT_GGML_Q3_K || t == RT_GGML_Q4_K || t == RT_GGML_Q5_K || t == RT_GGML_Q6_K;
 }
 
 constexpr size_t kPrefillChunk = 512;     // tokens per pass of the batched prefill

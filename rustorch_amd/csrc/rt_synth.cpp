@@ -9,6 +9,7 @@
 //   Q4_0 : w0 -> d;  w1,w2 -> the 16 qs bytes verbatim
 //   Q4_1 : w0 -> d from u24(r), m = -8 d' with d' from u24(r >> 32);  w1,w2 -> qs
 //   Q5_0 : w0 -> d, qh = bits 32..63 of r;  w1,w2 -> qs        Q5_1 : w0 -> d, m = -16 d';  w1,w2 -> qs;  w3 -> qh (low 32 bits)
+//   Q2_K : w0,w1 -> the 16 scale bytes verbatim;  w2..w9 -> qs;  w10 -> d from u24(r), dmin from u24(r >> 32)
 //   Q3_K : w0..w3 -> hmask;  w4..w11 -> qs;  w12 and the low half of w13 -> the 12 scale bytes verbatim;  w14 -> d
 //   Q4_K : w0 -> d from u24(r), dmin from u24(r >> 32);  w1 -> 8 scales (byte & 63);
 //          w2 -> 8 mins (byte & 63), packed into the 12-byte field;  w3..w18 -> qs
@@ -116,6 +117,13 @@ void gen_block(int type, uint64_t key, uint64_t b, double lo, double hi, uint8_t
         std::memcpy(o + 4, &qh, 4);
         put64(o + 8, mix(base + 1));
         put64(o + 16, mix(base + 2));
+        break;
+    }
+    case RT_GGML_Q2_K: {
+        for (int w = 0; w < 10; w++) put64(o + 8 * w, mix(base + w));
+        uint64_t r = mix(base + 10);
+        put16(o + 80, scale_f16(lo, hi, u24(r)));
+        put16(o + 82, scale_f16(lo, hi, u24(r >> 32)));
         break;
     }
     case RT_GGML_Q3_K: {

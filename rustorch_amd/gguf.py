@@ -56,7 +56,8 @@ class GGMLType(enum.IntEnum):
 _TYPE_SIZE = {
     GGMLType.F32: 4, GGMLType.I32: 4, GGMLType.F16: 2, GGMLType.I16: 2, GGMLType.I8: 1,
     GGMLType.Q4_0: 18, GGMLType.Q4_1: 20, GGMLType.Q5_0: 22, GGMLType.Q5_1: 24, GGMLType.Q8_0: 34,
-    GGMLType.Q8_1: 36, GGMLType.Q2_K: 82, GGMLType.Q3_K: 110, GGMLType.Q4_K: 144, GGMLType.Q5_K: 176,
+    GGMLType.Q8_1: 36, GGMLType.Q2_K: 84,   # the public ggml block (16 + 64 + 2 * 2); the reference's table lists 82
+    GGMLType.Q3_K: 110, GGMLType.Q4_K: 144, GGMLType.Q5_K: 176,
     GGMLType.Q6_K: 210, GGMLType.Q8_K: 292,
 }
 

@@ -20,6 +20,7 @@ D_RANGE = {
     GGMLType.Q4_1: (1e-3, 2e-2),      # offsets m are drawn from -8 * this range (Q5_1: -16 *)
     GGMLType.Q5_0: (5e-4, 1e-2),
     GGMLType.Q5_1: (5e-4, 1e-2),
+    GGMLType.Q2_K: (1e-3, 1e-2),
     GGMLType.Q3_K: (1e-3, 1e-2),
     GGMLType.Q4_K: (1e-3, 1e-2),
     GGMLType.Q5_K: (1e-3, 1e-2),

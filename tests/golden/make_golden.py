@@ -30,7 +30,7 @@ def main() -> None:
     for t, (bb, be, fn) in nb.DECODERS.items():
         n = 12
         raw = rng.integers(0, 256, size=(n, bb), dtype=np.uint8)
-        d_off = [208] if t == 14 else [108] if t == 11 else ([0, 2] if t in (12, 13, 3, 7) else [0])     # d (and dmin / m) fields
+        d_off = [208] if t == 14 else [108] if t == 11 else [80, 82] if t == 10 else ([0, 2] if t in (12, 13, 3, 7) else [0])     # d (and dmin / m) fields
         scales = rng.uniform(1e-3, 1e-2, size=(n, len(d_off)))
         for i in range(n):
             for k, off in enumerate(d_off):

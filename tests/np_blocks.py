@@ -61,6 +61,29 @@ def decode_q5_1(blk: np.ndarray) -> np.ndarray:
     return np.array([F32(F32(F32(_legacy5(blk, 4, 8, e)) * d) + m) for e in range(32)], dtype=F32)
 
 
+def decode_q2_k(blk: np.ndarray) -> np.ndarray:
+    scales, qs, d, dmin = blk[0:16], blk[16:80], _f16(blk, 80), _f16(blk, 82)
+    out = np.empty(256, dtype=F32)
+    for e in range(256):
+        half, run, pos = e // 128, (e % 128) // 32, e % 32
+        field = (int(qs[32 * half + pos]) >> (2 * run)) & 3
+        s = int(scales[e // 16])
+        out[e] = F32(F32(F32(d * F32(s & 15)) * F32(field)) - F32(dmin * F32(s >> 4)))
+    return out
+
+
+def encode_q2_k(d, dmin, sc, mn, q) -> np.ndarray:
+    """sc, mn: 16 four-bit scales and minima; q: 256 values in 0..3; the element is d * sc * q - dmin * mn."""
+    blk = np.zeros(84, dtype=np.uint8)
+    sc = np.asarray(sc, dtype=np.uint8); mn = np.asarray(mn, dtype=np.uint8); q = np.asarray(q, dtype=np.uint8)
+    blk[0:16] = (sc & 15) | ((mn & 15) << 4)
+    for e in range(256):
+        half, run, pos = e // 128, (e % 128) // 32, e % 32
+        blk[16 + 32 * half + pos] |= (int(q[e]) & 3) << (2 * run)
+    _put_f16(blk, 80, d); _put_f16(blk, 82, dmin)
+    return blk
+
+
 def q3k_scale(scales: np.ndarray, k: int) -> int:
     """Stored 6-bit scale k (0..15) of a Q3_K super-block from its 12 scale bytes."""
     lo = (int(scales[k]) & 15) if k < 8 else (int(scales[k - 8]) >> 4)
@@ -136,7 +159,7 @@ def decode_q6_k(blk: np.ndarray) -> np.ndarray:
 
 DECODERS = {8: (34, 32, decode_q8_0), 2: (18, 32, decode_q4_0), 12: (144, 256, decode_q4_k), 14: (210, 256, decode_q6_k),
             13: (176, 256, decode_q5_k), 3: (20, 32, decode_q4_1), 6: (22, 32, decode_q5_0), 7: (24, 32, decode_q5_1),
-            11: (110, 256, decode_q3_k)}
+            11: (110, 256, decode_q3_k), 10: (84, 256, decode_q2_k)}
 
 
 def decode(ggml_type: int, raw: np.ndarray) -> np.ndarray:

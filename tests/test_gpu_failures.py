@@ -46,7 +46,7 @@ def test_refused_arguments_leave_a_message_and_a_working_context(ex, orc):
     with pytest.raises(InvalidParameters):
         ex.qgemv_dev(w, ex.to_device(np.zeros(256, np.float32)), ex.buffer(32), 0)      # batch 0
     with pytest.raises(UnsupportedOperation):
-        ex.upload_qweight(10, 8, 256, np.zeros(8 * 84, np.uint8))                        # Q2_K: no kernel
+        ex.upload_qweight(15, 8, 256, np.zeros(8 * 292, np.uint8))                       # Q8_K: no kernel
     with pytest.raises(ShapeMismatch):
         ex.attn_decode(np.zeros(2 * 96, np.float32), np.zeros((4, 192), np.uint16), np.zeros((4, 192), np.uint16), 4, 2, 96)   # head_dim 96
     still_works(ex, orc)

@@ -88,12 +88,12 @@ def test_other_formats_and_small_m_use_the_row_form(ex, orc):
             assert (np.abs(ex.qgemm(w, X) - y64) / (wn[None, :] * xn)).max() <= HELD * np.sqrt(4096 / cols)
 
 
-@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 11, 13, 1, 0])
+@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 10, 11, 13, 1, 0])
 def test_formats_without_a_fused_contraction(ex, orc, t):
     """From 32 rows of X on these formats go through the fp16 matrix-core kernel (F16 weights as they are, the others
     through an fp16 copy of the exact block decode): the benchmark's FFN shape, then ragged shapes with extreme rows."""
     from rustorch_amd import synth
-    rows, cols, M = 4096, 11008 if t in (11, 13) else 4096, 160
+    rows, cols, M = 4096, 11008 if t in (10, 11, 13) else 4096, 160
     print("hgemm type", t, rows, cols, "M", M, flush=True)
     raw = synth.blocks(t, 35, 7, rows, cols)
     w = ex.upload_qweight(t, rows, cols, raw)

@@ -233,7 +233,7 @@ def test_prefill_in_several_passes_and_calls(ex, orc):
     assert np.median(ratios) <= 0.2
 
 
-@pytest.mark.parametrize("fmt", ["Q5_K", "Q8_0", "Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q3_K", "F16", "F32"])
+@pytest.mark.parametrize("fmt", ["Q5_K", "Q8_0", "Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q2_K", "Q3_K", "F16", "F32"])
 def test_model_in_a_format_without_matrix_core_path(ex, orc, fmt):
     """All seven matrices of every layer in one format that the dense contraction does not serve.  Decode: the GEMV
     kernels (Q5_K: one row per step, gate and up as two problems of one launch followed by the separate SwiGLU).

@@ -9,7 +9,7 @@ import pytest
 import np_blocks as nb
 
 GOLDEN = Path(__file__).resolve().parent / "golden" / "blocks_golden.npz"
-TYPES = [8, 2, 3, 6, 7, 11, 12, 13, 14]
+TYPES = [8, 2, 3, 6, 7, 10, 11, 12, 13, 14]
 
 
 def bits(a):
@@ -48,8 +48,8 @@ def test_f32_to_fp16_rne(orc):
 
 def test_block_geometry_matches_reference_type_size(orc):
     # example-cli/src/model/formats/gguf.rs:125-144
-    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 3, 6, 7, 8, 11, 12, 13, 14)] == [4, 2, 18, 20, 22, 24, 34, 110, 144, 176, 210]
-    assert [orc.load().orc_block_elems(t) for t in (2, 3, 6, 7, 8, 11, 12, 13, 14)] == [32, 32, 32, 32, 32, 256, 256, 256, 256]
+    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 3, 6, 7, 8, 10, 11, 12, 13, 14)] == [4, 2, 18, 20, 22, 24, 34, 84, 110, 144, 176, 210]
+    assert [orc.load().orc_block_elems(t) for t in (2, 3, 6, 7, 8, 10, 11, 12, 13, 14)] == [32, 32, 32, 32, 32, 256, 256, 256, 256, 256]
     assert orc.load().orc_row_bytes(12, 4096) == 2304 and orc.load().orc_row_bytes(14, 11008) == 9030
     assert orc.load().orc_row_bytes(12, 100) == 0
 
@@ -121,6 +121,35 @@ def test_q4_1_q5_0_q5_1_closed_forms(orc):
     blk[8 + 5] = 0x93                       # low nibble 3 -> element 5, high nibble 9 -> element 21
     y = orc.dequant(7, blk, 1, 32)[0]
     want = np.zeros(32, dtype=np.float32); want[5] = 3; want[21] = 9 + 16
+    assert np.array_equal(y, want)
+
+
+def test_q2_k_values_scales_and_positions(orc):
+    # every value 0..3 at a spread of positions; scale 3 at the element's 16-group, 0 elsewhere; no minimum
+    for e in (0, 15, 16, 31, 32, 100, 127, 128, 143, 200, 255):
+        for v in range(4):
+            q = np.zeros(256, dtype=np.uint8); q[e] = v
+            sc = np.zeros(16, dtype=np.uint8); sc[e // 16] = 3
+            others = np.full(256, 3, dtype=np.uint8); others[16 * (e // 16):16 * (e // 16) + 16] = 0; others[e] = v   # groups with scale 0 hold 3s
+            y = orc.dequant(10, nb.encode_q2_k(2.0, 1.0, sc, np.zeros(16, np.uint8), others), 1, 256)[0]
+            want = np.zeros(256, dtype=np.float32); want[e] = 2.0 * 3 * v
+            assert np.array_equal(y, want), (e, v)
+    # every (scale, minimum) nibble pair at every one of the 16 places
+    ones = np.ones(256, dtype=np.uint8)
+    for k in range(16):
+        for s4 in range(16):
+            sc = np.zeros(16, dtype=np.uint8); mn = np.zeros(16, dtype=np.uint8)
+            sc[k] = s4; mn[k] = 15 - s4; sc[(k + 5) % 16] = 15 - s4; mn[(k + 5) % 16] = s4
+            y = orc.dequant(10, nb.encode_q2_k(0.5, 0.25, sc, mn, ones), 1, 256)[0]
+            want = np.repeat(sc.astype(np.float32) * np.float32(0.5) - mn.astype(np.float32) * np.float32(0.25), 16)
+            assert np.array_equal(y, want), (k, s4)
+    # a hand-built block: one scale byte, one 2-bit field
+    blk = np.zeros(84, dtype=np.uint8)
+    blk[80:82] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8); blk[82:84] = np.frombuffer(np.float16(2.0).tobytes(), np.uint8)
+    blk[8 + 2 + 1] = 0x35                                            # half 1, run 1, second 16: scale 5, minimum 3
+    blk[16 + 32 + 20] = 0b00001100                                   # byte 20 of half 1: field of run 1 = 3
+    y = orc.dequant(10, blk, 1, 256)[0]
+    want = np.zeros(256, dtype=np.float32); want[128 + 32 + 16:128 + 32 + 32] = -6.0; want[128 + 32 + 20] = 5 * 3 - 6.0
     assert np.array_equal(y, want)
 
 

@@ -47,6 +47,9 @@ def ref_block(t, seed, tid, b, lo, hi):
     if t == 7:
         w = words(seed, tid, b, 4)
         return np.concatenate([scale(lo, hi, w[0]), scale(-16.0 * lo, -16.0 * hi, int(w[0]) >> 32), w[3:4].view(np.uint8)[:4], w[1:3].view(np.uint8)])
+    if t == 10:
+        w = words(seed, tid, b, 11)
+        return np.concatenate([w[:10].view(np.uint8), scale(lo, hi, w[10]), scale(lo, hi, int(w[10]) >> 32)])
     if t == 11:
         w = words(seed, tid, b, 15)
         return np.concatenate([w[:13].view(np.uint8), w[13:14].view(np.uint8)[:4], scale(lo, hi, w[14])])
@@ -65,7 +68,7 @@ def ref_block(t, seed, tid, b, lo, hi):
     return np.concatenate([w[:24].view(np.uint8), sc, scale(lo, hi, w[26])])
 
 
-@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 11, 12, 13, 14])
+@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 10, 11, 12, 13, 14])
 def test_blocks_follow_the_specification(lib, t):
     from rustorch_amd import synth, GGMLType
     lo, hi = synth.D_RANGE[GGMLType(t)]
