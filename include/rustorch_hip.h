@@ -47,7 +47,9 @@ typedef enum {
     RT_HIP_ERR_UNSUPPORTED_TYPE = 6
 } rt_hip_status;
 
-/* GGML type ids, the values of GGMLType (example-cli/src/model/formats/gguf.rs:78-99). */
+/* GGML type ids, the values of GGMLType (example-cli/src/model/formats/gguf.rs:78-99).  The ids listed here have the exact
+ * dequantization and a GEMV kernel; Q4_K and Q6_K also have the fused matrix-core contraction, the others reach the matrix
+ * cores through an fp16 copy.  Any other id is refused with RT_HIP_ERR_UNSUPPORTED_TYPE. */
 typedef enum {
     RT_GGML_F32 = 0,
     RT_GGML_F16 = 1,
