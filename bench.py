@@ -151,6 +151,37 @@ def bench_single_gemv(ex, reps=200):
 SHAPES = {"7b": dict(NL=NL, H=H, NH=NH, NKV=NH, F=F, V=V), "70b": dict(NL=80, H=8192, NH=64, NKV=8, F=28672, V=32000)}
 
 
+def bench_batch8(ex, reps=100):
+    """Config C3 at M = 8: the three layer shapes with eight activation rows per launch (the batch-1 kernel run per row as
+    grid slices; the weights of rows 2..8 come from L2 / Infinity Cache).  Weight GB/s counts the weights once."""
+    from rustorch_amd import synth, GGMLType
+    out = []
+    for name, t, rows, cols in (("q4k_4096x4096", GGMLType.Q4_K, 4096, 4096), ("q4k_11008x4096", GGMLType.Q4_K, 11008, 4096),
+                                ("q6k_4096x11008", GGMLType.Q6_K, 4096, 11008)):
+        ws = [ex.upload_qweight(t, rows, cols, synth.blocks(t, SEED, 9000 + i, rows, cols)) for i in range(8)]
+        x = ex.to_device(synth.normal(SEED, 9100, 8 * cols))
+        y = ex.buffer(4 * 8 * rows)
+        res = {}
+        for batch in (1, 8):
+            for i in range(8):
+                ex.qgemv_dev(ws[i % 8], x, y, batch)
+            ex.synchronize()
+            e0, e1 = ex.event(), ex.event()
+            e0.record()
+            for i in range(reps):
+                ex.qgemv_dev(ws[i % 8], x, y, batch)
+            e1.record()
+            ex.synchronize()
+            res[batch] = e0.elapsed_ms(e1) / reps
+        wbytes = t.row_bytes(cols) * rows
+        out.append({"shape": name, "us_batch1": round(res[1] * 1e3, 2), "us_batch8": round(res[8] * 1e3, 2),
+                    "weight_gbps_batch8": round(wbytes / res[8] / 1e6, 1), "rows_per_s_batch8": round(8 / (res[8] * 1e-3))})
+        for w in ws:
+            w.free()
+        x.free(); y.free()
+    return out
+
+
 def bench_decode(ex, n_prompt, n_gen, shape="7b"):
     from rustorch_amd import llama, synth
     sh = SHAPES[shape]
@@ -293,6 +324,7 @@ def main():
     out["single_gemv"] = bench_single_gemv(ex)
     if not args.no_prefill:
         out["prefill"] = bench_prefill(ex)
+        out["batch8"] = bench_batch8(ex)
     if not args.no_decode:
         out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen, args.decode_shape)
     ex.close()
