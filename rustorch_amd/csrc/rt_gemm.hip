@@ -602,7 +602,7 @@ template <int TYPE, int NW, int MF>
 __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t row_bytes, int N, int K, const _Float16 *Xp,
                                                         const float *inv_scale, int M, float *Y_out, size_t plane_stride,
                                                         const float *res, int sb_per_split, int ksplit, int tiles_n,
-                                                        int n_tiles_total, int per_xcd) {
+                                                        int n_tiles_total, int per_xcd, const uint8_t *W2, float *Y2, int tiles_one) {
     using Geo = WGeo<TYPE>;
     constexpr int BM = 32 * MF, BN = 32 * NW, XI = BM / 8 / NW;
     static_assert(XI >= 1 && XI * 8 * NW == BM, "every wave issues whole 8-row LDS-DMA loads");
@@ -610,8 +610,14 @@ __global__ __launch_bounds__(64 * NW) void qgemm_kernel(const uint8_t *W, size_t
     RT_DYN_LDS(_Float16, xs);
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, nl = lane & 31, h = lane >> 5;
     // tile of this workgroup
-    const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
     if ((int)(blockIdx.x >> 3) >= per_xcd || t >= n_tiles_total) return;
+    // a second weight matrix of the same shape against the same X (q and k, gate and up): its tiles follow the first one's
+    if (t >= tiles_one) {
+        t -= tiles_one;
+        W = W2;
+        Y_out = Y2;
+    }
     const int slab = t / tiles_n, nt = t - slab * tiles_n;
     const int mt = slab / ksplit, kz = slab - mt * ksplit;
     const int n0 = nt * BN, m0 = mt * BM;
@@ -776,10 +782,11 @@ struct GemmPlan { int mf, ksplit, sb_per_split; };
 constexpr int kGemmWaves = 8;     // waves per workgroup: two per SIMD, one workgroup per CU
 
 // Shape of the launch: token fragments per wave (tile 32*mf tokens x 256 rows) and k splits.
-GemmPlan gemm_plan(size_t M, size_t N, size_t K) {
+GemmPlan gemm_plan(size_t M, size_t N, size_t K, int matrices = 1) {
     GemmPlan p;
     p.mf = M > 64 ? 4 : 2;
-    const size_t bm = 32 * (size_t)p.mf, tiles = ((M + bm - 1) / bm) * ((N + 32 * kGemmWaves - 1) / (32 * kGemmWaves)), nsb = K / 256;
+    const size_t bm = 32 * (size_t)p.mf, nsb = K / 256;
+    const size_t tiles = (size_t)matrices * ((M + bm - 1) / bm) * ((N + 32 * kGemmWaves - 1) / (32 * kGemmWaves));
     // split k while that fills more of the 256 CUs in whole rounds and leaves every split at least two super-blocks
     p.ksplit = 1;
     while (tiles * p.ksplit * 2 <= 256 && nsb / (p.ksplit * 2) >= 2 && p.ksplit < kMaxSplit) p.ksplit *= 2;
@@ -790,7 +797,8 @@ GemmPlan gemm_plan(size_t M, size_t N, size_t K) {
 
 template <int TYPE, int NW, int MF>
 hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const _Float16 *Xp,
-                      const float *inv_scale, size_t M, float *Y, const float *res, float *partial, bool reduce) {
+                      const float *inv_scale, size_t M, float *Y, const float *res, float *partial, bool reduce, const uint8_t *w2 = nullptr,
+                      float *planes2 = nullptr) {
     constexpr int BM = 32 * MF, BN = 32 * NW;
     const size_t lds = (size_t)4 * BM * kBK * sizeof(_Float16) + (size_t)NW * WGeo<TYPE>::stage_bytes;
     auto kern = qgemm_kernel<TYPE, NW, MF>;
@@ -803,11 +811,11 @@ hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t
         attr_set[dev] = true;
     }
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
-    const int total = tiles_m * p.ksplit * tiles_n;
+    const int one = tiles_m * p.ksplit * tiles_n, total = w2 ? 2 * one : one;
     const int per_xcd = (total + 7) / 8;
     const size_t plane = M * N;
     kern<<<dim3((unsigned)(8 * per_xcd)), 64 * NW, lds, s>>>(w, row_bytes, (int)N, (int)K, Xp, inv_scale, (int)M, p.ksplit > 1 ? partial : Y,
-                                                             plane, res, p.sb_per_split, p.ksplit, tiles_n, total, per_xcd);
+                                                             plane, res, p.sb_per_split, p.ksplit, tiles_n, total, per_xcd, w2, planes2, one);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || p.ksplit == 1 || !reduce) return e;
     const size_t n4 = plane / 4;
@@ -818,9 +826,10 @@ hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t
 
 template <int TYPE>
 hipError_t launch_type(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const _Float16 *Xp,
-                       const float *inv_scale, size_t M, float *Y, const float *res, float *partial, bool reduce = true) {
-    if (p.mf == 4) return launch_cfg<TYPE, kGemmWaves, 4>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial, reduce);
-    return launch_cfg<TYPE, kGemmWaves, 2>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial, reduce);
+                       const float *inv_scale, size_t M, float *Y, const float *res, float *partial, bool reduce = true,
+                       const uint8_t *w2 = nullptr, float *planes2 = nullptr) {
+    if (p.mf == 4) return launch_cfg<TYPE, kGemmWaves, 4>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial, reduce, w2, planes2);
+    return launch_cfg<TYPE, kGemmWaves, 2>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial, reduce, w2, planes2);
 }
 
 bool mfma_path(int type, size_t N, size_t K, size_t M) {
@@ -878,6 +887,21 @@ hipError_t launch_qgemm_planes(hipStream_t s, int type, const uint8_t *w, size_t
     *out = PlaneSum{ planes, M * N, p.ksplit };
     if (type == RT_GGML_Q4_K) return launch_type<RT_GGML_Q4_K>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, planes, nullptr, planes, false);
     return launch_type<RT_GGML_Q6_K>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, planes, nullptr, planes, false);
+}
+
+// Two weight matrices of one shape and format against the same prepared X in one launch (q and k, gate and up): the tiles of
+// both fill the CUs together, so k is split less than for either alone.
+hipError_t launch_qgemm_planes2(hipStream_t s, int type, const uint8_t *wa, const uint8_t *wb, size_t N, size_t K, size_t row_bytes,
+                                const _Float16 *Xp, const float *inv_scale, size_t M, float *planes_a, float *planes_b, size_t planes_bytes,
+                                PlaneSum *out_a, PlaneSum *out_b) {
+    if (!mfma_path(type, N, K, M) || !out_a || !out_b || !wa || !wb) return hipErrorInvalidValue;
+    const GemmPlan p = gemm_plan(M, N, K, 2);
+    if ((size_t)p.ksplit * M * N * sizeof(float) > planes_bytes) return hipErrorInvalidValue;
+    *out_a = PlaneSum{ planes_a, M * N, p.ksplit };
+    *out_b = PlaneSum{ planes_b, M * N, p.ksplit };
+    if (type == RT_GGML_Q4_K)
+        return launch_type<RT_GGML_Q4_K>(s, p, wa, N, K, row_bytes, Xp, inv_scale, M, planes_a, nullptr, planes_a, false, wb, planes_b);
+    return launch_type<RT_GGML_Q6_K>(s, p, wa, N, K, row_bytes, Xp, inv_scale, M, planes_a, nullptr, planes_a, false, wb, planes_b);
 }
 
 hipError_t launch_plane_sum(hipStream_t s, PlaneSum in, const float *res, float *Y, size_t n) {

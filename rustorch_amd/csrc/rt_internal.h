@@ -196,6 +196,10 @@ hipError_t launch_xprep_rmsnorm(hipStream_t s, PlaneSum in, const float *res, fl
 hipError_t launch_xprep_swiglu(hipStream_t s, PlaneSum gate, PlaneSum up, size_t M, size_t K, _Float16 *Xp, float *inv_scale);
 hipError_t launch_qgemm_planes(hipStream_t s, int type, const uint8_t *w, size_t N, size_t K, size_t row_bytes, const _Float16 *Xp,
                                const float *inv_scale, size_t M, float *planes, size_t planes_bytes, PlaneSum *out);
+// the same for two weight matrices of one shape and format in one launch
+hipError_t launch_qgemm_planes2(hipStream_t s, int type, const uint8_t *wa, const uint8_t *wb, size_t N, size_t K, size_t row_bytes,
+                                const _Float16 *Xp, const float *inv_scale, size_t M, float *planes_a, float *planes_b, size_t planes_bytes,
+                                PlaneSum *out_a, PlaneSum *out_b);
 // Y = in (+ res), n elements (a multiple of 4)
 hipError_t launch_plane_sum(hipStream_t s, PlaneSum in, const float *res, float *Y, size_t n);
 // rope_kv_batch with q, k, v given as plane sums; the rotated q goes to q_out

@@ -270,6 +270,15 @@ int enqueue_prefill_chain(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
     auto mm = [&](const rt_hip_llama::T &t, float *planes, rt::PlaneSum *out) {
         return rt::launch_qgemm_planes(s, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, m->pf_xp, m->pf_inv, M, planes, m->pf_planes_bytes, out);
     };
+    // two matrices of one shape and format that meet the same prepared X (q and k without grouped-query attention, gate and up)
+    // go out as one launch
+    auto same_kind = [](const rt_hip_llama::T &a, const rt_hip_llama::T &b) {
+        return a.type == b.type && a.n_rows == b.n_rows && a.n_cols == b.n_cols && a.row_bytes == b.row_bytes;
+    };
+    auto mm2 = [&](const rt_hip_llama::T &a, const rt_hip_llama::T &b, float *pa, float *pb, rt::PlaneSum *oa, rt::PlaneSum *ob) {
+        return rt::launch_qgemm_planes2(s, a.type, a.dev, b.dev, a.n_rows, a.n_cols, a.row_bytes, m->pf_xp, m->pf_inv, M, pa, pb, m->pf_planes_bytes,
+                                        oa, ob);
+    };
     RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, m->pf_tok, M, c.vocab, x));
     rt::PlaneSum pending{ x, 0, 1 };             // what the next RMSNorm reads: first the embeddings themselves,
     const float *pending_res = nullptr;          // later the planes of a down-projection, to be added to x
@@ -278,16 +287,24 @@ int enqueue_prefill_chain(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
         uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
         rt::PlaneSum q, k, v, o, g, u, d;
         RT_TRY_HIP(ctx, rt::launch_xprep_rmsnorm(s, pending, pending_res, pending_res ? x : nullptr, m->attn_norm[l], c.rms_eps, M, H, m->pf_xp, m->pf_inv));
-        RT_TRY_HIP(ctx, mm(m->wq[l], P[0], &q));
-        RT_TRY_HIP(ctx, mm(m->wk[l], P[1], &k));
+        if (same_kind(m->wq[l], m->wk[l])) {
+            RT_TRY_HIP(ctx, mm2(m->wq[l], m->wk[l], P[0], P[1], &q, &k));
+        } else {
+            RT_TRY_HIP(ctx, mm(m->wq[l], P[0], &q));
+            RT_TRY_HIP(ctx, mm(m->wk[l], P[1], &k));
+        }
         RT_TRY_HIP(ctx, mm(m->wv[l], P[2], &v));
         RT_TRY_HIP(ctx, rt::launch_rope_kv_planes(s, q, k, v, m->pf_q, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
         RT_TRY_HIP(ctx, rt::launch_attn_causal(s, m->pf_q, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->pf_a));
         RT_TRY_HIP(ctx, rt::launch_xprep(s, m->pf_a, M, H, m->pf_xp, m->pf_inv));
         RT_TRY_HIP(ctx, mm(m->wo[l], P[0], &o));
         RT_TRY_HIP(ctx, rt::launch_xprep_rmsnorm(s, o, x, x, m->ffn_norm[l], c.rms_eps, M, H, m->pf_xp, m->pf_inv));      // x += o
-        RT_TRY_HIP(ctx, mm(m->wgate[l], P[1], &g));
-        RT_TRY_HIP(ctx, mm(m->wup[l], P[2], &u));
+        if (same_kind(m->wgate[l], m->wup[l])) {
+            RT_TRY_HIP(ctx, mm2(m->wgate[l], m->wup[l], P[1], P[2], &g, &u));
+        } else {
+            RT_TRY_HIP(ctx, mm(m->wgate[l], P[1], &g));
+            RT_TRY_HIP(ctx, mm(m->wup[l], P[2], &u));
+        }
         RT_TRY_HIP(ctx, rt::launch_xprep_swiglu(s, g, u, M, F, m->pf_xp, m->pf_inv));
         RT_TRY_HIP(ctx, mm(m->wdown[l], P[0], &d));
         pending = d;                             // x += d happens in the next layer's RMSNorm launch
