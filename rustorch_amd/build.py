@@ -22,7 +22,7 @@ OBJ = PKG / "build"
 LIB_SO = PKG / "librustorch_hip.so"
 LIB_A = PKG / "librustorch_hip.a"
 
-SOURCES = ["rt_api.hip", "rt_kernels.hip", "rt_attn_prefill.hip", "rt_gemv.hip", "rt_mega.hip", "rt_gemm.hip", "rt_hgemm.hip", "rt_llama.hip", "rt_synth.cpp"]
+SOURCES = ["rt_api.hip", "rt_kernels.hip", "rt_attn_prefill.hip", "rt_gemv.hip", "rt_gemv_mb.hip", "rt_mega.hip", "rt_gemm.hip", "rt_hgemm.hip", "rt_llama.hip", "rt_synth.cpp"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are kept out of the generated code on purpose.
 HIP_FLAGS = [

@@ -358,8 +358,14 @@ int rt_hip_dequant(rt_hip_ctx *ctx, const rt_hip_qweight *w, float *out_host) {
     return RT_HIP_OK;
 }
 
-// Enqueue the GEMV for one weight; x is quantized by the kernel while it is staged into LDS.
-static int enqueue_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x_dev, float *y_dev, int batch) {
+// Enqueue the GEMV for one weight; x is quantized by the kernel while it is staged into LDS.  Batches that the
+// matrix-core kernel serves go there (one pass over the weights); `work` then holds its operand buffers.
+static int enqueue_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x_dev, float *y_dev, int batch, void *work) {
+    if (work && rt::qgemv_mb_serves(w->type, w->n_rows, w->n_cols, batch)) {
+        RT_TRY_HIP(ctx, rt::launch_qgemv_mb(ctx->stream, w->type, w->dev, w->row_bytes, w->n_rows, w->n_cols, x_dev, batch, y_dev,
+                                            nullptr, work));
+        return RT_HIP_OK;
+    }
     rt::GemvArgs a;
     memset(&a, 0, sizeof a);
     a.n = 1;
@@ -384,7 +390,13 @@ int rt_hip_qgemv_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x_de
     if (rc) return rc;
     RT_REQUIRE(ctx, ((uintptr_t)x_dev & 15) == 0, RT_HIP_ERR_INVALID_ARG, "qgemv: x must be 16-byte aligned");
     Guard g(ctx);
-    return enqueue_qgemv(ctx, w, x_dev, y_dev, batch);
+    void *work = nullptr;
+    if (rt::qgemv_mb_serves(w->type, w->n_rows, w->n_cols, batch)) {
+        rc = ensure_scratch(ctx, rt::qgemv_mb_scratch_bytes(w->n_cols));
+        if (rc) return rc;
+        work = ctx->scratch;
+    }
+    return enqueue_qgemv(ctx, w, x_dev, y_dev, batch, work);
 }
 
 int rt_hip_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x, float *y, int batch) {
@@ -393,12 +405,13 @@ int rt_hip_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x, float
     if (rc) return rc;
     Guard g(ctx);
     size_t xb = align_up((size_t)batch * w->n_cols * 4, 256), yb = align_up((size_t)batch * w->n_rows * 4, 256);
-    rc = ensure_scratch(ctx, xb + yb);
+    const bool mb = rt::qgemv_mb_serves(w->type, w->n_rows, w->n_cols, batch);
+    rc = ensure_scratch(ctx, xb + yb + (mb ? rt::qgemv_mb_scratch_bytes(w->n_cols) : 0));
     if (rc) return rc;
     char *base = (char *)ctx->scratch;
     float *dx = (float *)base, *dy = (float *)(base + xb);
     RT_TRY_HIP(ctx, hipMemcpyAsync(dx, x, (size_t)batch * w->n_cols * 4, hipMemcpyHostToDevice, ctx->stream));
-    rc = enqueue_qgemv(ctx, w, dx, dy, batch);
+    rc = enqueue_qgemv(ctx, w, dx, dy, batch, mb ? base + xb + yb : nullptr);
     if (rc) return rc;
     RT_TRY_HIP(ctx, hipMemcpyAsync(y, dy, (size_t)batch * w->n_rows * 4, hipMemcpyDeviceToHost, ctx->stream));
     RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));

@@ -1,0 +1,409 @@
+// Dequant-fused GEMV for 2..8 activation rows at once on the integer matrix cores (Q4_K and Q6_K weights).
+//
+// The one-row GEMV kernel runs a batch as grid.y passes over the weights; here the weights are streamed once.
+// A wave owns 16 weight rows and a share of the super-blocks along k.  The 8 activation rows, quantized to the
+// 15 bits (per token and super-block of 256 a scale, and of every element a signed high plane q >> 7 and a low
+// plane q & 127), are the A operand of v_mfma_i32_16x16x32_i8: matrix row i = 8 * plane + token.  The raw
+// quants of 16 weight rows are the B operand (column j = weight row), so a lane's four results belong to the
+// weight row whose block header that lane itself loaded, and the block scales are applied lane-locally.
+//
+// Weights reach the lanes in two steps.  A wave loads the 16 block images of its rows with consecutive lanes on
+// consecutive dwords (a few cache lines per load instruction; lane-per-row addressing costs one line look-up per
+// lane and was measured at a third of the rate), writes them to an LDS slot of its own and reads the operand
+// layout back from there.
+//
+// Operand layout of v_mfma_i32_16x16x32_i8 (lane l, c = l / 16): A holds row l % 16, k = 8c .. 8c+7; B holds
+// column l % 16, k = 8c .. 8c+7; D holds column l % 16, rows 4c .. 4c+3.
+#include "rt_internal.h"
+#include "rt_device.h"
+
+namespace rt {
+
+namespace {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kMbThreads = 512;            // 8 waves: 8 / S groups of 16 weight rows, each group's k dealt out to S waves
+constexpr int kMbWaves = kMbThreads / 64;
+constexpr size_t kMbLdsMax = 32 * 1024;     // the x scales of a row in LDS: 32 bytes per super-block
+
+// Quantizes up to 8 activation rows into the operand form: per super-block of 256 elements and token a
+// scale s = amax / 16383 (xs[super-block][token]) and the 15-bit values q = round(x / s) as a signed high plane
+// q >> 7 and a low plane q & 127.  Per 32-element block of k, 512 bytes in the order the lanes load them:
+// [k chunk c = 0..3][matrix row i = 8 * plane + token][8 bytes], i.e. lane 16 c + i owns bytes 8 (16 c + i) .. + 7.
+// Tokens past `batch` are zero.  One wave per (super-block, token).
+__global__ __launch_bounds__(256) void xq8_prep_kernel(const float *__restrict__ X, int batch, int K, uint8_t *__restrict__ xq,
+                                                       float *__restrict__ xs) {
+    const int t = blockIdx.y, lane = threadIdx.x & 63;
+    const int sb = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (sb >= K / 256) return;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (t < batch) v = *reinterpret_cast<const float4 *>(X + (size_t)t * K + (size_t)sb * 256 + 4 * lane);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
+    const float inv = amax > 0.f ? 16383.0f / amax : 0.f;
+    const int q0 = max(-16383, min(16383, __float2int_rn(v.x * inv)));
+    const int q1 = max(-16383, min(16383, __float2int_rn(v.y * inv)));
+    const int q2 = max(-16383, min(16383, __float2int_rn(v.z * inv)));
+    const int q3 = max(-16383, min(16383, __float2int_rn(v.w * inv)));
+    const uint32_t hi = ((uint32_t)(q0 >> 7) & 0xFF) | (((uint32_t)(q1 >> 7) & 0xFF) << 8) | (((uint32_t)(q2 >> 7) & 0xFF) << 16) |
+                        (((uint32_t)(q3 >> 7) & 0xFF) << 24);
+    const uint32_t lo = (uint32_t)(q0 & 127) | ((uint32_t)(q1 & 127) << 8) | ((uint32_t)(q2 & 127) << 16) | ((uint32_t)(q3 & 127) << 24);
+    uint8_t *base = xq + (size_t)(8 * sb + (lane >> 3)) * 512 + ((lane & 7) >> 1) * 128 + t * 8 + (lane & 1) * 4;
+    *reinterpret_cast<uint32_t *>(base) = hi;
+    *reinterpret_cast<uint32_t *>(base + 64) = lo;
+    if (lane == 0) xs[sb * 8 + t] = amax / 16383.0f;
+}
+
+struct MbArgs {
+    const uint8_t *w;
+    size_t row_bytes;
+    int N, nsb;                            // rows, super-blocks of 256 along k
+    const uint8_t *xq;
+    const float *xs;                       // [nsb][8]
+    float *y;                              // [batch][N]
+    const float *res;                      // optional, added to y; may alias y
+    int batch;
+    int ksplit;                            // S: 1, 2, 4 or 8
+};
+
+__device__ __forceinline__ uint2 ld8(const uint8_t *p) {
+    uint2 v;
+    __builtin_memcpy(&v, p, 8);
+    return v;
+}
+__device__ __forceinline__ long pack8(uint32_t lo, uint32_t hi) { return (long)(((unsigned long)hi << 32) | lo); }
+__device__ __forceinline__ int mad24(int a, int b, int c) { return __mul24(a, b) + c; }
+__device__ __forceinline__ float4 ldf4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+
+// The lane's A operands of one super-block: 8 bytes of each of its 8 blocks of 32.
+struct XOps {
+    uint2 v[8];
+};
+__device__ __forceinline__ void x_load(XOps &x, const uint8_t *xq_lane, int sb) {
+#pragma unroll
+    for (int b = 0; b < 8; b++) x.v[b] = ld8(xq_lane + (size_t)(8 * sb + b) * 512);
+}
+
+// Copies n floats (a multiple of 4) into LDS with the whole workgroup.
+__device__ __forceinline__ void stage_floats(float *dst, const float *src, int n) {
+    for (int i = 4 * threadIdx.x; i < n; i += 4 * kMbThreads) *reinterpret_cast<float4 *>(dst + i) = ldf4(src + i);
+}
+
+__device__ __forceinline__ void wave_lds_fence() {     // orders one wave's own LDS writes and reads (no workgroup barrier)
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// The images of one super-block of 16 rows as a wave loads them: dword p = lane + 64 i is word p % WORDS of row
+// p / WORDS; in LDS the rows are STRIDE bytes apart (a stride that spreads the operand reads over the banks).
+template <int BLOCK, int WORDS, int LOADS, int STRIDE, bool TAIL> struct MbFmt {
+    static constexpr int kBlock = BLOCK, kWords = WORDS, kLoads = LOADS, kStride = STRIDE;
+    static constexpr bool kTail = TAIL;            // a last half word per row (BLOCK = 4 WORDS + 2)
+    static_assert(16 * WORDS == 64 * LOADS, "the dwords of 16 rows divide over 64 lanes");
+};
+using FmtQ4K = MbFmt<144, 36, 9, 152, false>;
+using FmtQ6K = MbFmt<210, 52, 13, 216, true>;
+
+template <class F> struct WImg {
+    uint32_t w[F::kLoads];
+    uint32_t tail;
+};
+template <class F> struct WOffs {
+    uint32_t g[F::kLoads], l[F::kLoads];           // byte offset from the group's first row in memory; word offset in the slot
+    uint32_t gt;
+};
+template <class F> __device__ __forceinline__ void img_offsets(WOffs<F> &o, int group, int N, size_t row_bytes) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int i = 0; i < F::kLoads; i++) {
+        const int p = lane + 64 * i, r = p / F::kWords, w = p % F::kWords;
+        const int rr = min(group * 16 + r, N - 1) - group * 16;        // rows past the end read the last row
+        o.g[i] = (uint32_t)(rr * row_bytes) + 4 * w;
+        o.l[i] = r * (F::kStride / 4) + w;
+    }
+    const int rt = min(group * 16 + (lane & 15), N - 1) - group * 16;
+    o.gt = (uint32_t)(rt * row_bytes) + 4 * F::kWords;
+}
+template <class F> __device__ __forceinline__ void img_load(WImg<F> &r, const uint8_t *blk0, const WOffs<F> &o) {
+#pragma unroll
+    for (int i = 0; i < F::kLoads; i++) __builtin_memcpy(&r.w[i], blk0 + o.g[i], 4);
+    if (F::kTail) {
+        uint16_t t;
+        __builtin_memcpy(&t, blk0 + o.gt, 2);
+        r.tail = t;
+    }
+}
+template <class F> __device__ __forceinline__ void img_store(uint32_t *slot, const WImg<F> &r, const WOffs<F> &o) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int i = 0; i < F::kLoads; i++) slot[o.l[i]] = r.w[i];
+    if (F::kTail && lane < 16) slot[lane * (F::kStride / 4) + F::kWords] = r.tail;
+}
+__device__ __forceinline__ uint2 lds8(const uint32_t *slot, int byte_off) { return *reinterpret_cast<const uint2 *>(slot + byte_off / 4); }
+
+// The wave's place: row group (16 weight rows) and k slice.
+struct MbPlace {
+    int group, ks;
+    bool live;
+};
+__device__ __forceinline__ MbPlace mb_place(const MbArgs &a) {
+    const int wv = threadIdx.x >> 6, per_wg = kMbWaves / a.ksplit;
+    MbPlace p;
+    p.group = blockIdx.x * per_wg + wv / a.ksplit;
+    p.ks = wv % a.ksplit;
+    p.live = p.group * 16 < a.N;
+    return p;
+}
+
+// Folds the two planes (lanes l and l ^ 32 hold the same weight row and tokens), then the k slices, and writes y.
+__device__ __forceinline__ void mb_finish(const MbArgs &a, float (&acc)[4], float (*part)[16][8]) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int j = lane & 15, c = lane >> 4;
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc[r] += __shfl_xor(acc[r], 32, 64);
+    if (c < 2) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) part[wv][j][4 * c + r] = acc[r];
+    }
+    __syncthreads();
+    const int per_wg = kMbWaves / a.ksplit;
+    if ((int)threadIdx.x < 128 * per_wg) {
+        const int gl = threadIdx.x >> 7, jj = (threadIdx.x >> 3) & 15, t = threadIdx.x & 7;
+        const int n = (blockIdx.x * per_wg + gl) * 16 + jj;
+        float s = 0.f;
+        for (int k = 0; k < a.ksplit; k++) s += part[gl * a.ksplit + k][jj][t];
+        if (n < a.N && t < a.batch) {
+            const size_t o = (size_t)t * a.N + n;
+            if (a.res) s += a.res[o];
+            a.y[o] = s;
+        }
+    }
+}
+
+// ---- Q4_K: 144-byte super-block = d, dmin (fp16), 12 bytes of 6-bit scales and mins, 128 bytes of nibbles;
+// unit g (64 elements) = bytes 32g..32g+31, low nibbles = sub-block 2g, high nibbles = sub-block 2g+1.
+struct Q4kRegs {
+    uint4 hdr;
+    uint2 q[4];
+};
+__device__ __forceinline__ void q4k_read(Q4kRegs &r, const uint32_t *slot, int j, int c) {
+    const int base = j * FmtQ4K::kStride;
+    const uint2 h0 = lds8(slot, base), h1 = lds8(slot, base + 8);
+    r.hdr = make_uint4(h0.x, h0.y, h1.x, h1.y);
+#pragma unroll
+    for (int g = 0; g < 4; g++) r.q[g] = lds8(slot, base + 16 + 32 * g + 8 * c);
+}
+
+__global__ __launch_bounds__(kMbThreads) void qgemv_mb_q4k_kernel(MbArgs a) {
+    RT_DYN_LDS(float4, lds4);                  // xs[nsb][8]
+    __shared__ float part[kMbWaves][16][8];
+    __shared__ uint32_t slots[kMbWaves][16 * FmtQ4K::kStride / 4];
+    float *xs = reinterpret_cast<float *>(lds4);
+    const int lane = threadIdx.x & 63;
+    const int j = lane & 15, c = lane >> 4;
+    uint32_t *slot = slots[threadIdx.x >> 6];
+    const MbPlace pl = mb_place(a);
+    const uint8_t *wrow = a.w + (size_t)pl.group * 16 * a.row_bytes;     // the group's first row (only read when live)
+    const float pf = c < 2 ? 128.f : 1.f;      // weight of the plane this lane's results belong to
+    const int tok4 = 4 * (c & 1);
+    const uint8_t *xq_lane = a.xq + 8 * lane;
+    float acc[4] = { 0.f, 0.f, 0.f, 0.f };
+    WOffs<FmtQ4K> offs;
+    img_offsets(offs, pl.group, a.N, a.row_bytes);
+    WImg<FmtQ4K> icur, inxt;
+    Q4kRegs cur;
+    XOps xc, xn;
+    int sb = pl.live ? pl.ks : a.nsb;
+    if (sb < a.nsb) {
+        img_load(icur, wrow + (size_t)sb * 144, offs);
+        x_load(xc, xq_lane, sb);
+    }
+    stage_floats(xs, a.xs, a.nsb * 8);
+    __syncthreads();
+    for (; sb < a.nsb; sb += a.ksplit) {
+        const int sbn = min(sb + a.ksplit, a.nsb - 1);
+        img_load(inxt, wrow + (size_t)sbn * 144, offs);
+        x_load(xn, xq_lane, sbn);
+        wave_lds_fence();                      // the previous super-block's operand reads come first
+        img_store(slot, icur, offs);
+        wave_lds_fence();
+        q4k_read(cur, slot, j, c);
+        // sum over the sub-blocks of scale * (x . q) in integers; sum of min * (sum of x) as a chain of matrix
+        // instructions whose weight operand is the min in every byte
+        int t0 = 0, t1 = 0, t2 = 0, t3 = 0;
+        i32x4 tm = { 0, 0, 0, 0 };
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            uint32_t scw, mw;
+            if (g < 2) {
+                scw = cur.hdr.y & 0x3f3f3f3fu;
+                mw = cur.hdr.z & 0x3f3f3f3fu;
+            } else {
+                scw = (cur.hdr.w & 0x0f0f0f0fu) | ((cur.hdr.y >> 2) & 0x30303030u);
+                mw = ((cur.hdr.w >> 4) & 0x0f0f0f0fu) | ((cur.hdr.z >> 2) & 0x30303030u);
+            }
+            scw >>= (g & 1) * 16;
+            mw >>= (g & 1) * 16;
+            const int sc0 = scw & 0xFF, sc1 = (scw >> 8) & 0xFF;
+            const uint32_t m0 = __builtin_amdgcn_perm(mw, mw, 0x00000000u), m1 = __builtin_amdgcn_perm(mw, mw, 0x01010101u);   // byte 0 / 1 in every byte
+            const long xa = pack8(xc.v[2 * g].x, xc.v[2 * g].y), xb = pack8(xc.v[2 * g + 1].x, xc.v[2 * g + 1].y);
+            const long wlo = pack8(cur.q[g].x & 0x0f0f0f0fu, cur.q[g].y & 0x0f0f0f0fu);
+            const long whi = pack8((cur.q[g].x >> 4) & 0x0f0f0f0fu, (cur.q[g].y >> 4) & 0x0f0f0f0fu);
+            const i32x4 z = { 0, 0, 0, 0 };
+            const i32x4 da = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wlo, z, 0, 0, 0);
+            const i32x4 db = __builtin_amdgcn_mfma_i32_16x16x32_i8(xb, whi, z, 0, 0, 0);
+            tm = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, pack8(m0, m0), tm, 0, 0, 0);
+            tm = __builtin_amdgcn_mfma_i32_16x16x32_i8(xb, pack8(m1, m1), tm, 0, 0, 0);
+            t0 = mad24(sc0, da[0], mad24(sc1, db[0], t0));
+            t1 = mad24(sc0, da[1], mad24(sc1, db[1], t1));
+            t2 = mad24(sc0, da[2], mad24(sc1, db[2], t2));
+            t3 = mad24(sc0, da[3], mad24(sc1, db[3], t3));
+        }
+        const float d = h2f(cur.hdr.x & 0xFFFF) * pf, dmin = h2f(cur.hdr.x >> 16) * pf;
+        const float4 sx = ldf4(xs + sb * 8 + tok4);
+        acc[0] += sx.x * (d * (float)t0 - dmin * (float)tm[0]);
+        acc[1] += sx.y * (d * (float)t1 - dmin * (float)tm[1]);
+        acc[2] += sx.z * (d * (float)t2 - dmin * (float)tm[2]);
+        acc[3] += sx.w * (d * (float)t3 - dmin * (float)tm[3]);
+        icur = inxt;
+        xc = xn;
+    }
+    mb_finish(a, acc, part);
+}
+
+// ---- Q6_K: 210-byte super-block = ql[128], qh[64], int8 scales[16], d (fp16).  Element 128h + 32r + l
+// (half h, run r, l = 0..31) = nibble (low for r < 2) of ql[64h + 32(r & 1) + l] | bits 2r..2r+1 of
+// qh[32h + l] << 4, minus 32; scale index 8h + 2r + l / 16.
+struct Q6kRegs {
+    uint2 ql[4], qh[2];                    // ql[2h + (r & 1)], qh[h]: the lane's 8 byte positions
+    uint32_t sc[4];
+    uint32_t d;
+};
+__device__ __forceinline__ void q6k_read(Q6kRegs &r, const uint32_t *slot, int j, int c) {
+    const int base = j * FmtQ6K::kStride;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r.ql[i] = lds8(slot, base + 32 * i + 8 * c);
+#pragma unroll
+    for (int h = 0; h < 2; h++) r.qh[h] = lds8(slot, base + 128 + 32 * h + 8 * c);
+    const uint2 s0 = lds8(slot, base + 192), s1 = lds8(slot, base + 200);
+    r.sc[0] = s0.x; r.sc[1] = s0.y; r.sc[2] = s1.x; r.sc[3] = s1.y;
+    r.d = slot[(base + 208) / 4] & 0xFFFF;
+}
+
+// Four 6-bit values of run r (nibbles of ql, bit pairs of qh) as signed bytes -32..31: bytes 0..63 plus 0x60 do not
+// carry into the next byte, and flipping bit 7 then takes off 0x80.
+template <int R> __device__ __forceinline__ uint32_t q6k_bytes(uint32_t ql, uint32_t qh) {
+    const uint32_t lo = (R < 2 ? ql : ql >> 4) & 0x0f0f0f0fu, hi = (qh >> (2 * R)) & 0x03030303u;
+    return (((hi << 4) | lo) + 0x60606060u) ^ 0x80808080u;
+}
+
+template <int H, int R> __device__ __forceinline__ void q6k_run(const Q6kRegs &w, const XOps &x, uint32_t keep0, int &t0, int &t1, int &t2, int &t3) {
+    const uint32_t vx = q6k_bytes<R>(w.ql[2 * H + (R & 1)].x, w.qh[H].x), vy = q6k_bytes<R>(w.ql[2 * H + (R & 1)].y, w.qh[H].y);
+    // the two 16-element runs of a 32-element block have their own scale: one matrix instruction each, with the
+    // other run's k positions (lanes c >= 2 resp. c < 2) zeroed in the weight operand
+    const long w0 = pack8(vx & keep0, vy & keep0), w1 = pack8(vx & ~keep0, vy & ~keep0);
+    const long xa = pack8(x.v[4 * H + R].x, x.v[4 * H + R].y);
+    const i32x4 z = { 0, 0, 0, 0 };
+    const i32x4 d0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, w0, z, 0, 0, 0);
+    const i32x4 d1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, w1, z, 0, 0, 0);
+    // scales 8H + 2R (first run) and 8H + 2R + 1 (second run), signed bytes
+    const uint32_t word = w.sc[2 * H + R / 2];
+    const int s0 = (int)(word << (24 - 16 * (R & 1))) >> 24, s1 = (int)(word << (16 - 16 * (R & 1))) >> 24;
+    t0 = mad24(s0, d0[0], mad24(s1, d1[0], t0));
+    t1 = mad24(s0, d0[1], mad24(s1, d1[1], t1));
+    t2 = mad24(s0, d0[2], mad24(s1, d1[2], t2));
+    t3 = mad24(s0, d0[3], mad24(s1, d1[3], t3));
+}
+
+__global__ __launch_bounds__(kMbThreads) void qgemv_mb_q6k_kernel(MbArgs a) {
+    RT_DYN_LDS(float4, lds4);                  // xs[nsb][8]
+    __shared__ float part[kMbWaves][16][8];
+    __shared__ uint32_t slots[kMbWaves][16 * FmtQ6K::kStride / 4];
+    float *xs = reinterpret_cast<float *>(lds4);
+    const int lane = threadIdx.x & 63;
+    const int j = lane & 15, c = lane >> 4;
+    uint32_t *slot = slots[threadIdx.x >> 6];
+    const MbPlace pl = mb_place(a);
+    const uint8_t *wrow = a.w + (size_t)pl.group * 16 * a.row_bytes;     // the group's first row (only read when live)
+    const float pf = c < 2 ? 128.f : 1.f;
+    const int tok4 = 4 * (c & 1);
+    const uint32_t keep0 = c < 2 ? 0xFFFFFFFFu : 0u;
+    const uint8_t *xq_lane = a.xq + 8 * lane;
+    float acc[4] = { 0.f, 0.f, 0.f, 0.f };
+    WOffs<FmtQ6K> offs;
+    img_offsets(offs, pl.group, a.N, a.row_bytes);
+    WImg<FmtQ6K> icur, inxt;
+    Q6kRegs cur;
+    XOps xc, xn;
+    int sb = pl.live ? pl.ks : a.nsb;
+    if (sb < a.nsb) {
+        img_load(icur, wrow + (size_t)sb * 210, offs);
+        x_load(xc, xq_lane, sb);
+    }
+    stage_floats(xs, a.xs, a.nsb * 8);
+    __syncthreads();
+    for (; sb < a.nsb; sb += a.ksplit) {
+        const int sbn = min(sb + a.ksplit, a.nsb - 1);
+        img_load(inxt, wrow + (size_t)sbn * 210, offs);
+        x_load(xn, xq_lane, sbn);
+        wave_lds_fence();                      // the previous super-block's operand reads come first
+        img_store(slot, icur, offs);
+        wave_lds_fence();
+        q6k_read(cur, slot, j, c);
+        int t0 = 0, t1 = 0, t2 = 0, t3 = 0;
+        q6k_run<0, 0>(cur, xc, keep0, t0, t1, t2, t3);
+        q6k_run<0, 1>(cur, xc, keep0, t0, t1, t2, t3);
+        q6k_run<0, 2>(cur, xc, keep0, t0, t1, t2, t3);
+        q6k_run<0, 3>(cur, xc, keep0, t0, t1, t2, t3);
+        q6k_run<1, 0>(cur, xc, keep0, t0, t1, t2, t3);
+        q6k_run<1, 1>(cur, xc, keep0, t0, t1, t2, t3);
+        q6k_run<1, 2>(cur, xc, keep0, t0, t1, t2, t3);
+        q6k_run<1, 3>(cur, xc, keep0, t0, t1, t2, t3);
+        const float d = h2f(cur.d) * pf;
+        const float4 sx = ldf4(xs + sb * 8 + tok4);
+        acc[0] += sx.x * d * (float)t0;
+        acc[1] += sx.y * d * (float)t1;
+        acc[2] += sx.z * d * (float)t2;
+        acc[3] += sx.w * d * (float)t3;
+        icur = inxt;
+        xc = xn;
+    }
+    mb_finish(a, acc, part);
+}
+
+}  // namespace
+
+bool qgemv_mb_serves(int type, size_t N, size_t K, int batch) {
+    if (type != RT_GGML_Q4_K && type != RT_GGML_Q6_K) return false;
+    return batch >= kGemvMbMinBatch && batch <= 8 && N >= 1 && K >= 256 && K % 256 == 0 && K / 8 <= kMbLdsMax;
+}
+
+size_t qgemv_mb_scratch_bytes(size_t K) { return 16 * K + K / 256 * 8 * 4; }
+
+hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_bytes, size_t N, size_t K, const float *x, int batch,
+                           float *y, const float *res, void *work) {
+    if (!qgemv_mb_serves(type, N, K, batch) || !w || !x || !y || !work) return hipErrorInvalidValue;
+    if (((uintptr_t)x & 15) || ((uintptr_t)work & 255) || (K * 4) % 16) return hipErrorInvalidValue;
+    if (type == RT_GGML_Q4_K && (((uintptr_t)w & 15) || row_bytes % 16)) return hipErrorInvalidValue;   // 16-byte header loads
+    if (row_bytes < K / 256 * (type == RT_GGML_Q4_K ? 144 : 210)) return hipErrorInvalidValue;
+    uint8_t *xq = static_cast<uint8_t *>(work);
+    float *xs = reinterpret_cast<float *>(xq + 16 * K);
+    dim3 pg((unsigned)((K / 256 + 3) / 4), 8);
+    xq8_prep_kernel<<<pg, 256, 0, s>>>(x, batch, (int)K, xq, xs);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    // k is dealt out to S waves per group of 16 rows: as few as still give every SIMD two waves
+    const size_t groups = (N + 15) / 16, nsb = K / 256;
+    int ksplit = 8;
+    while (ksplit > 1 && (groups * (ksplit / 2) >= 2048 || (size_t)ksplit > nsb)) ksplit /= 2;
+    MbArgs a{ static_cast<const uint8_t *>(w), row_bytes, (int)N, (int)nsb, xq, xs, y, res, batch, ksplit };
+    const size_t per_wg = kMbWaves / ksplit;
+    const unsigned grid = (unsigned)((groups + per_wg - 1) / per_wg);
+    if (type == RT_GGML_Q4_K) qgemv_mb_q4k_kernel<<<grid, kMbThreads, nsb * 32, s>>>(a);
+    else qgemv_mb_q6k_kernel<<<grid, kMbThreads, nsb * 32, s>>>(a);
+    return hipGetLastError();
+}
+
+}  // namespace rt

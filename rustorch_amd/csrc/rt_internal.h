@@ -119,6 +119,14 @@ hipError_t launch_set_state(hipStream_t s, int *state, int pos, int token, int s
 hipError_t launch_quantize_x(hipStream_t s, const float *x, uint8_t *xq, size_t K, size_t batch);
 hipError_t launch_quantize_group(hipStream_t s, const QuantGroupArgs &a);
 hipError_t launch_qgemv(hipStream_t s, GemvArgs &args, int batch);  // fills tile0 / rows_per_tile
+
+// 2..8 activation rows against Q4_K / Q6_K weights in one pass over the weights, on the integer matrix cores
+// (rt_gemv_mb.hip).  work: qgemv_mb_scratch_bytes(K) bytes, 256-byte aligned; res (optional) is added to y.
+constexpr int kGemvMbMinBatch = 2;
+bool qgemv_mb_serves(int type, size_t N, size_t K, int batch);
+size_t qgemv_mb_scratch_bytes(size_t K);
+hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_bytes, size_t N, size_t K, const float *x, int batch,
+                           float *y, const float *res, void *work);
 hipError_t launch_dequant(hipStream_t s, int type, const uint8_t *w, size_t n_rows, size_t n_cols, float *out);
 hipError_t launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *y, uint8_t *xq, size_t rows,
                           size_t n, float eps);
