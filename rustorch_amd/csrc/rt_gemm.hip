@@ -832,6 +832,12 @@ hipError_t launch_type(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_
     return launch_cfg<TYPE, kGemmWaves, 2>(s, p, w, N, K, row_bytes, Xp, inv_scale, M, Y, res, partial, reduce, w2, planes2);
 }
 
+// 3..15 rows of X against Q4_K / Q6_K: too few for the 16-row tiles of the fused contraction, enough for the integer
+// matrix-core GEMV, eight rows per launch.
+bool few_rows_on_matrix_cores(int type, size_t M, size_t N, size_t K) {
+    return M >= (size_t)kGemvMbMinBatch && M < 16 && qgemv_mb_serves(type, N, K, (int)std::min<size_t>(M, 8));
+}
+
 bool mfma_path(int type, size_t N, size_t K, size_t M) {
     return (type == RT_GGML_Q4_K || type == RT_GGML_Q6_K) && M >= 16 && K % 256 == 0 && N % 4 == 0;
 }
@@ -845,7 +851,10 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 bool qgemm_on_matrix_cores(int type, size_t M, size_t N, size_t K) { return mfma_path(type, N, K, M); }
 
 size_t qgemm_scratch_bytes(int type, size_t M, size_t N, size_t K) {
-    if (!mfma_path(type, N, K, M)) return hgemm_serves(type, M, N, K) ? hgemm_scratch_bytes(type, M, N, K) : 0;
+    if (!mfma_path(type, N, K, M)) {
+        if (hgemm_serves(type, M, N, K)) return hgemm_scratch_bytes(type, M, N, K);
+        return few_rows_on_matrix_cores(type, M, N, K) ? qgemv_mb_scratch_bytes(K) : 0;
+    }
     GemmPlan p = gemm_plan(M, N, K);
     return align256(M * K * sizeof(_Float16)) + align256(M * sizeof(float)) + (p.ksplit > 1 ? (size_t)p.ksplit * M * N * sizeof(float) : 0);
 }
@@ -935,6 +944,25 @@ hipError_t launch_qgemm(hipStream_t s, int type, const uint8_t *w, size_t N, siz
     // formats without a fused contraction: the fp16 matrix-core kernel over an fp16 copy of the weights
     if (hgemm_serves(type, M, N, K) && scratch_bytes >= hgemm_scratch_bytes(type, M, N, K))
         return launch_hgemm(s, type, w, N, K, row_bytes, X, M, Y, res, scratch, scratch_bytes);
+    if (few_rows_on_matrix_cores(type, M, N, K) && scratch_bytes >= qgemv_mb_scratch_bytes(K) && ((uintptr_t)scratch & 255) == 0) {
+        for (size_t m0 = 0; m0 < M; m0 += 8) {
+            const int b = (int)std::min<size_t>(8, M - m0);
+            const float *r = res ? res + m0 * N : nullptr;
+            hipError_t e;
+            if (b >= kGemvMbMinBatch) {
+                e = launch_qgemv_mb(s, type, w, row_bytes, N, K, X + m0 * K, b, Y + m0 * N, r, scratch);
+            } else {
+                GemvArgs a;
+                memset(&a, 0, sizeof a);
+                a.n = 1;
+                a.p[0].w = w; a.p[0].x = X + m0 * K; a.p[0].stage = kStageF32; a.p[0].y = Y + m0 * N; a.p[0].res = r;
+                a.p[0].row_bytes = row_bytes; a.p[0].type = type; a.p[0].N = (int)N; a.p[0].K = (int)K;
+                e = launch_qgemv(s, a, b);
+            }
+            if (e != hipSuccess) return e;
+        }
+        return hipSuccess;
+    }
     // Row-by-row form (few rows, in-place residual of the fused contraction): the GEMV kernel, one grid slice per row of X.
     GemvArgs a;
     memset(&a, 0, sizeof a);

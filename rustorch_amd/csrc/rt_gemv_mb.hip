@@ -2,8 +2,8 @@
 //
 // The one-row GEMV kernel runs a batch as grid.y passes over the weights; here the weights are streamed once.
 // A wave owns 16 weight rows and a share of the super-blocks along k.  The 8 activation rows, quantized to the
-// 15 bits (per token and super-block of 256 a scale, and of every element a signed high plane q >> 7 and a low
-// plane q & 127), are the A operand of v_mfma_i32_16x16x32_i8: matrix row i = 8 * plane + token.  The raw
+// 15 bits as in the one-row kernel (per token and 32 elements a scale, and of every element a signed high plane
+// q >> 7 and a low plane q & 127), are the A operand of v_mfma_i32_16x16x32_i8: matrix row i = 8 * plane + token.  The raw
 // quants of 16 weight rows are the B operand (column j = weight row), so a lane's four results belong to the
 // weight row whose block header that lane itself loaded, and the block scales are applied lane-locally.
 //
@@ -25,35 +25,26 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMbThreads = 512;            // 8 waves: 8 / S groups of 16 weight rows, each group's k dealt out to S waves
 constexpr int kMbWaves = kMbThreads / 64;
-constexpr size_t kMbLdsMax = 32 * 1024;     // the x scales of a row in LDS: 32 bytes per super-block
+constexpr size_t kMbLdsMax = 32 * 1024;     // the x scales in LDS: 8 tokens x 4 bytes per block of 32, i.e. K bytes
 
-// Quantizes up to 8 activation rows into the operand form: per super-block of 256 elements and token a
-// scale s = amax / 16383 (xs[super-block][token]) and the 15-bit values q = round(x / s) as a signed high plane
-// q >> 7 and a low plane q & 127.  Per 32-element block of k, 512 bytes in the order the lanes load them:
+// Quantizes up to 8 activation rows into the operand form, with the quantization step of the one-row kernel: per
+// token and 32-element block a scale s = amax / 16383 (xs[block][token]) and the 15-bit values q = round(x / s) as a
+// signed high plane q >> 7 and a low plane q & 127.  Per block 512 bytes in the order the lanes load them:
 // [k chunk c = 0..3][matrix row i = 8 * plane + token][8 bytes], i.e. lane 16 c + i owns bytes 8 (16 c + i) .. + 7.
-// Tokens past `batch` are zero.  One wave per (super-block, token).
+// Tokens past `batch` are zero.
 __global__ __launch_bounds__(256) void xq8_prep_kernel(const float *__restrict__ X, int batch, int K, uint8_t *__restrict__ xq,
                                                        float *__restrict__ xs) {
-    const int t = blockIdx.y, lane = threadIdx.x & 63;
-    const int sb = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (sb >= K / 256) return;
+    const int t = blockIdx.y;
+    const int i4 = blockIdx.x * 256 + threadIdx.x;         // four elements per lane, eight lanes per block
+    if (4 * i4 >= K) return;                               // K % 32 == 0: the lanes of a block leave together
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (t < batch) v = *reinterpret_cast<const float4 *>(X + (size_t)t * K + (size_t)sb * 256 + 4 * lane);
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
-    const float inv = amax > 0.f ? 16383.0f / amax : 0.f;
-    const int q0 = max(-16383, min(16383, __float2int_rn(v.x * inv)));
-    const int q1 = max(-16383, min(16383, __float2int_rn(v.y * inv)));
-    const int q2 = max(-16383, min(16383, __float2int_rn(v.z * inv)));
-    const int q3 = max(-16383, min(16383, __float2int_rn(v.w * inv)));
-    const uint32_t hi = ((uint32_t)(q0 >> 7) & 0xFF) | (((uint32_t)(q1 >> 7) & 0xFF) << 8) | (((uint32_t)(q2 >> 7) & 0xFF) << 16) |
-                        (((uint32_t)(q3 >> 7) & 0xFF) << 24);
-    const uint32_t lo = (uint32_t)(q0 & 127) | ((uint32_t)(q1 & 127) << 8) | ((uint32_t)(q2 & 127) << 16) | ((uint32_t)(q3 & 127) << 24);
-    uint8_t *base = xq + (size_t)(8 * sb + (lane >> 3)) * 512 + ((lane & 7) >> 1) * 128 + t * 8 + (lane & 1) * 4;
-    *reinterpret_cast<uint32_t *>(base) = hi;
-    *reinterpret_cast<uint32_t *>(base + 64) = lo;
-    if (lane == 0) xs[sb * 8 + t] = amax / 16383.0f;
+    if (t < batch) v = *reinterpret_cast<const float4 *>(X + (size_t)t * K + 4 * (size_t)i4);
+    const Q4Pack p = quantize4(v);
+    const int blk = i4 >> 3, l8 = i4 & 7;
+    uint8_t *base = xq + (size_t)blk * 512 + (l8 >> 1) * 128 + t * 8 + (l8 & 1) * 4;
+    *reinterpret_cast<uint32_t *>(base) = p.hi;
+    *reinterpret_cast<uint32_t *>(base + 64) = p.lo;
+    if (l8 == 0) xs[blk * 8 + t] = p.s;
 }
 
 struct MbArgs {
@@ -61,7 +52,7 @@ struct MbArgs {
     size_t row_bytes;
     int N, nsb;                            // rows, super-blocks of 256 along k
     const uint8_t *xq;
-    const float *xs;                       // [nsb][8]
+    const float *xs;                       // [K / 32][8]
     float *y;                              // [batch][N]
     const float *res;                      // optional, added to y; may alias y
     int batch;
@@ -96,50 +87,55 @@ __device__ __forceinline__ void wave_lds_fence() {     // orders one wave's own 
     __builtin_amdgcn_wave_barrier();
 }
 
-// The images of one super-block of 16 rows as a wave loads them: dword p = lane + 64 i is word p % WORDS of row
-// p / WORDS; in LDS the rows are STRIDE bytes apart (a stride that spreads the operand reads over the banks).
-template <int BLOCK, int WORDS, int LOADS, int STRIDE, bool TAIL> struct MbFmt {
-    static constexpr int kBlock = BLOCK, kWords = WORDS, kLoads = LOADS, kStride = STRIDE;
-    static constexpr bool kTail = TAIL;            // a last half word per row (BLOCK = 4 WORDS + 2)
-    static_assert(16 * WORDS == 64 * LOADS, "the dwords of 16 rows divide over 64 lanes");
+// The images of one super-block of 16 rows as a wave loads them: 16-byte piece p = lane + 64 i is piece p % PIECES of
+// row p / PIECES, and piece p of the wave's LDS slot; the last half words of 210-byte blocks follow the pieces, one
+// dword per row.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <int BLOCK, int PIECES, bool TAIL> struct MbFmt {
+    static constexpr int kBlock = BLOCK, kPieces = PIECES, kStride = 16 * PIECES;
+    static constexpr int kLoads = (16 * PIECES + 63) / 64, kLast = 16 * PIECES - 64 * (kLoads - 1);   // lanes of the last load
+    static constexpr bool kTail = TAIL;            // a last half word per row (BLOCK = 16 PIECES + 2)
+    static constexpr int kSlotWords = 64 * PIECES + (TAIL ? 16 : 0);
 };
-using FmtQ4K = MbFmt<144, 36, 9, 152, false>;
-using FmtQ6K = MbFmt<210, 52, 13, 216, true>;
+using FmtQ4K = MbFmt<144, 9, false>;
+using FmtQ6K = MbFmt<210, 13, true>;
 
 template <class F> struct WImg {
-    uint32_t w[F::kLoads];
+    u32x4 w[F::kLoads];
     uint32_t tail;
 };
 template <class F> struct WOffs {
-    uint32_t g[F::kLoads], l[F::kLoads];           // byte offset from the group's first row in memory; word offset in the slot
+    uint32_t g[F::kLoads];                         // byte offset from the group's first row in memory
     uint32_t gt;
 };
 template <class F> __device__ __forceinline__ void img_offsets(WOffs<F> &o, int group, int N, size_t row_bytes) {
     const int lane = threadIdx.x & 63;
 #pragma unroll
     for (int i = 0; i < F::kLoads; i++) {
-        const int p = lane + 64 * i, r = p / F::kWords, w = p % F::kWords;
+        const int p = min(lane + 64 * i, 16 * F::kPieces - 1), r = p / F::kPieces, w = p % F::kPieces;
         const int rr = min(group * 16 + r, N - 1) - group * 16;        // rows past the end read the last row
-        o.g[i] = (uint32_t)(rr * row_bytes) + 4 * w;
-        o.l[i] = r * (F::kStride / 4) + w;
+        o.g[i] = (uint32_t)(rr * row_bytes) + 16 * w;
     }
     const int rt = min(group * 16 + (lane & 15), N - 1) - group * 16;
-    o.gt = (uint32_t)(rt * row_bytes) + 4 * F::kWords;
+    o.gt = (uint32_t)(rt * row_bytes) + 16 * F::kPieces;
 }
 template <class F> __device__ __forceinline__ void img_load(WImg<F> &r, const uint8_t *blk0, const WOffs<F> &o) {
+    const int lane = threadIdx.x & 63;
 #pragma unroll
-    for (int i = 0; i < F::kLoads; i++) __builtin_memcpy(&r.w[i], blk0 + o.g[i], 4);
+    for (int i = 0; i < F::kLoads; i++)
+        if (i + 1 < F::kLoads || lane < F::kLast) __builtin_memcpy(&r.w[i], blk0 + o.g[i], 16);
     if (F::kTail) {
         uint16_t t;
         __builtin_memcpy(&t, blk0 + o.gt, 2);
         r.tail = t;
     }
 }
-template <class F> __device__ __forceinline__ void img_store(uint32_t *slot, const WImg<F> &r, const WOffs<F> &o) {
+template <class F> __device__ __forceinline__ void img_store(uint32_t *slot, const WImg<F> &r) {
     const int lane = threadIdx.x & 63;
 #pragma unroll
-    for (int i = 0; i < F::kLoads; i++) slot[o.l[i]] = r.w[i];
-    if (F::kTail && lane < 16) slot[lane * (F::kStride / 4) + F::kWords] = r.tail;
+    for (int i = 0; i < F::kLoads; i++)
+        if (i + 1 < F::kLoads || lane < F::kLast) *reinterpret_cast<u32x4 *>(slot + 4 * (lane + 64 * i)) = r.w[i];
+    if (F::kTail && lane < 16) slot[64 * F::kPieces + lane] = r.tail;
 }
 __device__ __forceinline__ uint2 lds8(const uint32_t *slot, int byte_off) { return *reinterpret_cast<const uint2 *>(slot + byte_off / 4); }
 
@@ -169,8 +165,8 @@ __device__ __forceinline__ void mb_finish(const MbArgs &a, float (&acc)[4], floa
     }
     __syncthreads();
     const int per_wg = kMbWaves / a.ksplit;
-    if ((int)threadIdx.x < 128 * per_wg) {
-        const int gl = threadIdx.x >> 7, jj = (threadIdx.x >> 3) & 15, t = threadIdx.x & 7;
+    for (int e = threadIdx.x; e < 128 * per_wg; e += kMbThreads) {     // 16 rows x 8 tokens per group: up to 1024 results
+        const int gl = e >> 7, jj = (e >> 3) & 15, t = e & 7;
         const int n = (blockIdx.x * per_wg + gl) * 16 + jj;
         float s = 0.f;
         for (int k = 0; k < a.ksplit; k++) s += part[gl * a.ksplit + k][jj][t];
@@ -196,10 +192,10 @@ __device__ __forceinline__ void q4k_read(Q4kRegs &r, const uint32_t *slot, int j
     for (int g = 0; g < 4; g++) r.q[g] = lds8(slot, base + 16 + 32 * g + 8 * c);
 }
 
-__global__ __launch_bounds__(kMbThreads) void qgemv_mb_q4k_kernel(MbArgs a) {
-    RT_DYN_LDS(float4, lds4);                  // xs[nsb][8]
+__global__ __launch_bounds__(kMbThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void qgemv_mb_q4k_kernel(MbArgs a) {
+    RT_DYN_LDS(float4, lds4);                  // xs[K / 32][8]
     __shared__ float part[kMbWaves][16][8];
-    __shared__ uint32_t slots[kMbWaves][16 * FmtQ4K::kStride / 4];
+    __shared__ __align__(16) uint32_t slots[kMbWaves][FmtQ4K::kSlotWords];
     float *xs = reinterpret_cast<float *>(lds4);
     const int lane = threadIdx.x & 63;
     const int j = lane & 15, c = lane >> 4;
@@ -212,28 +208,25 @@ __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q4k_kernel(MbArgs a) {
     float acc[4] = { 0.f, 0.f, 0.f, 0.f };
     WOffs<FmtQ4K> offs;
     img_offsets(offs, pl.group, a.N, a.row_bytes);
-    WImg<FmtQ4K> icur, inxt;
+    WImg<FmtQ4K> img;
     Q4kRegs cur;
     XOps xc, xn;
     int sb = pl.live ? pl.ks : a.nsb;
     if (sb < a.nsb) {
-        img_load(icur, wrow + (size_t)sb * 144, offs);
+        img_load(img, wrow + (size_t)sb * 144, offs);
         x_load(xc, xq_lane, sb);
     }
-    stage_floats(xs, a.xs, a.nsb * 8);
+    stage_floats(xs, a.xs, a.nsb * 64);
     __syncthreads();
     for (; sb < a.nsb; sb += a.ksplit) {
         const int sbn = min(sb + a.ksplit, a.nsb - 1);
-        img_load(inxt, wrow + (size_t)sbn * 144, offs);
-        x_load(xn, xq_lane, sbn);
         wave_lds_fence();                      // the previous super-block's operand reads come first
-        img_store(slot, icur, offs);
+        img_store(slot, img);
         wave_lds_fence();
+        img_load(img, wrow + (size_t)sbn * 144, offs);   // the next image into the registers just written out
+        x_load(xn, xq_lane, sbn);
         q4k_read(cur, slot, j, c);
-        // sum over the sub-blocks of scale * (x . q) in integers; sum of min * (sum of x) as a chain of matrix
-        // instructions whose weight operand is the min in every byte
-        int t0 = 0, t1 = 0, t2 = 0, t3 = 0;
-        i32x4 tm = { 0, 0, 0, 0 };
+        const float d = h2f(cur.hdr.x & 0xFFFF), dmin = h2f(cur.hdr.x >> 16);
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             uint32_t scw, mw;
@@ -246,30 +239,27 @@ __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q4k_kernel(MbArgs a) {
             }
             scw >>= (g & 1) * 16;
             mw >>= (g & 1) * 16;
-            const int sc0 = scw & 0xFF, sc1 = (scw >> 8) & 0xFF;
-            const uint32_t m0 = __builtin_amdgcn_perm(mw, mw, 0x00000000u), m1 = __builtin_amdgcn_perm(mw, mw, 0x01010101u);   // byte 0 / 1 in every byte
+            const float wa = d * (float)(scw & 0xFF), wb = d * (float)((scw >> 8) & 0xFF);
+            const float na = dmin * (float)(mw & 0xFF), nb = dmin * (float)((mw >> 8) & 0xFF);
             const long xa = pack8(xc.v[2 * g].x, xc.v[2 * g].y), xb = pack8(xc.v[2 * g + 1].x, xc.v[2 * g + 1].y);
             const long wlo = pack8(cur.q[g].x & 0x0f0f0f0fu, cur.q[g].y & 0x0f0f0f0fu);
             const long whi = pack8((cur.q[g].x >> 4) & 0x0f0f0f0fu, (cur.q[g].y >> 4) & 0x0f0f0f0fu);
+            const long ones = 0x0101010101010101L;             // x . 1 = the sum of the block's x, for the -min term
             const i32x4 z = { 0, 0, 0, 0 };
             const i32x4 da = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wlo, z, 0, 0, 0);
             const i32x4 db = __builtin_amdgcn_mfma_i32_16x16x32_i8(xb, whi, z, 0, 0, 0);
-            tm = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, pack8(m0, m0), tm, 0, 0, 0);
-            tm = __builtin_amdgcn_mfma_i32_16x16x32_i8(xb, pack8(m1, m1), tm, 0, 0, 0);
-            t0 = mad24(sc0, da[0], mad24(sc1, db[0], t0));
-            t1 = mad24(sc0, da[1], mad24(sc1, db[1], t1));
-            t2 = mad24(sc0, da[2], mad24(sc1, db[2], t2));
-            t3 = mad24(sc0, da[3], mad24(sc1, db[3], t3));
+            const i32x4 ua = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, ones, z, 0, 0, 0);
+            const i32x4 ub = __builtin_amdgcn_mfma_i32_16x16x32_i8(xb, ones, z, 0, 0, 0);
+            const float4 sa = ldf4(xs + (8 * sb + 2 * g) * 8 + tok4), sbv = ldf4(xs + (8 * sb + 2 * g + 1) * 8 + tok4);
+            acc[0] += sa.x * (wa * (float)da[0] - na * (float)ua[0]) + sbv.x * (wb * (float)db[0] - nb * (float)ub[0]);
+            acc[1] += sa.y * (wa * (float)da[1] - na * (float)ua[1]) + sbv.y * (wb * (float)db[1] - nb * (float)ub[1]);
+            acc[2] += sa.z * (wa * (float)da[2] - na * (float)ua[2]) + sbv.z * (wb * (float)db[2] - nb * (float)ub[2]);
+            acc[3] += sa.w * (wa * (float)da[3] - na * (float)ua[3]) + sbv.w * (wb * (float)db[3] - nb * (float)ub[3]);
         }
-        const float d = h2f(cur.hdr.x & 0xFFFF) * pf, dmin = h2f(cur.hdr.x >> 16) * pf;
-        const float4 sx = ldf4(xs + sb * 8 + tok4);
-        acc[0] += sx.x * (d * (float)t0 - dmin * (float)tm[0]);
-        acc[1] += sx.y * (d * (float)t1 - dmin * (float)tm[1]);
-        acc[2] += sx.z * (d * (float)t2 - dmin * (float)tm[2]);
-        acc[3] += sx.w * (d * (float)t3 - dmin * (float)tm[3]);
-        icur = inxt;
         xc = xn;
     }
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc[r] *= pf;
     mb_finish(a, acc, part);
 }
 
@@ -289,7 +279,7 @@ __device__ __forceinline__ void q6k_read(Q6kRegs &r, const uint32_t *slot, int j
     for (int h = 0; h < 2; h++) r.qh[h] = lds8(slot, base + 128 + 32 * h + 8 * c);
     const uint2 s0 = lds8(slot, base + 192), s1 = lds8(slot, base + 200);
     r.sc[0] = s0.x; r.sc[1] = s0.y; r.sc[2] = s1.x; r.sc[3] = s1.y;
-    r.d = slot[(base + 208) / 4] & 0xFFFF;
+    r.d = slot[64 * FmtQ6K::kPieces + j];
 }
 
 // Four 6-bit values of run r (nibbles of ql, bit pairs of qh) as signed bytes -32..31: bytes 0..63 plus 0x60 do not
@@ -299,7 +289,8 @@ template <int R> __device__ __forceinline__ uint32_t q6k_bytes(uint32_t ql, uint
     return (((hi << 4) | lo) + 0x60606060u) ^ 0x80808080u;
 }
 
-template <int H, int R> __device__ __forceinline__ void q6k_run(const Q6kRegs &w, const XOps &x, uint32_t keep0, int &t0, int &t1, int &t2, int &t3) {
+template <int H, int R>
+__device__ __forceinline__ void q6k_run(const Q6kRegs &w, const XOps &x, uint32_t keep0, float d, const float *xs_blk, float (&acc)[4]) {
     const uint32_t vx = q6k_bytes<R>(w.ql[2 * H + (R & 1)].x, w.qh[H].x), vy = q6k_bytes<R>(w.ql[2 * H + (R & 1)].y, w.qh[H].y);
     // the two 16-element runs of a 32-element block have their own scale: one matrix instruction each, with the
     // other run's k positions (lanes c >= 2 resp. c < 2) zeroed in the weight operand
@@ -308,19 +299,20 @@ template <int H, int R> __device__ __forceinline__ void q6k_run(const Q6kRegs &w
     const i32x4 z = { 0, 0, 0, 0 };
     const i32x4 d0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, w0, z, 0, 0, 0);
     const i32x4 d1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, w1, z, 0, 0, 0);
-    // scales 8H + 2R (first run) and 8H + 2R + 1 (second run), signed bytes
+    // scales 8H + 2R (first run) and 8H + 2R + 1 (second run), signed bytes; |s d| < 2^24
     const uint32_t word = w.sc[2 * H + R / 2];
     const int s0 = (int)(word << (24 - 16 * (R & 1))) >> 24, s1 = (int)(word << (16 - 16 * (R & 1))) >> 24;
-    t0 = mad24(s0, d0[0], mad24(s1, d1[0], t0));
-    t1 = mad24(s0, d0[1], mad24(s1, d1[1], t1));
-    t2 = mad24(s0, d0[2], mad24(s1, d1[2], t2));
-    t3 = mad24(s0, d0[3], mad24(s1, d1[3], t3));
+    const float4 sx = ldf4(xs_blk + (4 * H + R) * 8);
+    acc[0] += d * sx.x * (float)mad24(s0, d0[0], __mul24(s1, d1[0]));
+    acc[1] += d * sx.y * (float)mad24(s0, d0[1], __mul24(s1, d1[1]));
+    acc[2] += d * sx.z * (float)mad24(s0, d0[2], __mul24(s1, d1[2]));
+    acc[3] += d * sx.w * (float)mad24(s0, d0[3], __mul24(s1, d1[3]));
 }
 
 __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q6k_kernel(MbArgs a) {
-    RT_DYN_LDS(float4, lds4);                  // xs[nsb][8]
+    RT_DYN_LDS(float4, lds4);                  // xs[K / 32][8]
     __shared__ float part[kMbWaves][16][8];
-    __shared__ uint32_t slots[kMbWaves][16 * FmtQ6K::kStride / 4];
+    __shared__ __align__(16) uint32_t slots[kMbWaves][FmtQ6K::kSlotWords];
     float *xs = reinterpret_cast<float *>(lds4);
     const int lane = threadIdx.x & 63;
     const int j = lane & 15, c = lane >> 4;
@@ -334,42 +326,38 @@ __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q6k_kernel(MbArgs a) {
     float acc[4] = { 0.f, 0.f, 0.f, 0.f };
     WOffs<FmtQ6K> offs;
     img_offsets(offs, pl.group, a.N, a.row_bytes);
-    WImg<FmtQ6K> icur, inxt;
+    WImg<FmtQ6K> img;
     Q6kRegs cur;
     XOps xc, xn;
     int sb = pl.live ? pl.ks : a.nsb;
     if (sb < a.nsb) {
-        img_load(icur, wrow + (size_t)sb * 210, offs);
+        img_load(img, wrow + (size_t)sb * 210, offs);
         x_load(xc, xq_lane, sb);
     }
-    stage_floats(xs, a.xs, a.nsb * 8);
+    stage_floats(xs, a.xs, a.nsb * 64);
     __syncthreads();
     for (; sb < a.nsb; sb += a.ksplit) {
         const int sbn = min(sb + a.ksplit, a.nsb - 1);
-        img_load(inxt, wrow + (size_t)sbn * 210, offs);
-        x_load(xn, xq_lane, sbn);
         wave_lds_fence();                      // the previous super-block's operand reads come first
-        img_store(slot, icur, offs);
+        img_store(slot, img);
         wave_lds_fence();
+        img_load(img, wrow + (size_t)sbn * 210, offs);   // the next image into the registers just written out
+        x_load(xn, xq_lane, sbn);
         q6k_read(cur, slot, j, c);
-        int t0 = 0, t1 = 0, t2 = 0, t3 = 0;
-        q6k_run<0, 0>(cur, xc, keep0, t0, t1, t2, t3);
-        q6k_run<0, 1>(cur, xc, keep0, t0, t1, t2, t3);
-        q6k_run<0, 2>(cur, xc, keep0, t0, t1, t2, t3);
-        q6k_run<0, 3>(cur, xc, keep0, t0, t1, t2, t3);
-        q6k_run<1, 0>(cur, xc, keep0, t0, t1, t2, t3);
-        q6k_run<1, 1>(cur, xc, keep0, t0, t1, t2, t3);
-        q6k_run<1, 2>(cur, xc, keep0, t0, t1, t2, t3);
-        q6k_run<1, 3>(cur, xc, keep0, t0, t1, t2, t3);
-        const float d = h2f(cur.d) * pf;
-        const float4 sx = ldf4(xs + sb * 8 + tok4);
-        acc[0] += sx.x * d * (float)t0;
-        acc[1] += sx.y * d * (float)t1;
-        acc[2] += sx.z * d * (float)t2;
-        acc[3] += sx.w * d * (float)t3;
-        icur = inxt;
+        const float d = h2f(cur.d);
+        const float *xs_blk = xs + 8 * sb * 8 + tok4;
+        q6k_run<0, 0>(cur, xc, keep0, d, xs_blk, acc);
+        q6k_run<0, 1>(cur, xc, keep0, d, xs_blk, acc);
+        q6k_run<0, 2>(cur, xc, keep0, d, xs_blk, acc);
+        q6k_run<0, 3>(cur, xc, keep0, d, xs_blk, acc);
+        q6k_run<1, 0>(cur, xc, keep0, d, xs_blk, acc);
+        q6k_run<1, 1>(cur, xc, keep0, d, xs_blk, acc);
+        q6k_run<1, 2>(cur, xc, keep0, d, xs_blk, acc);
+        q6k_run<1, 3>(cur, xc, keep0, d, xs_blk, acc);
         xc = xn;
     }
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc[r] *= pf;
     mb_finish(a, acc, part);
 }
 
@@ -377,10 +365,10 @@ __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q6k_kernel(MbArgs a) {
 
 bool qgemv_mb_serves(int type, size_t N, size_t K, int batch) {
     if (type != RT_GGML_Q4_K && type != RT_GGML_Q6_K) return false;
-    return batch >= kGemvMbMinBatch && batch <= 8 && N >= 1 && K >= 256 && K % 256 == 0 && K / 8 <= kMbLdsMax;
+    return batch >= kGemvMbMinBatch && batch <= 8 && N >= 1 && K >= 256 && K % 256 == 0 && K <= kMbLdsMax;
 }
 
-size_t qgemv_mb_scratch_bytes(size_t K) { return 16 * K + K / 256 * 8 * 4; }
+size_t qgemv_mb_scratch_bytes(size_t K) { return 16 * K + K / 32 * 8 * 4; }
 
 hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_bytes, size_t N, size_t K, const float *x, int batch,
                            float *y, const float *res, void *work) {
@@ -390,7 +378,7 @@ hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_by
     if (row_bytes < K / 256 * (type == RT_GGML_Q4_K ? 144 : 210)) return hipErrorInvalidValue;
     uint8_t *xq = static_cast<uint8_t *>(work);
     float *xs = reinterpret_cast<float *>(xq + 16 * K);
-    dim3 pg((unsigned)((K / 256 + 3) / 4), 8);
+    dim3 pg((unsigned)((K / 4 + 255) / 256), 8);
     xq8_prep_kernel<<<pg, 256, 0, s>>>(x, batch, (int)K, xq, xs);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -401,8 +389,8 @@ hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_by
     MbArgs a{ static_cast<const uint8_t *>(w), row_bytes, (int)N, (int)nsb, xq, xs, y, res, batch, ksplit };
     const size_t per_wg = kMbWaves / ksplit;
     const unsigned grid = (unsigned)((groups + per_wg - 1) / per_wg);
-    if (type == RT_GGML_Q4_K) qgemv_mb_q4k_kernel<<<grid, kMbThreads, nsb * 32, s>>>(a);
-    else qgemv_mb_q6k_kernel<<<grid, kMbThreads, nsb * 32, s>>>(a);
+    if (type == RT_GGML_Q4_K) qgemv_mb_q4k_kernel<<<grid, kMbThreads, K, s>>>(a);
+    else qgemv_mb_q6k_kernel<<<grid, kMbThreads, K, s>>>(a);
     return hipGetLastError();
 }
 

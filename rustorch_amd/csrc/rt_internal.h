@@ -122,7 +122,7 @@ hipError_t launch_qgemv(hipStream_t s, GemvArgs &args, int batch);  // fills til
 
 // 2..8 activation rows against Q4_K / Q6_K weights in one pass over the weights, on the integer matrix cores
 // (rt_gemv_mb.hip).  work: qgemv_mb_scratch_bytes(K) bytes, 256-byte aligned; res (optional) is added to y.
-constexpr int kGemvMbMinBatch = 2;
+constexpr int kGemvMbMinBatch = 3;       // two rows are faster as two passes of the one-row kernel
 bool qgemv_mb_serves(int type, size_t N, size_t K, int batch);
 size_t qgemv_mb_scratch_bytes(size_t K);
 hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_bytes, size_t N, size_t K, const float *x, int batch,

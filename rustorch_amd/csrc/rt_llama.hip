@@ -189,6 +189,7 @@ bool gemv_type_ok(int t) {
 }
 
 constexpr size_t kPrefillChunk = 512;     // tokens per pass of the batched prefill
+constexpr int kPrefillMinRows = 3;        // fewer tokens go through the decode step; 3..15 run the contractions eight rows at a time
 
 // The batched prefill serves every block format: Q4_K / Q6_K matrices go to the matrix cores, the others run the GEMV
 // kernel with one grid slice per token (weights found in L2 / Infinity Cache after the first).
@@ -646,18 +647,18 @@ int rt_hip_llama_prefill(rt_hip_ctx *ctx, rt_hip_llama *m, const int *tokens, in
     int rc = check_complete(ctx, m);
     if (rc) return rc;
     Guard g(ctx);
-    if (n_tok >= 16 && prefill_batchable(m)) {
+    if (n_tok >= kPrefillMinRows && prefill_batchable(m)) {
         // dense-contraction path, kPrefillChunk tokens per pass; the logits of the last token come from the head GEMV
         rc = ensure_prefill_buffers(ctx, m, std::min((size_t)n_tok, kPrefillChunk));
         if (rc) return rc;
         for (size_t t0 = 0; t0 < (size_t)n_tok; t0 += kPrefillChunk) {
             const size_t M = std::min(kPrefillChunk, (size_t)n_tok - t0);
             RT_TRY_HIP(ctx, hipMemcpyAsync(m->pf_tok, tokens + t0, M * sizeof(int), hipMemcpyHostToDevice, ctx->stream));
-            if (M >= 16) {
+            if (M >= (size_t)kPrefillMinRows) {
                 rc = prefill_chainable(m, M) ? enqueue_prefill_chain(ctx, m, M, pos0 + (int)t0) : enqueue_prefill_batch(ctx, m, M, pos0 + (int)t0);
                 if (rc) return rc;
             } else {
-                // a short tail goes token by token (the row form of the contraction starts at 16 rows)
+                // a tail of one or two tokens goes token by token
                 for (size_t i = 0; i < M; i++) {
                     RT_TRY_HIP(ctx, rt::launch_set_state(ctx->stream, m->state, pos0 + (int)(t0 + i), tokens[t0 + i], 0));
                     rc = enqueue_step(ctx, m, false);

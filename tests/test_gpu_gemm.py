@@ -88,6 +88,24 @@ def test_other_formats_and_small_m_use_the_row_form(ex, orc):
             assert (np.abs(ex.qgemm(w, X) - y64) / (wn[None, :] * xn)).max() <= HELD * np.sqrt(4096 / cols)
 
 
+@pytest.mark.parametrize("t", [12, 14])
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (100, 11008)])
+def test_three_to_fifteen_rows_go_eight_at_a_time(ex, orc, t, rows, cols):
+    """Fewer rows of X than the fused contraction's tiles take: the integer matrix-core GEMV, eight rows per launch, the
+    remainder of one or two rows as passes of the one-row kernel (M = 9, 10)."""
+    from rustorch_amd import synth
+    print("gemm few rows", t, rows, cols, flush=True)
+    raw = synth.blocks(t, 35, t, rows, cols)
+    w = ex.upload_qweight(t, rows, cols, raw)
+    for M in (3, 8, 9, 10, 11, 15):
+        X = synth.normal(35, M, M * cols).reshape(M, cols)
+        y64, wn = orc.qgemv_f64(t, raw, rows, cols, X)
+        xn = np.linalg.norm(X.astype(np.float64), axis=1)[:, None]
+        worst = (np.abs(ex.qgemm(w, X) - y64) / (wn[None, :] * xn)).max()
+        print("  M=%d: %.3e" % (M, worst), flush=True)
+        assert worst <= 2e-5
+
+
 @pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 10, 11, 13, 1, 0])
 def test_formats_without_a_fused_contraction(ex, orc, t):
     """From 32 rows of X on these formats go through the fp16 matrix-core kernel (F16 weights as they are, the others

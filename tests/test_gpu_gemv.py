@@ -93,7 +93,7 @@ def test_gemv_edge_inputs(ex, orc, t):
 
 
 @pytest.mark.parametrize("t", [12, 14])
-@pytest.mark.parametrize("rows,cols", [(37, 256), (16, 768), (1, 4096), (4099, 2048), (300, 11008)])
+@pytest.mark.parametrize("rows,cols", [(37, 256), (256, 256), (16, 768), (1, 4096), (4099, 2048), (300, 11008), (40000, 512), (48, 28672)])
 def test_batches_of_two_to_eight_on_the_matrix_cores(ex, orc, t, rows, cols):
     """Every batch size the one-pass kernel takes, with row counts that do not fill its groups of 16 and k slices that
     leave some of a workgroup's waves without work; rows past the batch must not be written."""
