@@ -152,12 +152,13 @@ SHAPES = {"7b": dict(NL=NL, H=H, NH=NH, NKV=NH, F=F, V=V), "70b": dict(NL=80, H=
 
 
 def bench_batch8(ex, reps=100):
-    """Config C3 at M = 8: the three layer shapes with eight activation rows per launch (the batch-1 kernel run per row as
-    grid slices; the weights of rows 2..8 come from L2 / Infinity Cache).  Weight GB/s counts the weights once."""
+    """Config C3 at M = 8: the layer shapes and the output head with eight activation rows per call.  From three rows on
+    Q4_K / Q6_K weights take the integer matrix-core GEMV (one pass over the weights, preceded by a small launch that
+    quantizes the rows); the time is the call's, both launches.  Weight GB/s counts the weights once."""
     from rustorch_amd import synth, GGMLType
     out = []
     for name, t, rows, cols in (("q4k_4096x4096", GGMLType.Q4_K, 4096, 4096), ("q4k_11008x4096", GGMLType.Q4_K, 11008, 4096),
-                                ("q6k_4096x11008", GGMLType.Q6_K, 4096, 11008)):
+                                ("q6k_4096x11008", GGMLType.Q6_K, 4096, 11008), ("q6k_32000x4096", GGMLType.Q6_K, 32000, 4096)):
         ws = [ex.upload_qweight(t, rows, cols, synth.blocks(t, SEED, 9000 + i, rows, cols)) for i in range(8)]
         x = ex.to_device(synth.normal(SEED, 9100, 8 * cols))
         y = ex.buffer(4 * 8 * rows)
@@ -272,6 +273,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--prefill-only", action="store_true", help="run only the prefill contraction shapes (for kernel traces)")
+    ap.add_argument("--batch8-only", action="store_true", help="run only the eight-row GEMV shapes (for kernel traces)")
     ap.add_argument("--decode-prompt", type=int, default=128)
     ap.add_argument("--decode-gen", type=int, default=128)
     ap.add_argument("--decode-shape", choices=sorted(SHAPES), default="7b", help="model shape of the decode measurement (the benchmark's is 7b)")
@@ -300,6 +302,10 @@ def main():
 
     if args.prefill_only:
         print(json.dumps({"prefill": bench_prefill(ex)}), flush=True)
+        ex.close()
+        return
+    if args.batch8_only:
+        print(json.dumps({"batch8": bench_batch8(ex)}), flush=True)
         ex.close()
         return
 

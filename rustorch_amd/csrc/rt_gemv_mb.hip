@@ -25,15 +25,15 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMbThreads = 512;            // 8 waves: 8 / S groups of 16 weight rows, each group's k dealt out to S waves
 constexpr int kMbWaves = kMbThreads / 64;
-constexpr size_t kMbLdsMax = 32 * 1024;     // the x scales in LDS: 8 tokens x 4 bytes per block of 32, i.e. K bytes
+constexpr size_t kMbLdsMax = 32 * 1024;     // the x scales (Q4_K: and block sums) in LDS: 8 tokens x 4 bytes per block of 32, i.e. K bytes each
 
 // Quantizes up to 8 activation rows into the operand form, with the quantization step of the one-row kernel: per
 // token and 32-element block a scale s = amax / 16383 (xs[block][token]) and the 15-bit values q = round(x / s) as a
 // signed high plane q >> 7 and a low plane q & 127.  Per block 512 bytes in the order the lanes load them:
 // [k chunk c = 0..3][matrix row i = 8 * plane + token][8 bytes], i.e. lane 16 c + i owns bytes 8 (16 c + i) .. + 7.
-// Tokens past `batch` are zero.
+// xb[block][token] = s * (sum of the block's q), the x side of the -min term of Q4_K.  Tokens past `batch` are zero.
 __global__ __launch_bounds__(256) void xq8_prep_kernel(const float *__restrict__ X, int batch, int K, uint8_t *__restrict__ xq,
-                                                       float *__restrict__ xs) {
+                                                       float *__restrict__ xs, float *__restrict__ xb) {
     const int t = blockIdx.y;
     const int i4 = blockIdx.x * 256 + threadIdx.x;         // four elements per lane, eight lanes per block
     if (4 * i4 >= K) return;                               // K % 32 == 0: the lanes of a block leave together
@@ -44,7 +44,10 @@ __global__ __launch_bounds__(256) void xq8_prep_kernel(const float *__restrict__
     uint8_t *base = xq + (size_t)blk * 512 + (l8 >> 1) * 128 + t * 8 + (l8 & 1) * 4;
     *reinterpret_cast<uint32_t *>(base) = p.hi;
     *reinterpret_cast<uint32_t *>(base + 64) = p.lo;
-    if (l8 == 0) xs[blk * 8 + t] = p.s;
+    if (l8 == 0) {
+        xs[blk * 8 + t] = p.s;
+        xb[blk * 8 + t] = p.s * (float)p.sum32;
+    }
 }
 
 struct MbArgs {
@@ -52,7 +55,7 @@ struct MbArgs {
     size_t row_bytes;
     int N, nsb;                            // rows, super-blocks of 256 along k
     const uint8_t *xq;
-    const float *xs;                       // [K / 32][8]
+    const float *xs, *xb;                  // [K / 32][8] each
     float *y;                              // [batch][N]
     const float *res;                      // optional, added to y; may alias y
     int batch;
@@ -193,16 +196,17 @@ __device__ __forceinline__ void q4k_read(Q4kRegs &r, const uint32_t *slot, int j
 }
 
 __global__ __launch_bounds__(kMbThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void qgemv_mb_q4k_kernel(MbArgs a) {
-    RT_DYN_LDS(float4, lds4);                  // xs[K / 32][8]
+    RT_DYN_LDS(float4, lds4);                  // xs[K / 32][8], xb[K / 32][8]
     __shared__ float part[kMbWaves][16][8];
     __shared__ __align__(16) uint32_t slots[kMbWaves][FmtQ4K::kSlotWords];
-    float *xs = reinterpret_cast<float *>(lds4);
+    float *xs = reinterpret_cast<float *>(lds4), *xb = xs + a.nsb * 64;
     const int lane = threadIdx.x & 63;
     const int j = lane & 15, c = lane >> 4;
     uint32_t *slot = slots[threadIdx.x >> 6];
     const MbPlace pl = mb_place(a);
     const uint8_t *wrow = a.w + (size_t)pl.group * 16 * a.row_bytes;     // the group's first row (only read when live)
     const float pf = c < 2 ? 128.f : 1.f;      // weight of the plane this lane's results belong to
+    const float mf = c < 2 ? 1.f : 0.f;        // the -min term is counted once, with the high plane
     const int tok4 = 4 * (c & 1);
     const uint8_t *xq_lane = a.xq + 8 * lane;
     float acc[4] = { 0.f, 0.f, 0.f, 0.f };
@@ -217,6 +221,7 @@ __global__ __launch_bounds__(kMbThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         x_load(xc, xq_lane, sb);
     }
     stage_floats(xs, a.xs, a.nsb * 64);
+    stage_floats(xb, a.xb, a.nsb * 64);
     __syncthreads();
     for (; sb < a.nsb; sb += a.ksplit) {
         const int sbn = min(sb + a.ksplit, a.nsb - 1);
@@ -239,27 +244,23 @@ __global__ __launch_bounds__(kMbThreads) __attribute__((amdgpu_waves_per_eu(4, 4
             }
             scw >>= (g & 1) * 16;
             mw >>= (g & 1) * 16;
-            const float wa = d * (float)(scw & 0xFF), wb = d * (float)((scw >> 8) & 0xFF);
-            const float na = dmin * (float)(mw & 0xFF), nb = dmin * (float)((mw >> 8) & 0xFF);
-            const long xa = pack8(xc.v[2 * g].x, xc.v[2 * g].y), xb = pack8(xc.v[2 * g + 1].x, xc.v[2 * g + 1].y);
+            const float wa = d * (float)(scw & 0xFF) * pf, wb = d * (float)((scw >> 8) & 0xFF) * pf;
+            const float na = dmin * (float)(mw & 0xFF) * mf, nb = dmin * (float)((mw >> 8) & 0xFF) * mf;
+            const long xa = pack8(xc.v[2 * g].x, xc.v[2 * g].y), xbv = pack8(xc.v[2 * g + 1].x, xc.v[2 * g + 1].y);
             const long wlo = pack8(cur.q[g].x & 0x0f0f0f0fu, cur.q[g].y & 0x0f0f0f0fu);
             const long whi = pack8((cur.q[g].x >> 4) & 0x0f0f0f0fu, (cur.q[g].y >> 4) & 0x0f0f0f0fu);
-            const long ones = 0x0101010101010101L;             // x . 1 = the sum of the block's x, for the -min term
             const i32x4 z = { 0, 0, 0, 0 };
             const i32x4 da = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wlo, z, 0, 0, 0);
-            const i32x4 db = __builtin_amdgcn_mfma_i32_16x16x32_i8(xb, whi, z, 0, 0, 0);
-            const i32x4 ua = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, ones, z, 0, 0, 0);
-            const i32x4 ub = __builtin_amdgcn_mfma_i32_16x16x32_i8(xb, ones, z, 0, 0, 0);
-            const float4 sa = ldf4(xs + (8 * sb + 2 * g) * 8 + tok4), sbv = ldf4(xs + (8 * sb + 2 * g + 1) * 8 + tok4);
-            acc[0] += sa.x * (wa * (float)da[0] - na * (float)ua[0]) + sbv.x * (wb * (float)db[0] - nb * (float)ub[0]);
-            acc[1] += sa.y * (wa * (float)da[1] - na * (float)ua[1]) + sbv.y * (wb * (float)db[1] - nb * (float)ub[1]);
-            acc[2] += sa.z * (wa * (float)da[2] - na * (float)ua[2]) + sbv.z * (wb * (float)db[2] - nb * (float)ub[2]);
-            acc[3] += sa.w * (wa * (float)da[3] - na * (float)ua[3]) + sbv.w * (wb * (float)db[3] - nb * (float)ub[3]);
+            const i32x4 db = __builtin_amdgcn_mfma_i32_16x16x32_i8(xbv, whi, z, 0, 0, 0);
+            const int ba = (8 * sb + 2 * g) * 8 + tok4;
+            const float4 sa = ldf4(xs + ba), sbv = ldf4(xs + ba + 8), ma = ldf4(xb + ba), mb = ldf4(xb + ba + 8);
+            acc[0] += (wa * sa.x) * (float)da[0] + (wb * sbv.x) * (float)db[0] - (na * ma.x + nb * mb.x);
+            acc[1] += (wa * sa.y) * (float)da[1] + (wb * sbv.y) * (float)db[1] - (na * ma.y + nb * mb.y);
+            acc[2] += (wa * sa.z) * (float)da[2] + (wb * sbv.z) * (float)db[2] - (na * ma.z + nb * mb.z);
+            acc[3] += (wa * sa.w) * (float)da[3] + (wb * sbv.w) * (float)db[3] - (na * ma.w + nb * mb.w);
         }
         xc = xn;
     }
-#pragma unroll
-    for (int r = 0; r < 4; r++) acc[r] *= pf;
     mb_finish(a, acc, part);
 }
 
@@ -365,10 +366,10 @@ __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q6k_kernel(MbArgs a) {
 
 bool qgemv_mb_serves(int type, size_t N, size_t K, int batch) {
     if (type != RT_GGML_Q4_K && type != RT_GGML_Q6_K) return false;
-    return batch >= kGemvMbMinBatch && batch <= 8 && N >= 1 && K >= 256 && K % 256 == 0 && K <= kMbLdsMax;
+    return batch >= kGemvMbMinBatch && batch <= 8 && N >= 1 && K >= 256 && K % 256 == 0 && (type == RT_GGML_Q4_K ? 2 : 1) * K <= kMbLdsMax;
 }
 
-size_t qgemv_mb_scratch_bytes(size_t K) { return 16 * K + K / 32 * 8 * 4; }
+size_t qgemv_mb_scratch_bytes(size_t K) { return 16 * K + 2 * (K / 32 * 8 * 4); }
 
 hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_bytes, size_t N, size_t K, const float *x, int batch,
                            float *y, const float *res, void *work) {
@@ -379,17 +380,29 @@ hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_by
     uint8_t *xq = static_cast<uint8_t *>(work);
     float *xs = reinterpret_cast<float *>(xq + 16 * K);
     dim3 pg((unsigned)((K / 4 + 255) / 256), 8);
-    xq8_prep_kernel<<<pg, 256, 0, s>>>(x, batch, (int)K, xq, xs);
+    float *xb = xs + K / 4;
+    xq8_prep_kernel<<<pg, 256, 0, s>>>(x, batch, (int)K, xq, xs, xb);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    // k is dealt out to S waves per group of 16 rows: as few as still give every SIMD two waves
+    // k is dealt out to S waves per group of 16 rows.  Among the S that give every SIMD two waves, the one whose
+    // workgroups divide most evenly over the 256 CUs (344 workgroups would leave a third of the CUs with twice the work
+    // of the others); the smaller S on a tie.  Short of 2048 waves: the largest S the row allows.
     const size_t groups = (N + 15) / 16, nsb = K / 256;
-    int ksplit = 8;
-    while (ksplit > 1 && (groups * (ksplit / 2) >= 2048 || (size_t)ksplit > nsb)) ksplit /= 2;
-    MbArgs a{ static_cast<const uint8_t *>(w), row_bytes, (int)N, (int)nsb, xq, xs, y, res, batch, ksplit };
+    int ksplit = 0;
+    double best = 0;
+    for (int sp = 1; sp <= kMbWaves; sp *= 2) {
+        if ((size_t)sp > nsb || groups * sp < 2048) continue;
+        const double wgs = (double)((groups * sp + kMbWaves - 1) / kMbWaves), uneven = (double)(((size_t)wgs + 255) / 256) * 256.0 / wgs;
+        if (!ksplit || uneven < best - 1e-9) { ksplit = sp; best = uneven; }
+    }
+    if (!ksplit) {
+        ksplit = kMbWaves;
+        while ((size_t)ksplit > nsb) ksplit /= 2;
+    }
+    MbArgs a{ static_cast<const uint8_t *>(w), row_bytes, (int)N, (int)nsb, xq, xs, xb, y, res, batch, ksplit };
     const size_t per_wg = kMbWaves / ksplit;
     const unsigned grid = (unsigned)((groups + per_wg - 1) / per_wg);
-    if (type == RT_GGML_Q4_K) qgemv_mb_q4k_kernel<<<grid, kMbThreads, K, s>>>(a);
+    if (type == RT_GGML_Q4_K) qgemv_mb_q4k_kernel<<<grid, kMbThreads, 2 * K, s>>>(a);
     else qgemv_mb_q6k_kernel<<<grid, kMbThreads, K, s>>>(a);
     return hipGetLastError();
 }
