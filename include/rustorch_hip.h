@@ -143,7 +143,9 @@ RT_HIP_API int rt_hip_qweight_free(rt_hip_ctx *ctx, rt_hip_qweight *w);
  * (example-cli/src/model/formats/tensor_loader.rs:41-67,125-141) with real block decode; bit-exact. */
 RT_HIP_API int rt_hip_dequant(rt_hip_ctx *ctx, const rt_hip_qweight *w, float *out_host);
 RT_HIP_API int rt_hip_dequant_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, float *out_dev);
-/* y[batch, n_rows] = x[batch, n_cols] . dequant(W)^T, batch 1..8 (decode): Linear::forward without bias. */
+/* y[batch, n_rows] = x[batch, n_cols] . dequant(W)^T, batch 1..8 (decode): Linear::forward without bias.
+ * Q4_K / Q6_K weights with batch >= 3 are read once for the whole batch (integer matrix-core kernel, rows quantized by a
+ * small launch ahead of it); other formats and batch 2 run the one-row kernel per row. */
 RT_HIP_API int rt_hip_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x, float *y, int batch);
 RT_HIP_API int rt_hip_qgemv_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x_dev, float *y_dev,
                                 int batch);
