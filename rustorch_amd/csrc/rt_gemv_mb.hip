@@ -76,8 +76,9 @@ struct XOps {
     uint2 v[8];
 };
 __device__ __forceinline__ void x_load(XOps &x, const uint8_t *xq_lane, int sb) {
+    const uint8_t *p = xq_lane + (size_t)sb * 4096;        // one address, eight constant offsets
 #pragma unroll
-    for (int b = 0; b < 8; b++) x.v[b] = ld8(xq_lane + (size_t)(8 * sb + b) * 512);
+    for (int b = 0; b < 8; b++) x.v[b] = ld8(p + 512 * b);
 }
 
 // Copies n floats (a multiple of 4) into LDS with the whole workgroup.
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(kMbThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     stage_floats(xb, a.xb, a.nsb * 64);
     __syncthreads();
     for (; sb < a.nsb; sb += a.ksplit) {
-        const int sbn = min(sb + a.ksplit, a.nsb - 1);
+        const int sbn = min(sb + a.ksplit, a.nsb - 1);     // past the end a super-block is requested again: no branch around the loads
         wave_lds_fence();                      // the previous super-block's operand reads come first
         img_store(slot, img);
         wave_lds_fence();
@@ -291,23 +292,25 @@ template <int R> __device__ __forceinline__ uint32_t q6k_bytes(uint32_t ql, uint
 }
 
 template <int H, int R>
-__device__ __forceinline__ void q6k_run(const Q6kRegs &w, const XOps &x, uint32_t keep0, float d, const float *xs_blk, float (&acc)[4]) {
+__device__ __forceinline__ void q6k_run(const Q6kRegs &w, const XOps &x, uint32_t keep0, const float *xs_blk, float (&acc)[4]) {
     const uint32_t vx = q6k_bytes<R>(w.ql[2 * H + (R & 1)].x, w.qh[H].x), vy = q6k_bytes<R>(w.ql[2 * H + (R & 1)].y, w.qh[H].y);
-    // the two 16-element runs of a 32-element block have their own scale: one matrix instruction each, with the
-    // other run's k positions (lanes c >= 2 resp. c < 2) zeroed in the weight operand
-    const long w0 = pack8(vx & keep0, vy & keep0), w1 = pack8(vx & ~keep0, vy & ~keep0);
+    // The two 16-element runs of a 32-element block have their own scale.  One matrix instruction over the whole block
+    // (S0 + S1) and one with the second run's k positions (lanes c >= 2) zeroed in the weight operand (S0):
+    // s0 S0 + s1 S1 = (s0 - s1) S0 + s1 (S0 + S1).
+    const long wall = pack8(vx, vy), w0 = pack8(vx & keep0, vy & keep0);
     const long xa = pack8(x.v[4 * H + R].x, x.v[4 * H + R].y);
     const i32x4 z = { 0, 0, 0, 0 };
+    const i32x4 dall = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wall, z, 0, 0, 0);
     const i32x4 d0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, w0, z, 0, 0, 0);
-    const i32x4 d1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, w1, z, 0, 0, 0);
     // scales 8H + 2R (first run) and 8H + 2R + 1 (second run), signed bytes; |s d| < 2^24
     const uint32_t word = w.sc[2 * H + R / 2];
     const int s0 = (int)(word << (24 - 16 * (R & 1))) >> 24, s1 = (int)(word << (16 - 16 * (R & 1))) >> 24;
+    const int sd = s0 - s1;
     const float4 sx = ldf4(xs_blk + (4 * H + R) * 8);
-    acc[0] += d * sx.x * (float)mad24(s0, d0[0], __mul24(s1, d1[0]));
-    acc[1] += d * sx.y * (float)mad24(s0, d0[1], __mul24(s1, d1[1]));
-    acc[2] += d * sx.z * (float)mad24(s0, d0[2], __mul24(s1, d1[2]));
-    acc[3] += d * sx.w * (float)mad24(s0, d0[3], __mul24(s1, d1[3]));
+    acc[0] += sx.x * (float)mad24(sd, d0[0], __mul24(s1, dall[0]));
+    acc[1] += sx.y * (float)mad24(sd, d0[1], __mul24(s1, dall[1]));
+    acc[2] += sx.z * (float)mad24(sd, d0[2], __mul24(s1, dall[2]));
+    acc[3] += sx.w * (float)mad24(sd, d0[3], __mul24(s1, dall[3]));
 }
 
 __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q6k_kernel(MbArgs a) {
@@ -338,23 +341,26 @@ __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q6k_kernel(MbArgs a) {
     stage_floats(xs, a.xs, a.nsb * 64);
     __syncthreads();
     for (; sb < a.nsb; sb += a.ksplit) {
-        const int sbn = min(sb + a.ksplit, a.nsb - 1);
+        const int sbn = min(sb + a.ksplit, a.nsb - 1);     // past the end a super-block is requested again: no branch around the loads
         wave_lds_fence();                      // the previous super-block's operand reads come first
         img_store(slot, img);
         wave_lds_fence();
         img_load(img, wrow + (size_t)sbn * 210, offs);   // the next image into the registers just written out
         x_load(xn, xq_lane, sbn);
         q6k_read(cur, slot, j, c);
-        const float d = h2f(cur.d);
         const float *xs_blk = xs + 8 * sb * 8 + tok4;
-        q6k_run<0, 0>(cur, xc, keep0, d, xs_blk, acc);
-        q6k_run<0, 1>(cur, xc, keep0, d, xs_blk, acc);
-        q6k_run<0, 2>(cur, xc, keep0, d, xs_blk, acc);
-        q6k_run<0, 3>(cur, xc, keep0, d, xs_blk, acc);
-        q6k_run<1, 0>(cur, xc, keep0, d, xs_blk, acc);
-        q6k_run<1, 1>(cur, xc, keep0, d, xs_blk, acc);
-        q6k_run<1, 2>(cur, xc, keep0, d, xs_blk, acc);
-        q6k_run<1, 3>(cur, xc, keep0, d, xs_blk, acc);
+        float part_sb[4] = { 0.f, 0.f, 0.f, 0.f };           // the super-block's sum before its scale d
+        q6k_run<0, 0>(cur, xc, keep0, xs_blk, part_sb);
+        q6k_run<0, 1>(cur, xc, keep0, xs_blk, part_sb);
+        q6k_run<0, 2>(cur, xc, keep0, xs_blk, part_sb);
+        q6k_run<0, 3>(cur, xc, keep0, xs_blk, part_sb);
+        q6k_run<1, 0>(cur, xc, keep0, xs_blk, part_sb);
+        q6k_run<1, 1>(cur, xc, keep0, xs_blk, part_sb);
+        q6k_run<1, 2>(cur, xc, keep0, xs_blk, part_sb);
+        q6k_run<1, 3>(cur, xc, keep0, xs_blk, part_sb);
+        const float d = h2f(cur.d);
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] += d * part_sb[r];
         xc = xn;
     }
 #pragma unroll
