@@ -183,6 +183,44 @@ def bench_batch8(ex, reps=100):
     return out
 
 
+def bench_layer_batch8(ex, n_layers=4, reps=100):
+    """Config C3 at M = 8 as one step: the seven projections of a Llama-7B layer with eight activation rows each, issued the
+    way a layer would (q, k, v against the same rows; o; gate, up against the same rows; down), rotating through n_layers
+    sets of weights (520 MB, beyond the 256 MB Infinity Cache).  Weight GB/s counts the weights once."""
+    from rustorch_amd import synth
+    specs = synth.layer_tensor_specs(H, F)
+    wbytes, _ = layer_bytes_algorithmic(specs)
+    layers = [[ex.upload_qweight(t, r, c, synth.blocks(t, SEED, synth.layer_tid(l, slot), r, c)) for slot, t, r, c in specs]
+              for l in range(n_layers)]
+    xh = ex.to_device(synth.normal(SEED, 9200, 8 * H))
+    xf = ex.to_device(synth.normal(SEED, 9201, 8 * F))
+    ys = [ex.buffer(4 * 8 * r) for _, _, r, _ in specs]
+
+    def layer(ws):
+        ex.qgemv_shared_x_dev(ws[0:3], xh, ys[0:3], 8)
+        ex.qgemv_dev(ws[3], xh, ys[3], 8)
+        ex.qgemv_shared_x_dev(ws[4:6], xh, ys[4:6], 8)
+        ex.qgemv_dev(ws[6], xf, ys[6], 8)
+
+    for i in range(8):
+        layer(layers[i % n_layers])
+    ex.synchronize()
+    e0, e1 = ex.event(), ex.event()
+    e0.record()
+    for i in range(reps):
+        layer(layers[i % n_layers])
+    e1.record()
+    ex.synchronize()
+    ms = e0.elapsed_ms(e1) / reps
+    for ws in layers:
+        for w in ws:
+            w.free()
+    for b in [xh, xf] + ys:
+        b.free()
+    return {"us_layer_batch8": round(ms * 1e3, 2), "weight_gbps": round(wbytes / ms / 1e6, 1), "rows_per_s": round(8 / (ms * 1e-3)),
+            "launches_per_layer": 9}
+
+
 def bench_decode(ex, n_prompt, n_gen, shape="7b"):
     from rustorch_amd import llama, synth
     sh = SHAPES[shape]
@@ -305,7 +343,7 @@ def main():
         ex.close()
         return
     if args.batch8_only:
-        print(json.dumps({"batch8": bench_batch8(ex)}), flush=True)
+        print(json.dumps({"batch8": bench_batch8(ex), "layer_batch8": bench_layer_batch8(ex)}), flush=True)
         ex.close()
         return
 
@@ -331,6 +369,7 @@ def main():
     if not args.no_prefill:
         out["prefill"] = bench_prefill(ex)
         out["batch8"] = bench_batch8(ex)
+        out["layer_batch8"] = bench_layer_batch8(ex)
     if not args.no_decode:
         out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen, args.decode_shape)
     ex.close()

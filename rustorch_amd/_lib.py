@@ -57,6 +57,7 @@ SIGNATURES = {
     "rt_hip_qgemv": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]),
     "rt_hip_qgemv_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]),
     "rt_hip_qgemv_grouped_dev": (C.c_int, [C.c_void_p, C.c_int, c_void_pp, c_void_pp, c_void_pp]),
+    "rt_hip_qgemv_shared_x_dev": (C.c_int, [C.c_void_p, C.c_int, c_void_pp, C.c_void_p, c_void_pp, C.c_int]),
     "rt_hip_xq_bytes": (C.c_size_t, [C.c_size_t]),
     "rt_hip_quantize_act_dev": (C.c_int, [C.c_void_p, C.c_int, c_void_pp, C.POINTER(C.c_size_t), c_void_pp]),
     "rt_hip_qgemv_xq_grouped_dev": (C.c_int, [C.c_void_p, C.c_int, c_void_pp, c_void_pp, c_void_pp]),

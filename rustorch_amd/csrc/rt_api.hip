@@ -418,6 +418,47 @@ int rt_hip_qgemv(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *x, float
     return RT_HIP_OK;
 }
 
+int rt_hip_qgemv_shared_x_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const *ws, const float *x_dev, float *const *ys_dev, int batch) {
+    if (!ctx || !ws || !x_dev || !ys_dev) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_qgemv_shared_x_dev: NULL argument");
+    RT_REQUIRE(ctx, n >= 1 && n <= 8, RT_HIP_ERR_INVALID_ARG, "shared-x GEMV takes 1..8 weights, got %d", n);
+    RT_REQUIRE(ctx, ((uintptr_t)x_dev & 15) == 0, RT_HIP_ERR_INVALID_ARG, "shared-x GEMV: x must be 16-byte aligned");
+    bool any_mb = false;
+    for (int i = 0; i < n; i++) {
+        if (!ws[i] || !ys_dev[i]) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "shared-x GEMV: weight or output %d is NULL", i);
+        int rc = qgemv_check(ctx, ws[i], batch);
+        if (rc) return rc;
+        RT_REQUIRE(ctx, ws[i]->n_cols == ws[0]->n_cols, RT_HIP_ERR_SHAPE, "shared-x GEMV: weight %d has %zu columns, weight 0 has %zu", i,
+                   ws[i]->n_cols, ws[0]->n_cols);
+        any_mb = any_mb || rt::qgemv_mb_serves(ws[i]->type, ws[i]->n_rows, ws[i]->n_cols, batch);
+    }
+    Guard g(ctx);
+    const size_t K = ws[0]->n_cols;
+    if (any_mb) {
+        // the rows are quantized once; the matrices of each format go out together, up to four per launch
+        int rc = ensure_scratch(ctx, rt::qgemv_mb_scratch_bytes(K));
+        if (rc) return rc;
+        RT_TRY_HIP(ctx, rt::launch_qgemv_mb_prep(ctx->stream, x_dev, batch, K, ctx->scratch));
+        for (int type : { (int)RT_GGML_Q4_K, (int)RT_GGML_Q6_K }) {
+            rt::MbProb probs[4];
+            int m = 0;
+            for (int i = 0; i <= n; i++) {
+                const bool take = i < n && ws[i]->type == type && rt::qgemv_mb_serves(type, ws[i]->n_rows, K, batch);
+                if (take) probs[m++] = rt::MbProb{ ws[i]->dev, ws[i]->row_bytes, ws[i]->n_rows, ys_dev[i], nullptr };
+                if (m == 4 || (i == n && m > 0)) {
+                    RT_TRY_HIP(ctx, rt::launch_qgemv_mb_group(ctx->stream, type, probs, m, K, batch, ctx->scratch));
+                    m = 0;
+                }
+            }
+        }
+    }
+    for (int i = 0; i < n; i++)
+        if (!rt::qgemv_mb_serves(ws[i]->type, ws[i]->n_rows, K, batch)) {
+            int rc = enqueue_qgemv(ctx, ws[i], x_dev, ys_dev[i], batch, nullptr);
+            if (rc) return rc;
+        }
+    return RT_HIP_OK;
+}
+
 int rt_hip_qgemv_grouped_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const *ws, const float *const *xs_dev,
                              float *const *ys_dev) {
     if (!ctx || !ws || !xs_dev || !ys_dev) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_qgemv_grouped_dev: NULL argument");

@@ -17,6 +17,8 @@
 #include "rt_internal.h"
 #include "rt_device.h"
 
+#include <cstring>
+
 namespace rt {
 
 namespace {
@@ -50,14 +52,23 @@ __global__ __launch_bounds__(256) void xq8_prep_kernel(const float *__restrict__
     }
 }
 
-struct MbArgs {
+constexpr int kMbMaxProbs = 4;             // weight matrices of one format that meet the same prepared rows in one launch
+
+struct MbProbDev {
     const uint8_t *w;
     size_t row_bytes;
-    int N, nsb;                            // rows, super-blocks of 256 along k
-    const uint8_t *xq;
-    const float *xs, *xb;                  // [K / 32][8] each
     float *y;                              // [batch][N]
     const float *res;                      // optional, added to y; may alias y
+    int N;                                 // rows
+    int wg0;                               // first workgroup of the problem
+};
+
+struct MbArgs {
+    MbProbDev p[kMbMaxProbs];
+    int n;
+    int nsb;                               // super-blocks of 256 along k
+    const uint8_t *xq;
+    const float *xs, *xb;                  // [K / 32][8] each
     int batch;
     int ksplit;                            // S: 1, 2, 4 or 8
 };
@@ -143,22 +154,29 @@ template <class F> __device__ __forceinline__ void img_store(uint32_t *slot, con
 }
 __device__ __forceinline__ uint2 lds8(const uint32_t *slot, int byte_off) { return *reinterpret_cast<const uint2 *>(slot + byte_off / 4); }
 
-// The wave's place: row group (16 weight rows) and k slice.
+// The wave's place: problem, row group (16 weight rows) of it and k slice.
 struct MbPlace {
+    int prob, wg;                          // problem, workgroup within it
     int group, ks;
     bool live;
 };
 __device__ __forceinline__ MbPlace mb_place(const MbArgs &a) {
     const int wv = threadIdx.x >> 6, per_wg = kMbWaves / a.ksplit;
     MbPlace p;
-    p.group = blockIdx.x * per_wg + wv / a.ksplit;
+    p.prob = 0;
+#pragma unroll
+    for (int i = 1; i < kMbMaxProbs; i++)
+        if (i < a.n && (int)blockIdx.x >= a.p[i].wg0) p.prob = i;
+    p.wg = blockIdx.x - a.p[p.prob].wg0;
+    p.group = p.wg * per_wg + wv / a.ksplit;
     p.ks = wv % a.ksplit;
-    p.live = p.group * 16 < a.N;
+    p.live = p.group * 16 < a.p[p.prob].N;
     return p;
 }
 
 // Folds the two planes (lanes l and l ^ 32 hold the same weight row and tokens), then the k slices, and writes y.
-__device__ __forceinline__ void mb_finish(const MbArgs &a, float (&acc)[4], float (*part)[16][8]) {
+__device__ __forceinline__ void mb_finish(const MbArgs &a, const MbPlace &pl, float (&acc)[4], float (*part)[16][8]) {
+    const MbProbDev &P = a.p[pl.prob];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int j = lane & 15, c = lane >> 4;
 #pragma unroll
@@ -171,13 +189,13 @@ __device__ __forceinline__ void mb_finish(const MbArgs &a, float (&acc)[4], floa
     const int per_wg = kMbWaves / a.ksplit;
     for (int e = threadIdx.x; e < 128 * per_wg; e += kMbThreads) {     // 16 rows x 8 tokens per group: up to 1024 results
         const int gl = e >> 7, jj = (e >> 3) & 15, t = e & 7;
-        const int n = (blockIdx.x * per_wg + gl) * 16 + jj;
+        const int n = (pl.wg * per_wg + gl) * 16 + jj;
         float s = 0.f;
         for (int k = 0; k < a.ksplit; k++) s += part[gl * a.ksplit + k][jj][t];
-        if (n < a.N && t < a.batch) {
-            const size_t o = (size_t)t * a.N + n;
-            if (a.res) s += a.res[o];
-            a.y[o] = s;
+        if (n < P.N && t < a.batch) {
+            const size_t o = (size_t)t * P.N + n;
+            if (P.res) s += P.res[o];
+            P.y[o] = s;
         }
     }
 }
@@ -205,14 +223,15 @@ __global__ __launch_bounds__(kMbThreads) __attribute__((amdgpu_waves_per_eu(4, 4
     const int j = lane & 15, c = lane >> 4;
     uint32_t *slot = slots[threadIdx.x >> 6];
     const MbPlace pl = mb_place(a);
-    const uint8_t *wrow = a.w + (size_t)pl.group * 16 * a.row_bytes;     // the group's first row (only read when live)
+    const MbProbDev &P = a.p[pl.prob];
+    const uint8_t *wrow = P.w + (size_t)pl.group * 16 * P.row_bytes;     // the group's first row (only read when live)
     const float pf = c < 2 ? 128.f : 1.f;      // weight of the plane this lane's results belong to
     const float mf = c < 2 ? 1.f : 0.f;        // the -min term is counted once, with the high plane
     const int tok4 = 4 * (c & 1);
     const uint8_t *xq_lane = a.xq + 8 * lane;
     float acc[4] = { 0.f, 0.f, 0.f, 0.f };
     WOffs<FmtQ4K> offs;
-    img_offsets(offs, pl.group, a.N, a.row_bytes);
+    img_offsets(offs, pl.group, P.N, P.row_bytes);
     WImg<FmtQ4K> img;
     Q4kRegs cur;
     XOps xc, xn;
@@ -262,7 +281,7 @@ __global__ __launch_bounds__(kMbThreads) __attribute__((amdgpu_waves_per_eu(4, 4
         }
         xc = xn;
     }
-    mb_finish(a, acc, part);
+    mb_finish(a, pl, acc, part);
 }
 
 // ---- Q6_K: 210-byte super-block = ql[128], qh[64], int8 scales[16], d (fp16).  Element 128h + 32r + l
@@ -322,14 +341,15 @@ __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q6k_kernel(MbArgs a) {
     const int j = lane & 15, c = lane >> 4;
     uint32_t *slot = slots[threadIdx.x >> 6];
     const MbPlace pl = mb_place(a);
-    const uint8_t *wrow = a.w + (size_t)pl.group * 16 * a.row_bytes;     // the group's first row (only read when live)
+    const MbProbDev &P = a.p[pl.prob];
+    const uint8_t *wrow = P.w + (size_t)pl.group * 16 * P.row_bytes;     // the group's first row (only read when live)
     const float pf = c < 2 ? 128.f : 1.f;
     const int tok4 = 4 * (c & 1);
     const uint32_t keep0 = c < 2 ? 0xFFFFFFFFu : 0u;
     const uint8_t *xq_lane = a.xq + 8 * lane;
     float acc[4] = { 0.f, 0.f, 0.f, 0.f };
     WOffs<FmtQ6K> offs;
-    img_offsets(offs, pl.group, a.N, a.row_bytes);
+    img_offsets(offs, pl.group, P.N, P.row_bytes);
     WImg<FmtQ6K> img;
     Q6kRegs cur;
     XOps xc, xn;
@@ -365,35 +385,44 @@ __global__ __launch_bounds__(kMbThreads) void qgemv_mb_q6k_kernel(MbArgs a) {
     }
 #pragma unroll
     for (int r = 0; r < 4; r++) acc[r] *= pf;
-    mb_finish(a, acc, part);
+    mb_finish(a, pl, acc, part);
 }
 
 }  // namespace
 
 bool qgemv_mb_serves(int type, size_t N, size_t K, int batch) {
     if (type != RT_GGML_Q4_K && type != RT_GGML_Q6_K) return false;
-    return batch >= kGemvMbMinBatch && batch <= 8 && N >= 1 && K >= 256 && K % 256 == 0 && (type == RT_GGML_Q4_K ? 2 : 1) * K <= kMbLdsMax;
+    return batch >= kGemvMbMinBatch && batch <= 8 && N >= 1 && N < ((size_t)1 << 31) && K >= 256 && K % 256 == 0 &&
+           (type == RT_GGML_Q4_K ? 2 : 1) * K <= kMbLdsMax;
 }
 
 size_t qgemv_mb_scratch_bytes(size_t K) { return 16 * K + 2 * (K / 32 * 8 * 4); }
 
-hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_bytes, size_t N, size_t K, const float *x, int batch,
-                           float *y, const float *res, void *work) {
-    if (!qgemv_mb_serves(type, N, K, batch) || !w || !x || !y || !work) return hipErrorInvalidValue;
-    if (((uintptr_t)x & 15) || ((uintptr_t)work & 255) || (K * 4) % 16) return hipErrorInvalidValue;
-    if (type == RT_GGML_Q4_K && (((uintptr_t)w & 15) || row_bytes % 16)) return hipErrorInvalidValue;   // 16-byte header loads
-    if (row_bytes < K / 256 * (type == RT_GGML_Q4_K ? 144 : 210)) return hipErrorInvalidValue;
+hipError_t launch_qgemv_mb_prep(hipStream_t s, const float *x, int batch, size_t K, void *work) {
+    if (!x || !work || batch < 1 || batch > 8 || K < 256 || K % 256 != 0) return hipErrorInvalidValue;
+    if (((uintptr_t)x & 15) || ((uintptr_t)work & 255)) return hipErrorInvalidValue;
     uint8_t *xq = static_cast<uint8_t *>(work);
     float *xs = reinterpret_cast<float *>(xq + 16 * K);
-    dim3 pg((unsigned)((K / 4 + 255) / 256), 8);
     float *xb = xs + K / 4;
+    dim3 pg((unsigned)((K / 4 + 255) / 256), 8);
     xq8_prep_kernel<<<pg, 256, 0, s>>>(x, batch, (int)K, xq, xs, xb);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    return hipGetLastError();
+}
+
+hipError_t launch_qgemv_mb_group(hipStream_t s, int type, const MbProb *probs, int n, size_t K, int batch, const void *work) {
+    if (!probs || n < 1 || n > kMbMaxProbs || !work || ((uintptr_t)work & 255)) return hipErrorInvalidValue;
+    const size_t block = type == RT_GGML_Q4_K ? 144 : 210, nsb = K / 256;
+    size_t groups = 0;
+    for (int i = 0; i < n; i++) {
+        const MbProb &q = probs[i];
+        if (!qgemv_mb_serves(type, q.N, K, batch) || !q.w || !q.y) return hipErrorInvalidValue;
+        if (type == RT_GGML_Q4_K && (((uintptr_t)q.w & 15) || q.row_bytes % 16)) return hipErrorInvalidValue;   // 16-byte pieces of 16-byte aligned blocks
+        if (q.row_bytes < nsb * block || q.row_bytes * 16 >= ((size_t)1 << 32)) return hipErrorInvalidValue;    // 32-bit offsets within a group of rows
+        groups += (q.N + 15) / 16;
+    }
     // k is dealt out to S waves per group of 16 rows.  Among the S that give every SIMD two waves, the one whose
     // workgroups divide most evenly over the 256 CUs (344 workgroups would leave a third of the CUs with twice the work
     // of the others); the smaller S on a tie.  Short of 2048 waves: the largest S the row allows.
-    const size_t groups = (N + 15) / 16, nsb = K / 256;
     int ksplit = 0;
     double best = 0;
     for (int sp = 1; sp <= kMbWaves; sp *= 2) {
@@ -405,12 +434,31 @@ hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_by
         ksplit = kMbWaves;
         while ((size_t)ksplit > nsb) ksplit /= 2;
     }
-    MbArgs a{ static_cast<const uint8_t *>(w), row_bytes, (int)N, (int)nsb, xq, xs, xb, y, res, batch, ksplit };
     const size_t per_wg = kMbWaves / ksplit;
-    const unsigned grid = (unsigned)((groups + per_wg - 1) / per_wg);
-    if (type == RT_GGML_Q4_K) qgemv_mb_q4k_kernel<<<grid, kMbThreads, 2 * K, s>>>(a);
+    MbArgs a;
+    memset(&a, 0, sizeof a);
+    const uint8_t *xq = static_cast<const uint8_t *>(work);
+    a.n = n; a.nsb = (int)nsb; a.xq = xq; a.xs = reinterpret_cast<const float *>(xq + 16 * K); a.xb = a.xs + K / 4;
+    a.batch = batch; a.ksplit = ksplit;
+    size_t wgs = 0;
+    for (int i = 0; i < n; i++) {
+        a.p[i] = MbProbDev{ static_cast<const uint8_t *>(probs[i].w), probs[i].row_bytes, probs[i].y, probs[i].res, (int)probs[i].N, (int)wgs };
+        wgs += ((probs[i].N + 15) / 16 + per_wg - 1) / per_wg;
+    }
+    if (wgs >= ((size_t)1 << 31)) return hipErrorInvalidValue;
+    const unsigned grid = (unsigned)wgs;
+    if (type == RT_GGML_Q4_K) qgemv_mb_q4k_kernel<<<grid, kMbThreads, 2 * K, s>>>(a);     // x scales and block sums
     else qgemv_mb_q6k_kernel<<<grid, kMbThreads, K, s>>>(a);
     return hipGetLastError();
+}
+
+hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_bytes, size_t N, size_t K, const float *x, int batch,
+                           float *y, const float *res, void *work) {
+    if (!qgemv_mb_serves(type, N, K, batch)) return hipErrorInvalidValue;
+    hipError_t e = launch_qgemv_mb_prep(s, x, batch, K, work);
+    if (e != hipSuccess) return e;
+    const MbProb p{ w, row_bytes, N, y, res };
+    return launch_qgemv_mb_group(s, type, &p, 1, K, batch, work);
 }
 
 }  // namespace rt

@@ -127,6 +127,15 @@ bool qgemv_mb_serves(int type, size_t N, size_t K, int batch);
 size_t qgemv_mb_scratch_bytes(size_t K);
 hipError_t launch_qgemv_mb(hipStream_t s, int type, const void *w, size_t row_bytes, size_t N, size_t K, const float *x, int batch,
                            float *y, const float *res, void *work);
+// The two halves of it: quantize the rows into `work` once, then up to 4 matrices of one format against them per launch.
+struct MbProb {
+    const void *w;
+    size_t row_bytes, N;
+    float *y;                  // [batch][N]
+    const float *res;          // optional, added to y; may alias y
+};
+hipError_t launch_qgemv_mb_prep(hipStream_t s, const float *x, int batch, size_t K, void *work);
+hipError_t launch_qgemv_mb_group(hipStream_t s, int type, const MbProb *probs, int n, size_t K, int batch, const void *work);
 hipError_t launch_dequant(hipStream_t s, int type, const uint8_t *w, size_t n_rows, size_t n_cols, float *out);
 hipError_t launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *y, uint8_t *xq, size_t rows,
                           size_t n, float eps);

@@ -253,6 +253,15 @@ class HipKernelExecutor:
         wa = arr(*[w.handle for w in ws]); xa = arr(*[x.ptr for x in xs]); ya = arr(*[y.ptr for y in ys])
         _lib.check(self.lib.rt_hip_qgemv_grouped_dev(self.ctx, n, wa, xa, ya), self.ctx)
 
+    def qgemv_shared_x_dev(self, ws: Sequence[QWeight], x: DeviceBuffer, ys: Sequence[DeviceBuffer], batch: int) -> None:
+        """Several weights against one activation batch (q / k / v, gate / up): ys[i] = x[batch, n_cols] . dequant(ws[i])^T."""
+        n = len(ws)
+        if n != len(ys):
+            raise InvalidParameters("shared-x GEMV: %d weights, %d outputs" % (n, len(ys)))
+        arr = C.c_void_p * n
+        wa = arr(*[w.handle for w in ws]); ya = arr(*[y.ptr for y in ys])
+        _lib.check(self.lib.rt_hip_qgemv_shared_x_dev(self.ctx, n, wa, x.ptr, ya, batch), self.ctx)
+
     def xq_bytes(self, n_cols: int) -> int:
         return int(self.lib.rt_hip_xq_bytes(n_cols))
 

@@ -138,6 +138,33 @@ def test_grouped_launch_equals_single_launches(ex, orc):
         assert np.array_equal(y.download(np.float32), wv)
 
 
+@pytest.mark.parametrize("batch", [1, 2, 5, 8])
+def test_several_weights_against_one_batch(ex, orc, batch):
+    """q / k / v of an attention block and gate / up of a feed-forward block meet the same rows: one quantizing launch,
+    the Q4_K matrices in one launch and the Q6_K ones in another; a format the matrix-core kernel does not take (Q8_0) and
+    batches below three run per weight."""
+    from rustorch_amd import synth, ShapeMismatch
+    cols = 2048
+    specs = [(12, 1024), (12, 1024), (14, 512), (12, 37), (8, 256), (12, 2048), (14, 96)]
+    print("gemv shared x", specs, "batch", batch, flush=True)
+    x = synth.normal(98, 1, 8 * cols).reshape(8, cols)[:batch]
+    dx = ex.to_device(x)
+    ws, ys, raws = [], [], []
+    for i, (t, r) in enumerate(specs):
+        raw = synth.blocks(t, 98, 10 + i, r, cols)
+        raws.append(raw); ws.append(ex.upload_qweight(t, r, cols, raw)); ys.append(ex.buffer(8 * r * 4))
+    ex.qgemv_shared_x_dev(ws, dx, ys, batch)
+    for (t, r), raw, w, y in zip(specs, raws, ws, ys):
+        y64, wn = orc.qgemv_f64(t, raw, r, cols, x)
+        got = y.download(np.float32, batch * r).reshape(batch, r)
+        check(got, y64, wn, x, "type %d rows %d batch %d" % (t, r, batch))
+        single = np.atleast_2d(ex.qgemv(w, x))
+        assert np.all(np.abs(got - single) <= 2 * TIGHT * wn[None, :] * np.linalg.norm(x.astype(np.float64), axis=1)[:, None])
+    other = ex.upload_qweight(12, 64, 1024, synth.blocks(12, 98, 30, 64, 1024))
+    with pytest.raises(ShapeMismatch):
+        ex.qgemv_shared_x_dev([ws[0], other], dx, ys[:2], batch)          # another number of columns
+
+
 def test_device_pointer_form_and_errors(ex, orc):
     from rustorch_amd import synth, InvalidParameters, ShapeMismatch
     raw = synth.blocks(12, 3, 3, 64, 512)
