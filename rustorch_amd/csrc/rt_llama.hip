@@ -243,6 +243,34 @@ struct PrefillGemm {
         if (mc) prepared = X;
         return RT_HIP_OK;
     }
+    // n matrices against the same rows of X (q, k, v; gate, up).  3..15 rows of Q4_K / Q6_K: the rows are quantized once
+    // per eight and the matrices of one format share a launch; otherwise one contraction per matrix.
+    int shared(rt_hip_llama::T *const *ts, float *const *Ys, int n, const float *X, size_t M) {
+        const size_t K = ts[0]->n_cols;
+        bool ok = n <= 4 && M >= (size_t)rt::kGemvMbMinBatch && M < 16 && (M <= 8 || M - 8 >= (size_t)rt::kGemvMbMinBatch) &&
+                  ctx->scratch_bytes >= rt::qgemv_mb_scratch_bytes(K);
+        for (int i = 0; i < n && ok; i++)
+            ok = ts[i]->n_cols == K && rt::qgemv_mb_serves(ts[i]->type, ts[i]->n_rows, K, (int)std::min<size_t>(M, 8));
+        if (!ok) {
+            for (int i = 0; i < n; i++) {
+                int rc = (*this)(*ts[i], X, M, Ys[i], nullptr);
+                if (rc) return rc;
+            }
+            return RT_HIP_OK;
+        }
+        for (size_t m0 = 0; m0 < M; m0 += 8) {
+            const int b = (int)std::min<size_t>(8, M - m0);
+            RT_TRY_HIP(ctx, rt::launch_qgemv_mb_prep(ctx->stream, X + m0 * K, b, K, ctx->scratch));
+            for (int type : { (int)RT_GGML_Q4_K, (int)RT_GGML_Q6_K }) {
+                rt::MbProb probs[4];
+                int k = 0;
+                for (int i = 0; i < n; i++)
+                    if (ts[i]->type == type) probs[k++] = rt::MbProb{ ts[i]->dev, ts[i]->row_bytes, ts[i]->n_rows, Ys[i] + m0 * ts[i]->n_rows, nullptr };
+                if (k) RT_TRY_HIP(ctx, rt::launch_qgemv_mb_group(ctx->stream, type, probs, k, K, b, ctx->scratch));
+            }
+        }
+        return RT_HIP_OK;
+    }
 };
 
 // Every matrix of every layer goes to the matrix cores at this M, and the rows fit the fused pre-pass kernels.
@@ -340,17 +368,18 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
         uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->attn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
         gemm.prepared = nullptr;          // pf_n has new contents
-        if ((rc = gemm(m->wq[l], m->pf_n, M, m->pf_q, nullptr))) return rc;
-        if ((rc = gemm(m->wk[l], m->pf_n, M, m->pf_k, nullptr))) return rc;
-        if ((rc = gemm(m->wv[l], m->pf_n, M, m->pf_v, nullptr))) return rc;
+        rt_hip_llama::T *qkv[3] = { &m->wq[l], &m->wk[l], &m->wv[l] };
+        float *qkv_y[3] = { m->pf_q, m->pf_k, m->pf_v };
+        if ((rc = gemm.shared(qkv, qkv_y, 3, m->pf_n, M))) return rc;
         RT_TRY_HIP(ctx, rt::launch_rope_kv_batch(s, m->pf_q, m->pf_k, m->pf_v, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
         RT_TRY_HIP(ctx, rt::launch_attn_causal(s, m->pf_q, kc, vc, pos0, M, c.n_heads, m->n_kv, m->head_dim, m->pf_a));
         if ((rc = gemm(m->wo[l], m->pf_a, M, x2, x))) return rc;
         std::swap(x, x2);
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->ffn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
         gemm.prepared = nullptr;
-        if ((rc = gemm(m->wgate[l], m->pf_n, M, m->pf_g, nullptr))) return rc;
-        if ((rc = gemm(m->wup[l], m->pf_n, M, m->pf_u, nullptr))) return rc;
+        rt_hip_llama::T *gu[2] = { &m->wgate[l], &m->wup[l] };
+        float *gu_y[2] = { m->pf_g, m->pf_u };
+        if ((rc = gemm.shared(gu, gu_y, 2, m->pf_n, M))) return rc;
         RT_TRY_HIP(ctx, rt::launch_swiglu(s, m->pf_g, m->pf_u, m->pf_g, nullptr, M * F));
         gemm.prepared = nullptr;          // pf_g is rewritten in place
         if ((rc = gemm(m->wdown[l], m->pf_g, M, x2, x))) return rc;
