@@ -1,14 +1,15 @@
-// Dequant-fused GEMV for 2..8 activation rows at once on the integer matrix cores (Q4_K and Q6_K weights).
+// Dequant-fused GEMV for up to 8 activation rows at once on the integer matrix cores (Q4_K and Q6_K weights; the callers
+// send batches of 3 and more here).
 //
 // The one-row GEMV kernel runs a batch as grid.y passes over the weights; here the weights are streamed once.
 // A wave owns 16 weight rows and a share of the super-blocks along k.  The 8 activation rows, quantized to the
 // 15 bits as in the one-row kernel (per token and 32 elements a scale, and of every element a signed high plane
 // q >> 7 and a low plane q & 127), are the A operand of v_mfma_i32_16x16x32_i8: matrix row i = 8 * plane + token.  The raw
 // quants of 16 weight rows are the B operand (column j = weight row), so a lane's four results belong to the
-// weight row whose block header that lane itself loaded, and the block scales are applied lane-locally.
+// weight row whose block header that lane itself holds, and the block scales are applied lane-locally.
 //
 // Weights reach the lanes in two steps.  A wave loads the 16 block images of its rows with consecutive lanes on
-// consecutive dwords (a few cache lines per load instruction; lane-per-row addressing costs one line look-up per
+// consecutive 16-byte pieces (a few cache lines per load instruction; lane-per-row addressing costs one line look-up per
 // lane and was measured at a third of the rate), writes them to an LDS slot of its own and reads the operand
 // layout back from there.
 //
