@@ -49,6 +49,13 @@ def test_refused_arguments_leave_a_message_and_a_working_context(ex, orc):
         ex.upload_qweight(15, 8, 256, np.zeros(8 * 292, np.uint8))                       # Q8_K: no kernel
     with pytest.raises(ShapeMismatch):
         ex.attn_decode(np.zeros(2 * 96, np.float32), np.zeros((4, 192), np.uint16), np.zeros((4, 192), np.uint16), 4, 2, 96)   # head_dim 96
+    dx, dy = ex.to_device(np.zeros(8 * 256, np.float32)), ex.buffer(8 * 8 * 4)
+    with pytest.raises(InvalidParameters):
+        ex.qgemv_shared_x_dev([w] * 9, dx, [dy] * 9, 8)                                  # more than eight weights
+    with pytest.raises(InvalidParameters):
+        ex.qgemv_shared_x_dev([w], dx, [dy], 9)                                          # batch beyond eight
+    with pytest.raises(InvalidParameters):
+        ex.qgemv_shared_x_dev([w, w], dx, [dy], 8)                                       # one output for two weights
     still_works(ex, orc)
     y = ex.qgemv(w, np.ones(256, np.float32))
     assert np.isfinite(y).all()
