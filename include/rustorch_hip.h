@@ -152,8 +152,8 @@ RT_HIP_API int rt_hip_qgemv_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const 
 /* n weight matrices with the same n_cols against ONE activation batch x_dev[batch][n_cols] (the q / k / v projections of
  * an attention block, gate / up of a feed-forward block: example-cli/src/model/architectures/gpt.rs:192-215 calls
  * Linear::forward on the same input for each): ys_dev[i] is [batch][n_rows_i].  For Q4_K / Q6_K weights and batch >= 3 the
- * rows are quantized once and up to four matrices of one format share a launch; everything else runs as rt_hip_qgemv_dev
- * per weight.  n in 1..8. */
+ * rows are quantized once and up to four matrices of one format share a launch; the other weights (another format, fewer
+ * rows) are the problems of one launch of the one-row kernel.  n in 1..8. */
 RT_HIP_API int rt_hip_qgemv_shared_x_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const *ws, const float *x_dev,
                                          float *const *ys_dev, int batch);
 /* n independent GEMVs (batch 1 each) in one launch: ws[i], xs_dev[i] (n_cols_i floats), ys_dev[i] (n_rows_i floats). */

@@ -451,11 +451,17 @@ int rt_hip_qgemv_shared_x_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *cons
             }
         }
     }
-    for (int i = 0; i < n; i++)
-        if (!rt::qgemv_mb_serves(ws[i]->type, ws[i]->n_rows, K, batch)) {
-            int rc = enqueue_qgemv(ctx, ws[i], x_dev, ys_dev[i], batch, nullptr);
-            if (rc) return rc;
-        }
+    // the others (another format, fewer than three rows): problems of one launch of the one-row kernel, a grid slice per row
+    rt::GemvArgs a;
+    memset(&a, 0, sizeof a);
+    for (int i = 0; i < n; i++) {
+        const rt_hip_qweight *w = ws[i];
+        if (rt::qgemv_mb_serves(w->type, w->n_rows, K, batch)) continue;
+        rt::GemvProb &p = a.p[a.n++];
+        p.w = w->dev; p.x = x_dev; p.stage = rt::kStageF32; p.y = ys_dev[i]; p.row_bytes = w->row_bytes;
+        p.type = w->type; p.N = (int)w->n_rows; p.K = (int)w->n_cols;
+    }
+    if (a.n > 0) RT_TRY_HIP(ctx, rt::launch_qgemv(ctx->stream, a, batch));
     return RT_HIP_OK;
 }
 
