@@ -22,13 +22,13 @@ OBJ = PKG / "build"
 LIB_SO = PKG / "librustorch_hip.so"
 LIB_A = PKG / "librustorch_hip.a"
 
-SOURCES = ["rt_api.hip", "rt_kernels.hip", "rt_attn_prefill.hip", "rt_gemv.hip", "rt_gemv_mb.hip", "rt_mega.hip", "rt_gemm.hip", "rt_hgemm.hip", "rt_llama.hip", "rt_synth.cpp"]
+SOURCES = ["rt_api.hip", "rt_kernels.hip", "rt_attn_prefill.hip", "rt_gemv.hip", "rt_gemv_mb.hip", "rt_gemm.hip", "rt_hgemm.hip", "rt_llama.hip", "rt_synth.cpp"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are kept out of the generated code on purpose.
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-munsafe-fp-atomics",  # f32 atomic adds of the split-k GEMM epilogue as hardware atomics (device memory only)
+    "-munsafe-fp-atomics",  # the GEMV's in-place residual add (y += row sum) as a returnless hardware f32 atomic (device memory only)
     "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]
 
@@ -49,7 +49,7 @@ def find_hipcc() -> str:
 # Kernels whose speed depends on running without private (scratch) memory: the build fails if the compiler gave
 # one of them a scratch frame (register spills or an array it could not keep in registers).  One spilling variant
 # inside such a kernel slows every launch of it, also the ones that never reach the variant.
-NO_SCRATCH = {"rt_gemv.hip": ("qgemv_kernel",), "rt_gemm.hip": ("qgemm_kernel",), "rt_attn_prefill.hip": ("attn_causal_kernel",),
+NO_SCRATCH = {"rt_gemv.hip": ("qgemv_kernel", "qgemv_lean_kernel"), "rt_gemm.hip": ("qgemm_kernel",), "rt_attn_prefill.hip": ("attn_causal_kernel",),
               "rt_hgemm.hip": ("hgemm_kernel",), "rt_gemv_mb.hip": ("qgemv_mb_q4k_kernel", "qgemv_mb_q6k_kernel")}
 RESOURCE_FLAG = "-Rpass-analysis=kernel-resource-usage"
 

@@ -742,4 +742,11 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
     }
 }
 
+// The problem a workgroup of the grouped launch belongs to.  A macro, so that the kernel indexes its argument structure
+// where it lies (handing the structure to a function by reference makes the compiler copy all of it to private memory).
+#define RT_GEMV_PICK_PROBLEM(args, wg, pi)                   \
+    int pi = 0;                                              \
+    _Pragma("unroll") for (int i_ = 1; i_ < rt::kMaxGemvProbs; i_++) \
+        if (i_ < (args).n && (wg) >= (args).p[i_].tile0) pi = i_
+
 }  // namespace rt

@@ -100,6 +100,19 @@ inline int emu_sdot4(int a, int b, int c) {
     return c;
 }
 #define __builtin_amdgcn_sdot4(a, b, c, clamp) emu_sdot4(a, b, c)
+// v_perm_b32: byte i of the result is byte sel_i of the eight bytes { s1 (0..3), s0 (4..7) }; selectors from 12 up give constants
+inline unsigned emu_perm(unsigned s0, unsigned s1, unsigned sel) {
+    const unsigned long long src = ((unsigned long long)s0 << 32) | s1;
+    unsigned r = 0;
+    for (int i = 0; i < 4; i++) {
+        const unsigned k = (sel >> (8 * i)) & 0xFF;
+        const unsigned byte = k < 8 ? (unsigned)(src >> (8 * k)) & 0xFF : (k >= 13 ? 0xFFu : 0u);
+        r |= byte << (8 * i);
+    }
+    return r;
+}
+#define __builtin_amdgcn_perm(a, b, sel) emu_perm(a, b, sel)
+inline void unsafeAtomicAdd(float *p, float v) { *p += v; }
 // buffer resources: base pointer only (the emulation neither checks ranges nor strides), loads at base + voffset + soffset
 struct emu_buffer_rsrc { const unsigned char *base; };
 typedef emu_buffer_rsrc __amdgpu_buffer_rsrc_t;
