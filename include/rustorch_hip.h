@@ -23,7 +23,9 @@
  *     of CudaKernelExecutor::matmul_f32, src/gpu/cuda_kernels.rs:231-283).
  *   - a context may be moved between threads; calls on one context are
  *     serialised internally; distinct contexts are independent.  There is no
- *     global mutable state (contrast src/gpu/mod.rs:757-772).
+ *     global mutable state (contrast src/gpu/mod.rs:757-772) apart from atomic
+ *     per-device flags that record that a kernel's LDS limit has been raised
+ *     (setting it twice is harmless, so they need no lock).
  */
 #ifndef RUSTORCH_HIP_H
 #define RUSTORCH_HIP_H
@@ -135,7 +137,9 @@ RT_HIP_API int rt_hip_qmatmul_i8(rt_hip_ctx *ctx, const int8_t *a, float scale_a
  *      to HBM byte for byte.  nbytes must equal n_rows*(n_cols/block_elems)*block_bytes. */
 RT_HIP_API int rt_hip_qweight_upload(rt_hip_ctx *ctx, int ggml_type, size_t n_rows, size_t n_cols,
                                      const void *raw_blocks, size_t nbytes, rt_hip_qweight **out);
-/* Wrap blocks that are already in device memory (no copy; the caller keeps ownership of dev_blocks). */
+/* Wrap blocks that are already in device memory (no copy; the caller keeps ownership of dev_blocks).  The kernels read
+ * rows with 16-byte loads that may start inside a row's last block: dev_blocks must be 16-byte aligned and be followed by
+ * at least 64 readable bytes beyond nbytes (rt_hip_qweight_upload allocates that slack itself). */
 RT_HIP_API int rt_hip_qweight_wrap_dev(rt_hip_ctx *ctx, int ggml_type, size_t n_rows, size_t n_cols,
                                        const void *dev_blocks, size_t nbytes, rt_hip_qweight **out);
 RT_HIP_API int rt_hip_qweight_free(rt_hip_ctx *ctx, rt_hip_qweight *w);

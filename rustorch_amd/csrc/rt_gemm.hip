@@ -29,6 +29,7 @@
 #include "rt_device.h"
 
 #include <algorithm>
+#include <atomic>
 #include <type_traits>
 #include <cstring>
 
@@ -802,13 +803,15 @@ hipError_t launch_cfg(hipStream_t s, const GemmPlan &p, const uint8_t *w, size_t
     constexpr int BM = 32 * MF, BN = 32 * NW;
     const size_t lds = (size_t)4 * BM * kBK * sizeof(_Float16) + (size_t)NW * WGeo<TYPE>::stage_bytes;
     auto kern = qgemm_kernel<TYPE, NW, MF>;
-    static bool attr_set[64] = {};     // per instantiation and device: the attribute belongs to the function as loaded on a device
+    // Per instantiation and device (the attribute belongs to the function as loaded on a device).  Only a cache of "already
+    // asked": setting the attribute twice is harmless, so two threads that both find the flag clear just both set it.
+    static std::atomic<bool> attr_set[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorInvalidDevice;
-    if (!attr_set[dev] && lds > 64 * 1024) {
+    if (lds > 64 * 1024 && !attr_set[dev].load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        attr_set[dev] = true;
+        attr_set[dev].store(true, std::memory_order_release);
     }
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
     const int one = tiles_m * p.ksplit * tiles_n, total = w2 ? 2 * one : one;

@@ -75,47 +75,8 @@ struct QuantGroupArgs {
     int n;
 };
 
-// ---- persistent decode-step kernel (rt_mega.hip)
-struct MegaLayer {
-    const uint8_t *wq, *wk, *wv, *wo, *wgate, *wup, *wdown;
-    size_t rb_q, rb_k, rb_v, rb_o, rb_g, rb_d;
-    int t_q, t_k, t_v, t_o, t_g, t_d;
-    const float *attn_norm, *ffn_norm;
-    uint16_t *kc, *vc;  // this layer's fp16 cache rows [max_pos][hidden]
-};
-struct MegaArgs {
-    const MegaLayer *layers;  // device array
-    int n_layers, hidden, n_heads, head_dim, ffn, vocab, max_pos;
-    float eps;
-    const uint8_t *embd; size_t rb_embd; int t_embd;
-    const uint8_t *wout; size_t rb_out; int t_out;
-    const float *out_norm;
-    float *x, *q, *k, *v, *a, *f, *logits;
-    const float *inv_freq;
-    int *state;          // [0] pos, [1] token, [2] pick, [3] step
-    const int *forced;   // optional: token fed at the next step
-    int *out_tokens;     // optional: picks by step
-    unsigned *bar;       // kMegaBarBytes of barrier words, zeroed by the launcher
-    int wg_q, wg_k;      // workgroups given to the q and k matrices in the q/k/v phase (v takes the rest)
-    int want_logits, do_advance;
-};
-constexpr size_t kMegaBarBytes = 4096;
-constexpr size_t kMegaErrWord = 32 * 24;  // index of the time-out flag inside the barrier words
-constexpr int kMegaThreads = 1024;
-// Launch-sized LDS of the step kernel: the larger of the GEMV staging area, the attention phase
-// (q / k / v of the step, per-group partial outputs, scores) and the greedy-pick scratch.
-inline size_t mega_lds_bytes(int hidden, int ffn, int head_dim, int max_pos) {
-    size_t g = xq_stride((size_t)(hidden > ffn ? hidden : ffn));
-    size_t a = ((size_t)3 * head_dim + (size_t)(kMegaThreads / (head_dim / 8)) * head_dim + (size_t)max_pos) * sizeof(float);
-    size_t m = g > a ? g : a;
-    size_t am = (size_t)2 * kMegaThreads * sizeof(float);
-    return m > am ? m : am;
-}
-int mega_grid(int device, size_t lds_bytes);
-hipError_t launch_llama_step(hipStream_t s, MegaArgs &a, int grid, size_t lds_bytes);
-hipError_t launch_set_state(hipStream_t s, int *state, int pos, int token, int step);
-
 // ---- launchers (all enqueue on `s`, return hipError_t of the launch)
+hipError_t launch_set_state(hipStream_t s, int *state, int pos, int token, int step);
 hipError_t launch_quantize_x(hipStream_t s, const float *x, uint8_t *xq, size_t K, size_t batch);
 hipError_t launch_quantize_group(hipStream_t s, const QuantGroupArgs &a);
 hipError_t launch_qgemv(hipStream_t s, GemvArgs &args, int batch);  // fills tile0 / rows_per_tile

@@ -47,19 +47,13 @@ struct rt_hip_llama {
     int *forced_dev = nullptr, *out_tokens_dev = nullptr;
     int n_fed = 0;
     // persistent step kernel
-    int mode = 1;             // 0: persistent step kernel, 1: separate launches (default), 2: the same launches replayed from a captured graph
+    int mode = 1;             // 1: separate launches (default), 2: the same launches replayed from a captured graph (0, a persistent step kernel, is refused)
     // mode 2: one graph per (want_logits, advance, use_forced); a combination runs eagerly once, is captured at its
     // second use and replayed from then on.  Every argument of a step is a device pointer or a model constant
     // (position and token live in `state`), so one capture serves every later token.
     struct StepGraph { int uses = 0; hipGraph_t graph = nullptr; hipGraphExec_t exec = nullptr; };
     StepGraph step_graphs[8];
-    bool mega_ready = false;  // layer table uploaded and launch shape decided
-    bool mega_ok = false;
-    rt::MegaLayer *mega_layers = nullptr;
     float *a = nullptr;       // attention output, f32
-    unsigned *bar = nullptr;
-    int mega_grid = 0, wg_q = 0, wg_k = 0;
-    size_t mega_lds = 0;
     // batched prefill (dense contraction path): activations of up to pf_cap tokens
     size_t pf_cap = 0;
     float *pf_x = nullptr, *pf_x2 = nullptr, *pf_n = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_a = nullptr;
@@ -235,12 +229,13 @@ struct PrefillGemm {
             }
             RT_TRY_HIP(ctx, rt::launch_hgemm(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, X, M, Y, res, ctx->scratch,
                                              ctx->scratch_bytes, t.f16));
+            prepared = nullptr;      // this contraction's own form of X now lies where the matrix-core pre-pass keeps its
             return RT_HIP_OK;
         }
         const bool mc = rt::qgemm_on_matrix_cores(t.type, M, t.n_rows, t.n_cols) && res != Y;
         RT_TRY_HIP(ctx, rt::launch_qgemm(ctx->stream, t.type, t.dev, t.n_rows, t.n_cols, t.row_bytes, X, M, Y, res, ctx->scratch, ctx->scratch_bytes,
                                          mc && prepared == X));
-        if (mc) prepared = X;
+        prepared = mc ? X : nullptr;      // every other branch of launch_qgemm may use the workspace for something else
         return RT_HIP_OK;
     }
     // n matrices against the same rows of X (q, k, v; gate, up).  3..15 rows of Q4_K / Q6_K: the rows are quantized once
@@ -433,7 +428,7 @@ int rt_hip_llama_create(rt_hip_ctx *ctx, const rt_hip_llama_config *cfg, rt_hip_
     A((void **)&m->xq_h, rt::xq_stride(H)); A((void **)&m->xq_a, rt::xq_stride(H)); A((void **)&m->xq_f, rt::xq_stride(F));
     A((void **)&m->inv_freq, (size_t)(hd / 2) * 4); A((void **)&m->state, 4 * sizeof(int));
     A((void **)&m->forced_dev, (P + 1) * sizeof(int)); A((void **)&m->out_tokens_dev, (P + 1) * sizeof(int));
-    A((void **)&m->a, H * 4); A((void **)&m->bar, rt::kMegaBarBytes); A((void **)&m->mega_layers, L * sizeof(rt::MegaLayer));
+    A((void **)&m->a, H * 4);
     if (rc != RT_HIP_OK) { free_all(m); delete m; return rc; }
     std::vector<float> inv((size_t)hd / 2);
     for (int i = 0; i < hd / 2; i++) inv[(size_t)i] = (float)std::pow((double)cfg->rope_theta, -2.0 * (double)i / (double)hd);
@@ -490,7 +485,6 @@ int rt_hip_llama_upload_tensor(rt_hip_ctx *ctx, rt_hip_llama *m, int slot, int l
                    nbytes, n_rows, n_cols, ggml_type);
     }
     Guard g(ctx);
-    m->mega_ready = false;
     void *dev = nullptr;
     drop_step_graphs(m);      // a captured step names the old buffer of this slot
     int rc = dev_alloc(ctx, m, &dev, nbytes + 64);
@@ -530,63 +524,9 @@ int rt_hip_llama_reset(rt_hip_ctx *ctx, rt_hip_llama *m) {
     return RT_HIP_OK;
 }
 
-// Decide whether the persistent step kernel can serve this model and upload its layer table.
-static int ensure_mega(rt_hip_ctx *ctx, rt_hip_llama *m) {
-    if (m->mega_ready) return RT_HIP_OK;
-    const rt_hip_llama_config &c = m->cfg;
-    m->mega_ok = false;
-    bool same = true;
-    for (int l = 0; l < c.n_layers; l++) same = same && m->wgate[l].type == m->wup[l].type;
-    m->mega_lds = rt::mega_lds_bytes(c.hidden, c.ffn, m->head_dim, c.max_pos);
-    same = same && m->n_kv == c.n_heads;      // the step kernel knows one head count
-    m->mega_grid = same ? rt::mega_grid(ctx->device, m->mega_lds) : 0;
-    if (m->mega_grid >= 8 && m->mega_grid >= c.n_heads) {
-        std::vector<rt::MegaLayer> tab((size_t)c.n_layers);
-        const size_t H = (size_t)c.hidden;
-        for (int l = 0; l < c.n_layers; l++) {
-            rt::MegaLayer &t = tab[(size_t)l];
-            t.wq = m->wq[l].dev; t.wk = m->wk[l].dev; t.wv = m->wv[l].dev; t.wo = m->wo[l].dev;
-            t.wgate = m->wgate[l].dev; t.wup = m->wup[l].dev; t.wdown = m->wdown[l].dev;
-            t.rb_q = m->wq[l].row_bytes; t.rb_k = m->wk[l].row_bytes; t.rb_v = m->wv[l].row_bytes; t.rb_o = m->wo[l].row_bytes;
-            t.rb_g = m->wgate[l].row_bytes; t.rb_d = m->wdown[l].row_bytes;
-            t.t_q = m->wq[l].type; t.t_k = m->wk[l].type; t.t_v = m->wv[l].type; t.t_o = m->wo[l].type;
-            t.t_g = m->wgate[l].type; t.t_d = m->wdown[l].type;
-            t.attn_norm = m->attn_norm[l]; t.ffn_norm = m->ffn_norm[l];
-            t.kc = m->kcache + (size_t)l * (size_t)c.max_pos * H;
-            t.vc = m->vcache + (size_t)l * (size_t)c.max_pos * H;
-        }
-        RT_TRY_HIP(ctx, hipMemcpyAsync(m->mega_layers, tab.data(), tab.size() * sizeof(rt::MegaLayer), hipMemcpyHostToDevice, ctx->stream));
-        RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
-        // q / k / v share the workgroups in proportion to their bytes (layer 0 is representative)
-        double bq = (double)m->wq[0].nbytes, bk = (double)m->wk[0].nbytes, bv = (double)m->wv[0].nbytes, tot = bq + bk + bv;
-        m->wg_q = (int)(m->mega_grid * bq / tot + 0.5);
-        m->wg_k = (int)(m->mega_grid * bk / tot + 0.5);
-        if (m->wg_q < 1) m->wg_q = 1;
-        if (m->wg_k < 1) m->wg_k = 1;
-        if (m->wg_q + m->wg_k > m->mega_grid - 1) { m->wg_q = m->mega_grid / 3; m->wg_k = m->mega_grid / 3; }
-        m->mega_ok = true;
-    }
-    m->mega_ready = true;
-    return RT_HIP_OK;
-}
-
 // Enqueue the step for the token in the device state.  advance: afterwards the state names the next token
 // (forced_dev[step] when use_forced, else the pick) and the next position.
 static int enqueue_token(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits, bool advance, bool use_forced) {
-    if (m->mode == 0 && m->mega_ok) {
-        const rt_hip_llama_config &c = m->cfg;
-        rt::MegaArgs a;
-        memset(&a, 0, sizeof a);
-        a.layers = m->mega_layers; a.n_layers = c.n_layers; a.hidden = c.hidden; a.n_heads = c.n_heads; a.head_dim = m->head_dim;
-        a.ffn = c.ffn; a.vocab = c.vocab; a.max_pos = c.max_pos; a.eps = c.rms_eps;
-        a.embd = m->tok_embd.dev; a.rb_embd = m->tok_embd.row_bytes; a.t_embd = m->tok_embd.type;
-        a.wout = m->output.dev; a.rb_out = m->output.row_bytes; a.t_out = m->output.type; a.out_norm = m->out_norm;
-        a.x = m->x; a.q = m->q; a.k = m->k; a.v = m->v; a.a = m->a; a.f = m->g; a.logits = m->logits;
-        a.inv_freq = m->inv_freq; a.state = m->state; a.forced = use_forced ? m->forced_dev : nullptr; a.out_tokens = m->out_tokens_dev;
-        a.bar = m->bar; a.wg_q = m->wg_q; a.wg_k = m->wg_k; a.want_logits = want_logits ? 1 : 0; a.do_advance = advance ? 1 : 0;
-        RT_TRY_HIP(ctx, rt::launch_llama_step(ctx->stream, a, m->mega_grid, m->mega_lds));
-        return RT_HIP_OK;
-    }
     auto enqueue = [&]() -> int {
         int rc = enqueue_step(ctx, m, want_logits);
         if (rc) return rc;
@@ -621,16 +561,6 @@ static int enqueue_token(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits, boo
     return RT_HIP_OK;
 }
 
-// After a synchronisation: did a grid barrier of the persistent kernel time out?
-static int check_barrier_flag(rt_hip_ctx *ctx, rt_hip_llama *m) {
-    if (!(m->mode == 0 && m->mega_ok)) return RT_HIP_OK;
-    unsigned flag = 0;
-    RT_TRY_HIP(ctx, hipMemcpyAsync(&flag, m->bar + rt::kMegaErrWord, sizeof flag, hipMemcpyDeviceToHost, ctx->stream));
-    RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    RT_REQUIRE(ctx, flag == 0, RT_HIP_ERR_HIP, "decode step kernel: a grid barrier timed out (device busy with other work?)");
-    return RT_HIP_OK;
-}
-
 int rt_hip_llama_set_mode(rt_hip_ctx *ctx, rt_hip_llama *m, int mode) {
     if (!ctx || !m) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_set_mode: NULL argument");
     RT_REQUIRE(ctx, mode >= 0 && mode <= 2, RT_HIP_ERR_INVALID_ARG,
@@ -652,8 +582,6 @@ int rt_hip_llama_step(rt_hip_ctx *ctx, rt_hip_llama *m, int token, int pos, int 
     int rc = check_complete(ctx, m);
     if (rc) return rc;
     Guard g(ctx);
-    rc = ensure_mega(ctx, m);
-    if (rc) return rc;
     RT_TRY_HIP(ctx, rt::launch_set_state(ctx->stream, m->state, pos, token, 0));
     rc = enqueue_token(ctx, m, true, false, false);
     if (rc) return rc;
@@ -661,7 +589,7 @@ int rt_hip_llama_step(rt_hip_ctx *ctx, rt_hip_llama *m, int token, int pos, int 
     if (next_token) {
         RT_TRY_HIP(ctx, hipMemcpyAsync(next_token, m->state + 2, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
         RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
-        return check_barrier_flag(ctx, m);
+        return RT_HIP_OK;
     }
     return RT_HIP_OK;
 }
@@ -708,8 +636,6 @@ int rt_hip_llama_prefill(rt_hip_ctx *ctx, rt_hip_llama *m, const int *tokens, in
         m->n_fed = pos0 + n_tok;
         return RT_HIP_OK;
     }
-    rc = ensure_mega(ctx, m);
-    if (rc) return rc;
     // forced_dev[i] = token fed after step i (the last entry repeats the last token and is never used)
     std::vector<int> next((size_t)n_tok);
     for (int i = 0; i < n_tok; i++) next[(size_t)i] = tokens[i + 1 < n_tok ? i + 1 : i];
@@ -729,7 +655,7 @@ int rt_hip_llama_logits(rt_hip_ctx *ctx, rt_hip_llama *m, float *logits_host) {
     Guard g(ctx);
     RT_TRY_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
     RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    return check_barrier_flag(ctx, m);
+    return RT_HIP_OK;
 }
 
 int rt_hip_llama_decode(rt_hip_ctx *ctx, rt_hip_llama *m, int first_token, int pos0, int n_steps, const int *forced,
@@ -745,8 +671,6 @@ int rt_hip_llama_decode(rt_hip_ctx *ctx, rt_hip_llama *m, int first_token, int p
     int rc = check_complete(ctx, m);
     if (rc) return rc;
     Guard g(ctx);
-    rc = ensure_mega(ctx, m);
-    if (rc) return rc;
     if (forced) {
         RT_TRY_HIP(ctx, hipMemcpyAsync(m->forced_dev, forced, (size_t)n_steps * sizeof(int), hipMemcpyHostToDevice, ctx->stream));
         RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -759,7 +683,7 @@ int rt_hip_llama_decode(rt_hip_ctx *ctx, rt_hip_llama *m, int first_token, int p
     m->n_fed = pos0 + n_steps;
     RT_TRY_HIP(ctx, hipMemcpyAsync(out_tokens, m->out_tokens_dev, (size_t)n_steps * sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
     RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    return check_barrier_flag(ctx, m);
+    return RT_HIP_OK;
 }
 
 }  // extern "C"

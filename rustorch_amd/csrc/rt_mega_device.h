@@ -14,6 +14,10 @@
 // drains the workgroup's own stores and then synchronises on counters.  Weights and the KV cache of
 // earlier tokens are read-only during a launch and use the normal cached path.
 //
+// State of this code: NOT part of the library.  Its one run on the GPU ended in a memory fault whose cause has not been
+// found, so no translation unit of the product includes this header and rt_hip_llama_set_mode refuses mode 0; what
+// remains is the device code and its CPU run as fibers under AddressSanitizer (tests/emu/emu_main.cpp).
+//
 // Barrier: two levels (8 group counters on separate cache lines, one top counter, one generation flag);
 // every spin is bounded, a time-out raises an error flag that makes all workgroups leave the kernel.
 #pragma once
@@ -21,6 +25,44 @@
 #include "rt_gemv_device.h"
 
 namespace rt {
+
+// ---- arguments of the step kernel
+struct MegaLayer {
+    const uint8_t *wq, *wk, *wv, *wo, *wgate, *wup, *wdown;
+    size_t rb_q, rb_k, rb_v, rb_o, rb_g, rb_d;
+    int t_q, t_k, t_v, t_o, t_g, t_d;
+    const float *attn_norm, *ffn_norm;
+    uint16_t *kc, *vc;  // this layer's fp16 cache rows [max_pos][hidden]
+};
+struct MegaArgs {
+    const MegaLayer *layers;  // device array
+    int n_layers, hidden, n_heads, head_dim, ffn, vocab, max_pos;
+    float eps;
+    const uint8_t *embd; size_t rb_embd; int t_embd;
+    const uint8_t *wout; size_t rb_out; int t_out;
+    const float *out_norm;
+    float *x, *q, *k, *v, *a, *f, *logits;
+    const float *inv_freq;
+    int *state;          // [0] pos, [1] token, [2] pick, [3] step
+    const int *forced;   // optional: token fed at the next step
+    int *out_tokens;     // optional: picks by step
+    unsigned *bar;       // kMegaBarBytes of barrier words, zeroed by the launcher
+    int wg_q, wg_k;      // workgroups given to the q and k matrices in the q/k/v phase (v takes the rest)
+    int want_logits, do_advance;
+};
+constexpr size_t kMegaBarBytes = 4096;
+constexpr size_t kMegaErrWord = 32 * 24;  // index of the time-out flag inside the barrier words
+constexpr int kMegaThreads = 1024;
+// Launch-sized LDS of the step kernel: the larger of the GEMV staging area, the attention phase
+// (q / k / v of the step, per-group partial outputs, scores) and the greedy-pick scratch.
+inline size_t mega_lds_bytes(int hidden, int ffn, int head_dim, int max_pos) {
+    size_t g = xq_stride((size_t)(hidden > ffn ? hidden : ffn));
+    size_t a = ((size_t)3 * head_dim + (size_t)(kMegaThreads / (head_dim / 8)) * head_dim + (size_t)max_pos) * sizeof(float);
+    size_t m = g > a ? g : a;
+    size_t am = (size_t)2 * kMegaThreads * sizeof(float);
+    return m > am ? m : am;
+}
+
 
 constexpr unsigned kSpinLimit = 1u << 21;
 constexpr unsigned kBarGroups = 8;
