@@ -23,6 +23,30 @@ def test_header_symbols_are_exported_and_bound(lib):
     assert sorted(syms) == sorted(_lib.SIGNATURES), "ctypes table and header disagree"
 
 
+def test_rust_binding_in_the_integration_notes_is_generated_from_the_header():
+    """INTEGRATION.md holds the Rust `extern "C"` module a maintainer would add; it is generated from the header, declares
+    every exported function with the header's argument count, pointer-ness and return kind, and agrees with the ctypes table."""
+    import ctypes as C
+    from rustorch_amd import _lib, ffi_gen
+    assert ffi_gen.doc_block() == ffi_gen.generate(), "run python -m rustorch_amd.ffi_gen --write"
+    block = ffi_gen.doc_block()
+    decls = dict(re.findall(r"^    pub fn (rt_\w+)\((.*)\) -> [^;]+;$", block, flags=re.M))
+    rets = dict(re.findall(r"^    pub fn (rt_\w+)\(.*\) -> ([^;]+);$", block, flags=re.M))
+    stubs = set(re.findall(r"^    pub unsafe fn (rt_\w+)\(", block, flags=re.M))
+    assert sorted(decls) == sorted(header_symbols()) and stubs == set(decls)
+    for name, (res, args) in _lib.SIGNATURES.items():
+        rust_args = [a.split(": ", 1)[1] for a in decls[name].split(", ")] if decls[name] else []
+        assert len(rust_args) == len(args), name
+        for ra, ca in zip(rust_args, args):
+            is_ptr = ra.startswith("*")
+            c_ptr = ca in (C.c_void_p, C.c_char_p) or hasattr(ca, "contents")
+            assert is_ptr == c_ptr, "%s: %s against %s" % (name, ra, ca)
+            if not is_ptr:
+                want = {C.c_int: ("i32",), C.c_float: ("f32",)}.get(ca, ("usize", "u64"))       # size_t and uint64_t are one ctypes class here
+                assert ra in want, "%s: %s against %s" % (name, ra, ca)
+        assert rets[name] == {C.c_int: "i32", C.c_size_t: "usize", C.c_char_p: "*const std::os::raw::c_char"}[res], name
+
+
 def test_static_archive_holds_the_same_entry_points(lib):
     import subprocess
     a = ROOT / "rustorch_amd" / "librustorch_hip.a"

@@ -97,6 +97,26 @@ def test_tensor_table_alignment_and_payload(tmpfile):
     assert g.tensor_data_offset + last.offset + last.n_bytes == g.file_size
 
 
+def test_reference_scalar_decode_vectors(tmpfile):
+    """The reference loader's own known-answer vectors for the unquantized element types
+    (example-cli/src/model/formats/tensor_loader.rs:323-356): F32 `00 00 80 3F` -> 1.0, I8 `00 7F FF` -> 0, 127, -1,
+    I16 `00 00 01 00` -> 0, 1, I32 `00 00 00 00 01 00 00 00` -> 0, 1, and a payload whose length is no multiple of the
+    element size is an error."""
+    f32, i8, i16, i32 = b"\x00\x00\x80\x3f", b"\x00\x7f\xff", b"\x00\x00\x01\x00", b"\x00\x00\x00\x00\x01\x00\x00\x00"
+    data = f32 + b"\0" * 28 + i8 + b"\0" * 29 + i16 + b"\0" * 28 + i32
+    blob = build([], [tinfo("f", (1,), 0, 0), tinfo("b", (3,), 16, 32), tinfo("h", (2,), 17, 64), tinfo("w", (2,), 18, 96)], data)
+    g = GGUFLoader(tmpfile(blob))
+    assert g.load_f32("f").tolist() == [1.0]
+    assert g.load_f32("b").tolist() == [0.0, 127.0, -1.0]
+    assert g.load_f32("h").tolist() == [0.0, 1.0]
+    assert g.load_f32("w").tolist() == [0.0, 1.0]
+    assert all(g.load_f32(n).dtype == np.float32 for n in "fbhw")
+    # three bytes where an f32 tensor of one element is declared: the read runs past the end of the file
+    short = build([], [tinfo("f", (1,), 0, 0)], b"\x00\x00\x00")
+    with pytest.raises(GGUFError):
+        GGUFLoader(tmpfile(short)).load_f32("f")
+
+
 def test_stated_alignment_is_honoured(tmpfile):
     data = b"\x00\x00\x80\x3f"
     blob = build([kv("general.alignment", 4, struct.pack("<I", 64))], [tinfo("x", (1,), 0, 0)], data, align=64)
