@@ -13,13 +13,39 @@ def build_pair(ex, orc, seed, n_layers, hidden, n_heads, ffn, vocab, max_pos, n_
     gm = llama.HipLlama(ex, n_layers, hidden, n_heads, ffn, vocab, max_pos, n_kv_heads=n_kv_heads)
     om = orc.OracleLlama(n_layers, hidden, n_heads, ffn, vocab, max_pos, n_kv_heads=n_kv_heads)
     head = {}
+    om.attn_norms = {}                                          # layer -> gamma, for stable_positions
 
     def sink(slot, layer, t, r, c, raw):
         om.set_tensor(slot, layer, t, r, c, raw)
         if slot == "output":
             head["wn"] = np.linalg.norm(orc.dequant(t, raw, r, c).astype(np.float64), axis=1)
+        if slot == "attn_norm":
+            om.attn_norms[layer] = np.array(raw, dtype=np.float32)
     llama.load_synthetic(gm, seed, sink)
     return gm, om, head["wn"]
+
+
+def stable_positions(om, toks, want, tol, rel=3e-4, frac=0.02):
+    """Positions at which the oracle itself is well conditioned.
+
+    The tiny random models of this file have attention scores in the thousands, so a softmax is one-hot, and where two
+    scores nearly tie an input change far below any kernel's rounding moves the attended row -- and the logits by many
+    tolerances -- in the oracle just as on the GPU.  To tell those positions from real kernel errors the oracle is run a
+    second and a third time with every attention-norm weight multiplied by 1 + rel * N(0, 1) (rel = 3e-4: ten times the relative
+    rounding of the GPU's 15-bit activations): a position whose oracle logits move by more than `frac` of the tolerance in either run is
+    ill conditioned and exempt from the bound on the maximum; every other position has to keep the bound itself."""
+    rng = np.random.default_rng(12345)
+    n_layers = len(om.attn_norms)
+    hidden = om.attn_norms[0].size
+    ok = np.ones(len(toks), dtype=bool)
+    for draw in range(2):                                       # two independent directions: a tie that one misses the other meets
+        for l in range(n_layers):
+            om.set_tensor("attn_norm", l, 0, 1, hidden, (om.attn_norms[l] * (1.0 + rel * rng.standard_normal(hidden))).astype(np.float32))
+        moved = om.forward(toks, 0)
+        ok &= (np.abs(moved - want) / tol).max(axis=1) <= frac
+    for l in range(n_layers):
+        om.set_tensor("attn_norm", l, 0, 1, hidden, om.attn_norms[l])
+    return ok
 
 
 def logit_tol(wn, hidden):
@@ -125,20 +151,23 @@ def test_grouped_query_attention_model(ex, orc, n_heads, n_kv):
     toks = synth.tokens(31, synth.TID_PROMPT, 40, cfg["vocab"])
     want = om.forward(toks, 0)
     tol = logit_tol(wn, cfg["hidden"])
-    ratios = []
+    stable = stable_positions(om, toks, want, tol)
+    ratios, at = [], []
     for p, t in enumerate(toks[:24]):
         gm.step(int(t), p); twin.step(int(t), p)
         got = gm.logits()
         assert np.array_equal(got, twin.logits()), "position %d" % p
-        ratios.append(float((np.abs(got - want[p]) / tol).max()))
+        ratios.append(float((np.abs(got - want[p]) / tol).max())); at.append(p)
     gm.reset()
     gm.prefill(toks[:30], 0)                                     # 30 tokens: the dense-contraction path
-    ratios.append(float((np.abs(gm.logits() - want[29]) / tol).max()))
+    ratios.append(float((np.abs(gm.logits() - want[29]) / tol).max())); at.append(29)
     out = gm.decode(int(toks[30]), 30, 9, toks[31:40])           # teacher forced continuation on the device
-    ratios.append(float((np.abs(gm.logits() - want[38]) / tol).max()))
-    ratios = np.array(ratios)
-    print("ratio to the tolerance: median %.3f, max %.2f, %d of %d above 1" % (np.median(ratios), ratios.max(), (ratios > 1).sum(), ratios.size), flush=True)
+    ratios.append(float((np.abs(gm.logits() - want[38]) / tol).max())); at.append(38)
+    ratios, ok = np.array(ratios), stable[np.array(at)]
+    print("ratio to the tolerance: median %.3f, max %.2f, %d of %d above 1; well-conditioned positions: %d, max %.3f"
+          % (np.median(ratios), ratios.max(), (ratios > 1).sum(), ratios.size, ok.sum(), ratios[ok].max() if ok.any() else 0.0), flush=True)
     assert np.median(ratios) <= 0.1 and (ratios <= 1).mean() >= 0.9
+    assert np.all(ratios[ok] <= 1.0), "positions %s" % [a for a, r, k in zip(at, ratios, ok) if k and r > 1.0]
     with pytest.raises(ShapeMismatch):                           # k must have n_kv * head_dim rows
         gm.upload("attn_k", 0, 12, 512, 512, synth.blocks(12, 1, 1, 512, 512))
 
@@ -158,7 +187,8 @@ def test_long_context_attention_split_over_workgroups(ex, orc, n_heads, n_kv):
     toks = synth.tokens(37, synth.TID_PROMPT, 420, base["vocab"])
     want = om.forward(toks, 0)
     tol = logit_tol(wn, base["hidden"])
-    ratios, between = [], []
+    stable = stable_positions(om, toks, want, tol)
+    ratios, between, at = [], [], []
     for n0 in (1, 112, 352):                      # the first steps, then across the chunk boundaries at 120 and 360
         split.reset(); single.reset()
         split.prefill(toks[:n0], 0); single.prefill(toks[:n0], 0)
@@ -166,12 +196,15 @@ def test_long_context_attention_split_over_workgroups(ex, orc, n_heads, n_kv):
             split.step(int(toks[p]), p); single.step(int(toks[p]), p)
             a, b = split.logits(), single.logits()
             between.append(float((np.abs(a - b) / tol).max()))
-            ratios.append(float((np.abs(a - want[p]) / tol).max()))
-    ratios, between = np.array(ratios), np.array(between)
-    print("split vs single: max %.3f of the tolerance; split vs oracle: median %.3f, max %.2f" % (between.max(), np.median(ratios), ratios.max()), flush=True)
+            ratios.append(float((np.abs(a - want[p]) / tol).max())); at.append(p)
+    ratios, between, ok = np.array(ratios), np.array(between), stable[np.array(at)]
+    print("split vs single: max %.3f of the tolerance; split vs oracle: median %.3f, max %.2f; well-conditioned positions: %d of %d, max %.3f"
+          % (between.max(), np.median(ratios), ratios.max(), ok.sum(), ok.size, ratios[ok].max() if ok.any() else 0.0), flush=True)
     assert between.max() <= 0.1
-    # with hundreds of positions near-ties of the one-hot softmax are frequent: only the typical position is held to the oracle
+    # with hundreds of positions near-ties of the one-hot softmax are frequent: the typical position is held to the oracle,
+    # and so is every position at which the oracle itself is well conditioned
     assert np.median(ratios) <= 0.2
+    assert np.all(ratios[ok] <= 1.0), "positions %s" % [a for a, r, k in zip(at, ratios, ok) if k and r > 1.0]
 
 
 def test_70b_class_widths(ex, orc):
@@ -225,12 +258,19 @@ def test_prefill_in_several_passes_and_calls(ex, orc):
     print("one call vs stepped %.3f, two calls vs stepped %.3f, vs oracle %.3f of the tolerance" % (d1, d2, r), flush=True)
     assert d1 <= 0.1 and d2 <= 0.1
     # the cache the passes left serves the decode steps that follow
+    stable = stable_positions(om, toks, want, tol)
     ratios = []
     gm.reset(); gm.prefill(toks[:n], 0)
     for p in range(n, n + 12):
         gm.step(int(toks[p]), p)
         ratios.append(float((np.abs(gm.logits() - want[p]) / tol).max()))
+    ratios, ok = np.array(ratios), stable[n:n + 12]
+    print("steps after the passes: median %.3f, max %.2f; well-conditioned positions: %d of 12, max %.3f"
+          % (np.median(ratios), ratios.max(), ok.sum(), ratios[ok].max() if ok.any() else 0.0), flush=True)
     assert np.median(ratios) <= 0.2
+    assert np.all(ratios[ok] <= 1.0)
+    if stable[n - 1]:
+        assert r <= 1.0
 
 
 def test_short_prompts_take_the_batched_pass(ex, orc):
