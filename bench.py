@@ -42,6 +42,26 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def timed_regions(ex, region, min_ms=10.0, max_regions=500):
+    """Times `region()` -- a callable that enqueues a fixed number of launches -- between two events and a synchronisation on
+    both sides, again and again until at least `min_ms` of device time have been measured (at least three regions).  Returns
+    the median region: (milliseconds between the events, wall seconds, number of regions).  A region of 20 launches of
+    30 us is 0.6 ms, too short to hang a headline on; the median over the repeats is what is reported."""
+    ev, wall, total = [], [], 0.0
+    while (total < min_ms or len(ev) < 3) and len(ev) < max_regions:
+        e0, e1 = ex.event(), ex.event()
+        ex.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        region()
+        e1.record()
+        ex.synchronize()
+        wall.append(time.perf_counter() - t0)
+        ev.append(e0.elapsed_ms(e1))
+        total += ev[-1]
+    return float(np.median(ev)), float(np.median(wall)), len(ev)
+
+
 def layer_bytes_algorithmic(specs):
     """weights once + f32 x + f32 y per projection."""
     w = sum(t.row_bytes(c) * r for _, t, r, c in specs)
@@ -71,47 +91,26 @@ def bench_layer_gemv(ex, steps, warmup, n_layers):
     for i in range(warmup):
         step(i)
     ex.synchronize()
-    e0, e1 = ex.event(), ex.event()
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        step(warmup + i)
-    e1.record()
-    ex.synchronize()
-    wall = time.perf_counter() - t0
-    ev_ms = e0.elapsed_ms(e1)
+    # every region below is `steps` launches (or steps) back to back, timed as a whole and repeated (timed_regions)
+    ev_ms, wall, n_regions = timed_regions(ex, lambda: [step(warmup + i) for i in range(steps)])
     # kernel-only region: the grouped GEMV launch alone, back to back
     ex.quantize_act_dev(xs, ncols, xqs)
-    ex.synchronize()
-    k0, k1 = ex.event(), ex.event()
-    k0.record()
-    for i in range(steps):
-        ex.qgemv_xq_grouped_dev(layers[(warmup + i) % n_layers], xqs, ys)
-    k1.record()
-    ex.synchronize()
-    kern_ms = k0.elapsed_ms(k1) / steps
+    kern_ms = timed_regions(ex, lambda: [ex.qgemv_xq_grouped_dev(layers[(warmup + i) % n_layers], xqs, ys) for i in range(steps)])[0] / steps
     # the step with the quantization folded into the GEMV's staging (what the decode loop launches)
-    f0, f1 = ex.event(), ex.event()
-    f0.record()
-    for i in range(steps):
-        ex.qgemv_grouped_dev(layers[(warmup + i) % n_layers], xs, ys)
-    f1.record()
-    ex.synchronize()
-    fused_ms = f0.elapsed_ms(f1) / steps
+    fused_ms = timed_regions(ex, lambda: [ex.qgemv_grouped_dev(layers[(warmup + i) % n_layers], xs, ys) for i in range(steps)])[0] / steps
     # the same launch on one layer over and over: its 130 MB stay in the 256 MB Infinity Cache
-    h0, h1 = ex.event(), ex.event()
     for i in range(8):
         ex.qgemv_xq_grouped_dev(layers[0], xqs, ys)
-    h0.record()
-    for i in range(steps):
-        ex.qgemv_xq_grouped_dev(layers[0], xqs, ys)
-    h1.record()
+    hot_ms = timed_regions(ex, lambda: [ex.qgemv_xq_grouped_dev(layers[0], xqs, ys) for i in range(steps)])[0] / steps
+    # what the benchmarked launch computes for layer 0, for the correctness gate (checked outside the timed regions)
+    ex.qgemv_xq_grouped_dev(layers[0], xqs, ys)
     ex.synchronize()
-    hot_ms = h0.elapsed_ms(h1) / steps
+    results = [y.download(np.float32) for y in ys]
     for ws in layers:
         for w in ws:
             w.free()
-    return dict(wbytes=wbytes, abytes=abytes, wall_s=wall, event_ms=ev_ms, kernel_ms=kern_ms, hot_ms=hot_ms, fused_ms=fused_ms)
+    return dict(wbytes=wbytes, abytes=abytes, wall_s=wall, event_ms=ev_ms, kernel_ms=kern_ms, hot_ms=hot_ms, fused_ms=fused_ms, regions=n_regions,
+                results=results)
 
 
 def bench_single_gemv(ex, reps=200):
@@ -130,14 +129,7 @@ def bench_single_gemv(ex, reps=200):
         y = ex.buffer(4 * rows)
         for i in range(16):
             ex.qgemv_dev(ws[i % 8], x, y)
-        ex.synchronize()
-        e0, e1 = ex.event(), ex.event()
-        e0.record()
-        for i in range(reps):
-            ex.qgemv_dev(ws[i % 8], x, y)
-        e1.record()
-        ex.synchronize()
-        ms = e0.elapsed_ms(e1) / reps
+        ms = timed_regions(ex, lambda: [ex.qgemv_dev(ws[i % 8], x, y) for i in range(reps)])[0] / reps
         wbytes = t.row_bytes(cols) * rows
         out.append({"shape": name, "us": round(ms * 1e3, 2), "weight_gbps": round(wbytes / ms / 1e6, 1),
                     "hbm_frac": round(wbytes / (ms * 1e-3) / HBM_PEAK, 4)})
@@ -166,14 +158,7 @@ def bench_batch8(ex, reps=100):
         for batch in (1, 8):
             for i in range(8):
                 ex.qgemv_dev(ws[i % 8], x, y, batch)
-            ex.synchronize()
-            e0, e1 = ex.event(), ex.event()
-            e0.record()
-            for i in range(reps):
-                ex.qgemv_dev(ws[i % 8], x, y, batch)
-            e1.record()
-            ex.synchronize()
-            res[batch] = e0.elapsed_ms(e1) / reps
+            res[batch] = timed_regions(ex, lambda: [ex.qgemv_dev(ws[i % 8], x, y, batch) for i in range(reps)])[0] / reps
         wbytes = t.row_bytes(cols) * rows
         out.append({"shape": name, "us_batch1": round(res[1] * 1e3, 2), "us_batch8": round(res[8] * 1e3, 2),
                     "weight_gbps_batch8": round(wbytes / res[8] / 1e6, 1), "rows_per_s_batch8": round(8 / (res[8] * 1e-3))})
@@ -204,14 +189,7 @@ def bench_layer_batch8(ex, n_layers=4, reps=100):
 
     for i in range(8):
         layer(layers[i % n_layers])
-    ex.synchronize()
-    e0, e1 = ex.event(), ex.event()
-    e0.record()
-    for i in range(reps):
-        layer(layers[i % n_layers])
-    e1.record()
-    ex.synchronize()
-    ms = e0.elapsed_ms(e1) / reps
+    ms = timed_regions(ex, lambda: [layer(layers[i % n_layers]) for i in range(reps)])[0] / reps
     for ws in layers:
         for w in ws:
             w.free()
@@ -263,14 +241,7 @@ def bench_prefill(ex, reps=20):
             y = ex.buffer(4 * M * rows)
             for _ in range(3):
                 ex.qgemm_dev(w, x, M, y)
-            ex.synchronize()
-            e0, e1 = ex.event(), ex.event()
-            e0.record()
-            for _ in range(reps):
-                ex.qgemm_dev(w, x, M, y)
-            e1.record()
-            ex.synchronize()
-            ms = e0.elapsed_ms(e1) / reps
+            ms = timed_regions(ex, lambda: [ex.qgemm_dev(w, x, M, y) for _ in range(reps)])[0] / reps
             flops = 2.0 * M * rows * cols
             out.append({"shape": name, "M": M, "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
                         "mfma_frac": round(flops / (ms * 1e-3) / MFMA_PEAK, 4)})
@@ -279,8 +250,10 @@ def bench_prefill(ex, reps=20):
     return out
 
 
-def cpu_baseline(reps):
-    """Reference CPU path for one layer: dequantize each tensor to dense f32, then x . W^T with sequential k-sums."""
+def cpu_baseline(reps, gpu_results=None):
+    """Reference CPU path for one layer: dequantize each tensor to dense f32, then x . W^T with sequential k-sums.
+    With `gpu_results` (what the benchmarked launch left for this layer) also the correctness gate of the timing: the
+    worst |y_gpu - y_f64| / (||w_row|| ||x||) over the seven projections, against the f64 products of the same blocks."""
     from oracle import oracle as orc
     from rustorch_amd import synth
     specs = synth.layer_tensor_specs(H, F)
@@ -288,6 +261,13 @@ def cpu_baseline(reps):
     tensors = [(t, r, c, synth.blocks(t, SEED, synth.layer_tid(0, slot), r, c), synth.normal(SEED, 1000 + i, c))
                for i, (slot, t, r, c) in enumerate(specs)]
     ncores = orc.num_threads()
+    worst = None
+    if gpu_results is not None:
+        worst = 0.0
+        for (t, r, c, raw, x), got in zip(tensors, gpu_results):
+            y64, wn = orc.qgemv_f64(t, raw, r, c, x)
+            yard = wn * np.linalg.norm(x.astype(np.float64))
+            worst = max(worst, float((np.abs(got.astype(np.float64) - np.asarray(y64).reshape(-1)) / yard).max()))
     best = {}
     for threads in (1, ncores):
         ts = []
@@ -298,7 +278,7 @@ def cpu_baseline(reps):
                 orc.matmul_xwt(x, W, threads)
             ts.append(time.perf_counter() - t0)
         best[threads] = min(ts)
-    return wbytes, best[1], best[ncores], ncores
+    return wbytes, best[1], best[ncores], ncores, worst
 
 
 def main():
@@ -348,6 +328,7 @@ def main():
         return
 
     g = bench_layer_gemv(ex, args.steps, args.warmup, args.layers)
+    # wall_s, event_ms: the median region of `steps` steps (timed_regions)
     ms_per_step = 1e3 * g["wall_s"] / args.steps
     value = g["wbytes"] / (g["wall_s"] / args.steps) / 1e9
     achieved = g["abytes"] / (g["kernel_ms"] * 1e-3) / 1e9
@@ -358,9 +339,11 @@ def main():
         "dtype": "q4_K/q6_K blocks x int16 block-scaled activations (int8 dot4, f32 accumulate)", "data": "synthetic",
         "config": {"workload": "C3: seven projections of one Llama-7B decoder layer, batch 1, q/k/o/gate/up Q4_K, v/down Q6_K",
                    "weight_bytes_per_step": g["wbytes"], "layers_rotated": args.layers, "hbm_frac_of_value": round(value * 1e9 / HBM_PEAK, 4),
-                   "event_ms_per_step": round(g["event_ms"] / args.steps, 5)},
+                   "event_ms_per_step": round(g["event_ms"] / args.steps, 5),
+                   "timing": "every figure is the median over %d repeats of a region of `steps` launches (repeated until 10 ms of device time are covered)" % g["regions"],
+                   "tolerance": "max |y - y_f64| <= 1e-3 * ||w_row|| * ||x|| per element", "parity_worst": None},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": GEMV_TRAFFIC_BYTES, "kernel": "qgemv_kernel",
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": GEMV_TRAFFIC_BYTES, "kernel": "qgemv_lean_kernel<512,1>",
                      "bytes_per_launch": g["abytes"], "avg_launch_ms": round(g["kernel_ms"], 5),
                      "cache_resident_launch_ms": round(g["hot_ms"], 5),
                      "fused_quantize_launch_ms": round(g["fused_ms"], 5)},
@@ -374,7 +357,8 @@ def main():
         out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen, args.decode_shape)
     ex.close()
     if not args.no_cpu:
-        wbytes, t1, tn, ncores = cpu_baseline(3)
+        wbytes, t1, tn, ncores, worst = cpu_baseline(3, g["results"])
+        out["config"]["parity_worst"] = worst       # of the benchmarked launch on one layer, in units of ||w_row|| ||x||; the bound is 1e-3
         out["cpu_baseline"] = {"value": round(wbytes / t1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": "one of the 32 layers (seven projections, batch 1): dequantize to dense f32, then naive x.W^T; best of 3",
                                "all_cores_value": round(wbytes / tn / 1e9, 4), "all_cores": ncores}

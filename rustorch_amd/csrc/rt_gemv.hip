@@ -18,8 +18,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
     gemv_dispatch<false, true>(P, wg - P.tile0, P.rows_per_tile, blockIdx.y, r2 != 0, reinterpret_cast<uint32_t *>(lds4), red);
 }
 
-// The same launch for problems that are all in the benchmark's four formats: the lean code path, two rows per step
-// (R = 2) or one.
+// The same launch for problems that are all in the benchmark's four formats: the lean code path, R rows per step (the
+// gate / up pair form always takes a pair).
 template <int THREADS, int R>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void qgemv_lean_kernel(GemvArgs a) {
     RT_DYN_LDS(uint4, lds4);
@@ -45,14 +45,9 @@ hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvLdsMax);
         if (e != hipSuccess) return e;
     }
-    if (pl.lean) {
-        if (pl.threads == 512) {
-            if (pl.r2) qgemv_lean_kernel<512, 2><<<grid, 512, lds, s>>>(a);
-            else qgemv_lean_kernel<512, 1><<<grid, 512, lds, s>>>(a);
-        } else {
-            if (pl.r2) qgemv_lean_kernel<1024, 2><<<grid, 1024, lds, s>>>(a);
-            else qgemv_lean_kernel<1024, 1><<<grid, 1024, lds, s>>>(a);
-        }
+    if (pl.lean) {      // the planner gives this path one row per step
+        if (pl.threads == 512) qgemv_lean_kernel<512, 1><<<grid, 512, lds, s>>>(a);
+        else qgemv_lean_kernel<1024, 1><<<grid, 1024, lds, s>>>(a);
     } else if (pl.threads == 512) qgemv_kernel<512><<<grid, 512, lds, s>>>(a, pl.r2);
     else qgemv_kernel<1024><<<grid, 1024, lds, s>>>(a, pl.r2);
     return hipGetLastError();

@@ -45,13 +45,22 @@ inline bool plan_qgemv(GemvArgs &a, int batch, GemvPlan &pl, const GemvPlanHints
     }
     if (total_bytes <= 0) return false;
     if (lds > kGemvLdsMax) return false;    // x of the longest row must fit the workgroup's LDS
+    bool lean = lds <= 64 * 1024;
+    for (int i = 0; i < a.n; i++) {
+        const GemvProb &p = a.p[i];
+        lean = lean && (p.res == nullptr || p.res == p.y) &&
+               (p.type == RT_GGML_Q4_K || p.type == RT_GGML_Q6_K || p.type == RT_GGML_Q8_0 || p.type == RT_GGML_Q4_0);
+    }
     // 16 resident waves per CU over 256 CUs, as one or two workgroups
     const int threads = hints.threads > 0 ? hints.threads : (total_bytes >= RT_GEMV_BIG_BYTES ? 512 : 1024);
     const int waves = threads / 64;
     int budget = hints.budget > 0 ? hints.budget : 256 * (1024 / threads) / batch;
     if (budget < a.n) budget = a.n;
-    // two rows per wave step once every wave has at least three steps of work, else one
-    const int r2 = hints.r2 >= 0 ? hints.r2 : (total_rows >= (size_t)3 * 2 * (size_t)budget * waves ? 1 : 0);
+    // General path: two rows per wave step once every wave has at least three steps of work, else one (two rows share one
+    // read of x from LDS).  Lean path: one row per step at every size -- measured on the layer workload and on single
+    // matrices of each format and row length, one row was as fast or faster (28.6 against 31.1 us for the layer): the finer
+    // steps even out the end of the launch, and its x reads are cheap next to the rest.
+    const int r2 = hints.r2 >= 0 ? hints.r2 : (lean ? 0 : (total_rows >= (size_t)3 * 2 * (size_t)budget * waves ? 1 : 0));
     int wgs = 0;
     for (int i = 0; i < a.n; i++) {
         const GemvProb &p = a.p[i];
@@ -64,12 +73,6 @@ inline bool plan_qgemv(GemvArgs &a, int batch, GemvPlan &pl, const GemvPlanHints
         a.p[i].tile0 = wgs;
         a.p[i].rows_per_tile = n;
         wgs += n;
-    }
-    bool lean = lds <= 64 * 1024;
-    for (int i = 0; i < a.n; i++) {
-        const GemvProb &p = a.p[i];
-        lean = lean && (p.res == nullptr || p.res == p.y) &&
-               (p.type == RT_GGML_Q4_K || p.type == RT_GGML_Q6_K || p.type == RT_GGML_Q8_0 || p.type == RT_GGML_Q4_0);
     }
     pl.threads = threads; pl.r2 = r2; pl.wgs = wgs; pl.lds = lds; pl.lean = lean;
     return true;
