@@ -117,6 +117,13 @@ RT_HIP_API int rt_hip_event_destroy(rt_hip_ctx *ctx, rt_hip_event *ev);
 RT_HIP_API int rt_hip_matmul_f32(rt_hip_ctx *ctx, const float *a, const float *b, float *c, size_t m, size_t n,
                                  size_t k);
 
+/* The same product on resident buffers (the GpuBuffer idiom, src/gpu/memory_ops/buffer.rs:22-48), enqueue only, and for a
+ * batch of products laid out one after the other: c_dev[i] = a_dev[i] . b_dev[i], i < batch -- what
+ * GpuLinearAlgebra::{gpu_matmul, gpu_batch_matmul, gpu_matvec} (src/gpu/matrix_ops.rs:562-595) and
+ * GpuBatchMatrixExecutor::batch_matmul (:308-343) ask of a device; a matrix-vector product is n = 1. */
+RT_HIP_API int rt_hip_matmul_f32_dev(rt_hip_ctx *ctx, const float *a_dev, const float *b_dev, float *c_dev, size_t m,
+                                     size_t n, size_t k, size_t batch);
+
 /* ---- per-tensor affine int8 matmul: QuantizedOps::qmatmul
  *      (src/quantization/operations.rs:195-260), which OptimizedOps::qmatmul
  *      (src/quantization/hardware/mod.rs:25-46) reaches on every device through

@@ -243,6 +243,17 @@ int rt_hip_matmul_f32(rt_hip_ctx *ctx, const float *a, const float *b, float *c,
     return RT_HIP_OK;
 }
 
+int rt_hip_matmul_f32_dev(rt_hip_ctx *ctx, const float *a_dev, const float *b_dev, float *c_dev, size_t m, size_t n, size_t k, size_t batch) {
+    if (!ctx) return fail(nullptr, RT_HIP_ERR_INVALID_ARG, "ctx is NULL");
+    RT_REQUIRE(ctx, a_dev && b_dev && c_dev, RT_HIP_ERR_INVALID_ARG, "matmul_f32_dev: NULL operand");
+    RT_REQUIRE(ctx, m > 0 && n > 0 && k > 0 && batch > 0, RT_HIP_ERR_SHAPE, "matmul_f32_dev: empty dimension (m=%zu n=%zu k=%zu batch=%zu)", m, n, k,
+               batch);
+    RT_REQUIRE(ctx, batch <= 65535 && (m + 31) / 32 <= 65535, RT_HIP_ERR_SHAPE, "matmul_f32_dev: batch=%zu or m=%zu beyond one grid", batch, m);
+    Guard g(ctx);
+    RT_TRY_HIP(ctx, rt::launch_matmul_f32(ctx->stream, a_dev, b_dev, c_dev, m, n, k, batch));
+    return RT_HIP_OK;
+}
+
 int rt_hip_qmatmul_i8(rt_hip_ctx *ctx, const int8_t *a, float scale_a, int zero_point_a, const int8_t *b, float scale_b,
                       int zero_point_b, size_t m, size_t n, size_t k, int8_t *out, float *out_scale, int *out_zero_point) {
     if (!ctx) return fail(nullptr, RT_HIP_ERR_INVALID_ARG, "ctx is NULL");

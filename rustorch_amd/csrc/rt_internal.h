@@ -132,7 +132,7 @@ hipError_t launch_argmax_advance(hipStream_t s, const float *v, size_t n, int *p
                                  int *out_tokens_dev, int *step_dev);
 hipError_t launch_embed_row(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,
                             const int *token_dev, int vocab, float *out);
-hipError_t launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *c, size_t m, size_t n, size_t k);
+hipError_t launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *c, size_t m, size_t n, size_t k, size_t batch = 1);
 hipError_t launch_qmatmul_i8(hipStream_t s, const int8_t *a, const int8_t *b, int8_t *out, size_t m, size_t n, size_t k, int za, int zb,
                              float scale);
 hipError_t launch_set_int(hipStream_t s, int *dst, int value);

@@ -622,11 +622,15 @@ __global__ void step_advance_kernel(int *pos_dev, int *token_dev, const int *pic
     *step_dev = step + 1;
 }
 
-// Dense row-major f32 C[m,n] = A[m,k] . B[k,n], 32x32 tiles through LDS, k summed in ascending order.
+// Dense row-major f32 C[m,n] = A[m,k] . B[k,n], 32x32 tiles through LDS, k summed in ascending order; grid.z walks a batch
+// of such products laid out one after the other (batch_matmul: src/gpu/matrix_ops.rs:308-343).
 __global__ __launch_bounds__(1024) void matmul_f32_kernel(const float *a, const float *b, float *c, size_t m, size_t n,
                                                           size_t k) {
     __shared__ float as[32][33];
     __shared__ float bs[32][33];
+    a += (size_t)blockIdx.z * m * k;
+    b += (size_t)blockIdx.z * k * n;
+    c += (size_t)blockIdx.z * m * n;
     size_t row = (size_t)blockIdx.y * 32 + threadIdx.y, col = (size_t)blockIdx.x * 32 + threadIdx.x;
     float acc = 0.f;
     for (size_t k0 = 0; k0 < k; k0 += 32) {
@@ -873,9 +877,10 @@ hipError_t launch_embed_rows(hipStream_t s, int type, const uint8_t *w, size_t r
     return hipGetLastError();
 }
 
-hipError_t launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *c, size_t m, size_t n, size_t k) {
-    if (m == 0 || n == 0) return hipSuccess;
-    dim3 grid((unsigned)((n + 31) / 32), (unsigned)((m + 31) / 32));
+hipError_t launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *c, size_t m, size_t n, size_t k, size_t batch) {
+    if (m == 0 || n == 0 || batch == 0) return hipSuccess;
+    if (batch > 65535 || (m + 31) / 32 > 65535) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((n + 31) / 32), (unsigned)((m + 31) / 32), (unsigned)batch);
     matmul_f32_kernel<<<grid, dim3(32, 32), 0, s>>>(a, b, c, m, n, k);
     return hipGetLastError();
 }

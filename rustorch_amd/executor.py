@@ -184,6 +184,13 @@ class HipKernelExecutor:
             raise InvalidParameters("matmul_f32: c must be a contiguous float32 array")
         _lib.check(self.lib.rt_hip_matmul_f32(self.ctx, _ptr(a), _ptr(b), _ptr(c), m, n, k), self.ctx)
 
+    def matmul_f32_dev(self, a: DeviceBuffer, b: DeviceBuffer, c: DeviceBuffer, m: int, n: int, k: int, batch: int = 1) -> None:
+        """c[i] = a[i] . b[i] for i < batch on resident buffers (gpu_matmul / gpu_batch_matmul / gpu_matvec with n = 1,
+        src/gpu/matrix_ops.rs:562-595); enqueues only."""
+        if a.nbytes < 4 * batch * m * k or b.nbytes < 4 * batch * k * n or c.nbytes < 4 * batch * m * n:
+            raise ShapeMismatch("matmul_f32_dev: buffers of %d, %d, %d bytes for batch=%d m=%d n=%d k=%d" % (a.nbytes, b.nbytes, c.nbytes, batch, m, n, k))
+        _lib.check(self.lib.rt_hip_matmul_f32_dev(self.ctx, a.ptr, b.ptr, c.ptr, m, n, k, batch), self.ctx)
+
     # -- per-tensor affine int8 tensors: QuantizedOps::qmatmul (src/quantization/operations.rs:195-260)
     def qmatmul_i8(self, a, scale_a: float, zero_point_a: int, b, scale_b: float, zero_point_b: int):
         """(int8 [m, n], output scale = scale_a * scale_b, output zero point = 0)."""

@@ -194,3 +194,34 @@ def test_dense_matmul_f32_kat(ex):
     I = np.eye(45, dtype=np.float32); out = np.zeros((70, 45), dtype=np.float32)
     ex.matmul_f32(A, I, out, 70, 45, 45)
     assert np.array_equal(out, A)
+
+
+def test_dense_matmul_on_resident_buffers_and_batches(ex):
+    """The dense product on device buffers that stay resident between calls (GpuBuffer, src/gpu/memory_ops/buffer.rs:22-48):
+    the reference's known answer (src/tensor/ops/matrix.rs:328-336), a batch of products in one launch against NumPy f64
+    (gpu_batch_matmul, src/gpu/matrix_ops.rs:562-595), the matrix-vector form (gpu_matvec: n = 1), and the same bits as the
+    host-slice entry point."""
+    from rustorch_amd import ShapeMismatch
+    a = ex.to_device(np.array([1, 2, 3, 4], dtype=np.float32)); b = ex.to_device(np.array([5, 6, 7, 8], dtype=np.float32))
+    c = ex.buffer(16)
+    ex.matmul_f32_dev(a, b, c, 2, 2, 2)
+    assert np.array_equal(c.download(np.float32), np.array([19, 22, 43, 50], dtype=np.float32))
+    rng = np.random.default_rng(1)
+    batch, m, n, k = 5, 70, 33, 45
+    A = rng.standard_normal((batch, m, k)).astype(np.float32); B = rng.standard_normal((batch, k, n)).astype(np.float32)
+    dA, dB, dC = ex.to_device(A), ex.to_device(B), ex.buffer(4 * batch * m * n)
+    ex.matmul_f32_dev(dA, dB, dC, m, n, k, batch)
+    got = dC.download(np.float32).reshape(batch, m, n)
+    assert np.allclose(got, A.astype(np.float64) @ B.astype(np.float64), rtol=1e-5, atol=1e-5)
+    one = np.zeros((m, n), dtype=np.float32)
+    ex.matmul_f32(A[3], B[3], one, m, n, k)
+    assert np.array_equal(got[3], one)
+    ex.matmul_f32_dev(dA, dB, dC, m, n, k, batch)               # the operands are still there: no upload between the calls
+    assert np.array_equal(dC.download(np.float32).reshape(batch, m, n), got)
+    v = ex.to_device(B[0][:, 0].copy()); y = ex.buffer(4 * m)
+    ex.matmul_f32_dev(dA, v, y, m, 1, k)
+    assert np.allclose(y.download(np.float32), A[0].astype(np.float64) @ B[0][:, 0].astype(np.float64), rtol=1e-5, atol=1e-5)
+    with pytest.raises(ShapeMismatch):
+        ex.matmul_f32_dev(dA, dB, c, m, n, k, batch)
+    for buf in (a, b, c, dA, dB, dC, v, y):
+        buf.free()
