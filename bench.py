@@ -113,6 +113,21 @@ def bench_layer_gemv(ex, steps, warmup, n_layers):
                 results=results)
 
 
+def bench_read_probe(ex, nbytes, steps):
+    """What a plain read kernel reaches on launches of the headline's size: `steps` launches over rotating 130 MB pieces of a
+    4 GB buffer (HBM) and over one piece again and again (Infinity Cache), in the GEMV's own access shape."""
+    n_sets = 32
+    buf = ex.buffer(n_sets * nbytes)
+    buf.zero()
+    for i in range(8):
+        ex.stream_read_dev(buf, i * nbytes, nbytes)
+    hbm_ms = timed_regions(ex, lambda: [ex.stream_read_dev(buf, ((i + 8) % n_sets) * nbytes, nbytes) for i in range(steps)])[0] / steps
+    hot_ms = timed_regions(ex, lambda: [ex.stream_read_dev(buf, 0, nbytes) for i in range(steps)])[0] / steps
+    buf.free()
+    return {"bytes_per_launch": nbytes, "hbm_launch_ms": round(hbm_ms, 5), "hbm_gbps": round(nbytes / hbm_ms / 1e6, 1),
+            "hbm_frac": round(nbytes / (hbm_ms * 1e-3) / HBM_PEAK, 4), "cache_resident_launch_ms": round(hot_ms, 5)}
+
+
 def bench_single_gemv(ex, reps=200):
     """The single-matrix decode configurations: Q8_0 4096x4096 and Q4_0 at the two FFN shapes (and one Q5_K and one unquantized F16 matrix), batch 1, x resident
     in HBM as f32 (quantized in the kernel's staging).  Eight synthetic copies of each matrix are rotated so that
@@ -348,6 +363,8 @@ def main():
                      "cache_resident_launch_ms": round(g["hot_ms"], 5),
                      "fused_quantize_launch_ms": round(g["fused_ms"], 5)},
     }
+    # the same number of bytes through a kernel that only reads: what the device grants a weight stream of this size
+    out["roofline"]["read_probe"] = bench_read_probe(ex, g["wbytes"] // 2048 * 2048, args.steps)
     out["single_gemv"] = bench_single_gemv(ex)
     if not args.no_prefill:
         out["prefill"] = bench_prefill(ex)

@@ -111,6 +111,11 @@ RT_HIP_API int rt_hip_event_record(rt_hip_ctx *ctx, rt_hip_event *ev);
 RT_HIP_API int rt_hip_event_elapsed_ms(rt_hip_ctx *ctx, rt_hip_event *start, rt_hip_event *stop, float *ms);
 RT_HIP_API int rt_hip_event_destroy(rt_hip_ctx *ctx, rt_hip_event *ev);
 
+/* Measurement aid (used by the bench; no reference counterpart): read the first nbytes / 2048 * 2048 bytes of a device
+ * buffer once, in the access shape of the decode GEMV's weight stream, and discard them.  The rate it reaches is the
+ * practical read ceiling of the device that the GEMV's achieved rate is reported beside. */
+RT_HIP_API int rt_hip_stream_read_dev(rt_hip_ctx *ctx, const void *dev, size_t nbytes);
+
 /* ---- dense f32 matmul: CudaKernelExecutor::matmul_f32(a,b,c,m,n,k)
  *      (src/gpu/cuda_kernels.rs:231-239; callers src/gpu/kernels.rs:316,
  *      src/gpu/matrix_ops.rs:378-386).  Row-major a[m,k] . b[k,n] -> c[m,n], host slices, blocking. */

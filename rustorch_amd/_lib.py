@@ -46,6 +46,7 @@ SIGNATURES = {
     "rt_hip_event_record": (C.c_int, [C.c_void_p, C.c_void_p]),
     "rt_hip_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, c_float_p]),
     "rt_hip_event_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "rt_hip_stream_read_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "rt_hip_matmul_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]),
     "rt_hip_matmul_f32_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t]),
     "rt_hip_qmatmul_i8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_void_p, C.c_float, C.c_int, C.c_size_t, C.c_size_t,

@@ -644,6 +644,16 @@ int rt_hip_add_dev(rt_hip_ctx *ctx, float *x, const float *y, size_t n) {
     return RT_HIP_OK;
 }
 
+int rt_hip_stream_read_dev(rt_hip_ctx *ctx, const void *dev, size_t nbytes) {
+    if (!ctx || !dev) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_stream_read_dev: NULL argument");
+    RT_REQUIRE(ctx, ((uintptr_t)dev & 15) == 0, RT_HIP_ERR_INVALID_ARG, "stream_read: the buffer must be 16-byte aligned");
+    Guard g(ctx);
+    int rc = ensure_scratch(ctx, 256);
+    if (rc) return rc;
+    RT_TRY_HIP(ctx, rt::launch_stream_read(ctx->stream, dev, nbytes, (unsigned *)ctx->scratch));
+    return RT_HIP_OK;
+}
+
 int rt_hip_argmax_dev(rt_hip_ctx *ctx, const float *v, size_t n, int *out_index_dev) {
     if (!ctx || !v || !out_index_dev) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_argmax_dev: NULL argument");
     RT_REQUIRE(ctx, n > 0 && n < ((size_t)1 << 31), RT_HIP_ERR_SHAPE, "argmax: n=%zu", n);

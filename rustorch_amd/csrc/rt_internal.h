@@ -126,6 +126,7 @@ hipError_t launch_attn_causal(hipStream_t s, const float *q, const uint16_t *kc,
 hipError_t launch_embed_rows(hipStream_t s, int type, const uint8_t *w, size_t row_bytes, size_t n_cols,
                              const int *tokens_dev, size_t n_tok, int vocab, float *out);
 hipError_t launch_add(hipStream_t s, float *x, const float *y, size_t n);
+hipError_t launch_stream_read(hipStream_t s, const void *p, size_t nbytes, unsigned *sink);
 hipError_t launch_argmax(hipStream_t s, const float *v, size_t n, int *out_dev);
 // the greedy pick and the end of the decode step (as launch_step_advance) in one launch
 hipError_t launch_argmax_advance(hipStream_t s, const float *v, size_t n, int *pick_dev, int *pos_dev, int *token_dev, const int *forced_dev,

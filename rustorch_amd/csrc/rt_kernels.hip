@@ -553,6 +553,30 @@ __global__ void add_kernel(float *x, const float *y, size_t n) {
     if (i < n) x[i] = x[i] + y[i];
 }
 
+// Measurement aid: reads n_chunks pieces of 2 KB once and throws them away, in the shape the decode GEMV reads its weights
+// (persistent waves take pieces round-robin, the next piece requested before the current one is used, lanes on
+// consecutive 16 bytes).  What this reaches is the practical ceiling a weight-streaming kernel is measured against.
+__global__ __launch_bounds__(512) void stream_read_kernel(const uint4 *__restrict__ p, size_t n_chunks, unsigned *sink) {
+    const int lane = (int)(threadIdx.x & 63);
+    size_t c = (size_t)blockIdx.x * 8 + (threadIdx.x >> 6);
+    const size_t n_gw = (size_t)gridDim.x * 8;
+    unsigned acc = 0;
+    uint4 a[2], b[2];
+    if (c < n_chunks) { a[0] = p[c * 128 + lane]; a[1] = p[c * 128 + 64 + lane]; }
+    while (c < n_chunks) {
+        size_t c2 = c + n_gw;
+        if (c2 < n_chunks) { b[0] = p[c2 * 128 + lane]; b[1] = p[c2 * 128 + 64 + lane]; }
+        acc += a[0].x ^ a[0].y ^ a[0].z ^ a[0].w ^ a[1].x ^ a[1].y ^ a[1].z ^ a[1].w;
+        c = c2;
+        if (c >= n_chunks) break;
+        c2 = c + n_gw;
+        if (c2 < n_chunks) { a[0] = p[c2 * 128 + lane]; a[1] = p[c2 * 128 + 64 + lane]; }
+        acc += b[0].x ^ b[0].y ^ b[0].z ^ b[0].w ^ b[1].x ^ b[1].y ^ b[1].z ^ b[1].w;
+        c = c2;
+    }
+    if (acc == 0x12345678u) sink[0] = acc;      // keeps the loads alive; practically never taken
+}
+
 // Greedy pick; ties resolve to the lowest index.
 // A thread's candidates are loaded eight at a time before they are compared (independent loads, one round trip per
 // eight).  With `adv` the same launch ends the decode step: record the pick, choose the next input token, advance.
@@ -851,6 +875,13 @@ hipError_t launch_attn_decode_split(hipStream_t s, const float *q, const float *
 hipError_t launch_add(hipStream_t s, float *x, const float *y, size_t n) {
     if (n == 0) return hipSuccess;
     add_kernel<<<dim3((unsigned)((n + 255) / 256)), 256, 0, s>>>(x, y, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_stream_read(hipStream_t s, const void *p, size_t nbytes, unsigned *sink) {
+    const size_t n_chunks = nbytes / 2048;       // whole pieces only: nothing past p + nbytes is touched
+    if (n_chunks == 0) return hipSuccess;
+    stream_read_kernel<<<512, 512, 0, s>>>(reinterpret_cast<const uint4 *>(p), n_chunks, sink);
     return hipGetLastError();
 }
 

@@ -184,6 +184,14 @@ class HipKernelExecutor:
             raise InvalidParameters("matmul_f32: c must be a contiguous float32 array")
         _lib.check(self.lib.rt_hip_matmul_f32(self.ctx, _ptr(a), _ptr(b), _ptr(c), m, n, k), self.ctx)
 
+    def stream_read_dev(self, buf: DeviceBuffer, offset: int = 0, nbytes: int | None = None) -> None:
+        """Measurement aid: one pass of plain reads over buf[offset : offset + nbytes] in the GEMV's access shape
+        (rt_hip_stream_read_dev); offset a multiple of 16."""
+        n = buf.nbytes - offset if nbytes is None else int(nbytes)
+        if offset < 0 or n < 0 or offset + n > buf.nbytes:
+            raise ShapeMismatch("stream_read_dev: bytes %d .. %d of a buffer of %d" % (offset, offset + n, buf.nbytes))
+        _lib.check(self.lib.rt_hip_stream_read_dev(self.ctx, C.c_void_p(buf.ptr.value + offset), n), self.ctx)
+
     def matmul_f32_dev(self, a: DeviceBuffer, b: DeviceBuffer, c: DeviceBuffer, m: int, n: int, k: int, batch: int = 1) -> None:
         """c[i] = a[i] . b[i] for i < batch on resident buffers (gpu_matmul / gpu_batch_matmul / gpu_matvec with n = 1,
         src/gpu/matrix_ops.rs:562-595); enqueues only."""

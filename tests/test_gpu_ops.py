@@ -131,3 +131,17 @@ def test_add_and_argmax(ex, orc):
     assert ex.argmax(v) == 123                               # ties: lowest index
     assert ex.argmax(np.full(5000, -3.0, np.float32)) == 0
     assert ex.argmax(np.array([1.0], np.float32)) == 0
+
+
+def test_stream_read_probe_stays_inside_its_buffer(ex):
+    """The bench's read probe touches whole 2 KB pieces of the range it is given and nothing else: ranges shorter than a
+    piece, ragged ends and an offset range are all accepted; a range past the buffer is refused on the host."""
+    from rustorch_amd import ShapeMismatch
+    buf = ex.buffer(3 * 2048 + 100)
+    buf.zero()
+    for off, n in ((0, None), (0, 100), (16, 2048), (2048, 2 * 2048 + 100), (0, 0)):
+        ex.stream_read_dev(buf, off, n)
+    ex.synchronize()
+    with pytest.raises(ShapeMismatch):
+        ex.stream_read_dev(buf, 2048, 3 * 2048)
+    buf.free()
