@@ -78,6 +78,20 @@ int dev_alloc(rt_hip_ctx *ctx, rt_hip_llama *m, void **p, size_t bytes) {
     return RT_HIP_OK;
 }
 
+// Gives a buffer of the model back before the model itself goes (a replaced tensor, an outgrown workspace).  The stream is
+// drained first: launches that still name the buffer may be in flight.
+void dev_release(rt_hip_ctx *ctx, rt_hip_llama *m, void *p) {
+    if (!p) return;
+    for (size_t i = 0; i < m->allocs.size(); i++) {
+        if (m->allocs[i] != p) continue;
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipFree(p);
+        m->allocs[i] = m->allocs.back();
+        m->allocs.pop_back();
+        return;
+    }
+}
+
 // Captured steps name device pointers: drop them whenever a tensor or buffer they name may change.
 void drop_step_graphs(rt_hip_llama *m) {
     for (auto &g : m->step_graphs) {
@@ -194,8 +208,14 @@ int ensure_prefill_buffers(rt_hip_ctx *ctx, rt_hip_llama *m, size_t n_tok) {
     const size_t H = (size_t)m->cfg.hidden, F = (size_t)m->cfg.ffn, cap = n_tok;
     int rc;
     float **hs[] = { &m->pf_x, &m->pf_x2, &m->pf_n, &m->pf_q, &m->pf_k, &m->pf_v, &m->pf_a };
+    // a longer prompt than any before: the smaller set goes back first (prompts of rising length would otherwise pile up sets)
+    for (float **p : hs) { dev_release(ctx, m, *p); *p = nullptr; }
+    dev_release(ctx, m, m->pf_g); dev_release(ctx, m, m->pf_u); dev_release(ctx, m, m->pf_tok); dev_release(ctx, m, m->pf_xp); dev_release(ctx, m, m->pf_inv);
+    m->pf_g = m->pf_u = nullptr; m->pf_tok = nullptr; m->pf_xp = nullptr; m->pf_inv = nullptr;
+    for (float *&p : m->pf_planes) { dev_release(ctx, m, p); p = nullptr; }
+    m->pf_cap = 0;
     for (float **p : hs)
-        if ((rc = dev_alloc(ctx, m, (void **)p, cap * H * sizeof(float)))) return rc;     // earlier, smaller ones are freed with the model
+        if ((rc = dev_alloc(ctx, m, (void **)p, cap * H * sizeof(float)))) return rc;
     if ((rc = dev_alloc(ctx, m, (void **)&m->pf_g, cap * F * sizeof(float)))) return rc;
     if ((rc = dev_alloc(ctx, m, (void **)&m->pf_u, cap * F * sizeof(float)))) return rc;
     if ((rc = dev_alloc(ctx, m, (void **)&m->pf_tok, cap * sizeof(int)))) return rc;
@@ -493,9 +513,9 @@ int rt_hip_llama_upload_tensor(rt_hip_ctx *ctx, rt_hip_llama *m, int slot, int l
     RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
     if (is_norm) {
         float *f = (float *)dev;
-        if (slot == RT_LLAMA_OUTPUT_NORM) m->out_norm = f;
-        else if (slot == RT_LLAMA_ATTN_NORM) m->attn_norm[(size_t)layer] = f;
-        else m->ffn_norm[(size_t)layer] = f;
+        float *&dst = slot == RT_LLAMA_OUTPUT_NORM ? m->out_norm : (slot == RT_LLAMA_ATTN_NORM ? m->attn_norm[(size_t)layer] : m->ffn_norm[(size_t)layer]);
+        dev_release(ctx, m, dst);        // a slot uploaded again: the old vector goes back
+        dst = f;
         return RT_HIP_OK;
     }
     rt_hip_llama::T t;
@@ -503,17 +523,22 @@ int rt_hip_llama_upload_tensor(rt_hip_ctx *ctx, rt_hip_llama *m, int slot, int l
     t.row_bytes = n_cols / rt::type_block_elems(ggml_type) * rt::type_block_bytes(ggml_type);
     t.dev = (uint8_t *)dev;
     size_t l = (size_t)(layer < 0 ? 0 : layer);
+    rt_hip_llama::T *dst = nullptr;
     switch (slot) {
-    case RT_LLAMA_TOK_EMBD: m->tok_embd = t; break;
-    case RT_LLAMA_OUTPUT: m->output = t; break;
-    case RT_LLAMA_ATTN_Q: m->wq[l] = t; break;
-    case RT_LLAMA_ATTN_K: m->wk[l] = t; break;
-    case RT_LLAMA_ATTN_V: m->wv[l] = t; break;
-    case RT_LLAMA_ATTN_OUT: m->wo[l] = t; break;
-    case RT_LLAMA_FFN_GATE: m->wgate[l] = t; break;
-    case RT_LLAMA_FFN_UP: m->wup[l] = t; break;
-    case RT_LLAMA_FFN_DOWN: m->wdown[l] = t; break;
+    case RT_LLAMA_TOK_EMBD: dst = &m->tok_embd; break;
+    case RT_LLAMA_OUTPUT: dst = &m->output; break;
+    case RT_LLAMA_ATTN_Q: dst = &m->wq[l]; break;
+    case RT_LLAMA_ATTN_K: dst = &m->wk[l]; break;
+    case RT_LLAMA_ATTN_V: dst = &m->wv[l]; break;
+    case RT_LLAMA_ATTN_OUT: dst = &m->wo[l]; break;
+    case RT_LLAMA_FFN_GATE: dst = &m->wgate[l]; break;
+    case RT_LLAMA_FFN_UP: dst = &m->wup[l]; break;
+    case RT_LLAMA_FFN_DOWN: dst = &m->wdown[l]; break;
     }
+    // a slot uploaded again: the old blocks and the fp16 copy the prefill may have made of them go back
+    dev_release(ctx, m, dst->dev);
+    dev_release(ctx, m, dst->f16);
+    *dst = t;
     return RT_HIP_OK;
 }
 
