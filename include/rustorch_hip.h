@@ -60,6 +60,7 @@ typedef enum {
     RT_GGML_Q5_0 = 6,
     RT_GGML_Q5_1 = 7,
     RT_GGML_Q8_0 = 8,
+    RT_GGML_Q8_1 = 9,
     RT_GGML_Q2_K = 10,
     RT_GGML_Q3_K = 11,
     RT_GGML_Q4_K = 12,

@@ -22,7 +22,7 @@
  * What the reference does NOT hold and this file therefore owns (parity with
  * the reference is unpinned for these; they are pinned by closed forms,
  * exhaustive packer round trips and an independent NumPy decoder in tests/):
- *   - the Q8_0 / Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q2_K / Q3_K / Q4_K / Q5_K / Q6_K block decoders.  The reference only fixes
+ *   - the Q8_0 / Q8_1 / Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q2_K / Q3_K / Q4_K / Q5_K / Q6_K block decoders.  The reference only fixes
  *     type ids and block byte sizes (example-cli/src/model/formats/gguf.rs:78-144)
  *     and decodes every quantized type with a placeholder
  *     (tensor_loader.rs:125-141,213-218).  The layouts below are the public
@@ -43,7 +43,7 @@
 
 #define ORC_API __attribute__((visibility("default")))
 
-enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q4_1 = 3, ORC_Q5_0 = 6, ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q2_K = 10, ORC_Q3_K = 11, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };
+enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q4_1 = 3, ORC_Q5_0 = 6, ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q8_1 = 9, ORC_Q2_K = 10, ORC_Q3_K = 11, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14 };
 
 /* ------------------------------------------------------------------ fp16 */
 
@@ -104,7 +104,7 @@ static inline uint16_t rd_u16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1]
 
 ORC_API int orc_block_elems(int type) {
     switch (type) {
-    case ORC_Q8_0: case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: return 32;
+    case ORC_Q8_0: case ORC_Q8_1: case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: return 32;
     case ORC_Q2_K: case ORC_Q3_K: case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 256;
     case ORC_F32: case ORC_F16: return 1;
     default: return 0;
@@ -115,6 +115,7 @@ ORC_API int orc_block_elems(int type) {
 ORC_API int orc_block_bytes(int type) {
     switch (type) {
     case ORC_Q8_0: return 34;
+    case ORC_Q8_1: return 36;
     case ORC_Q4_0: return 18;
     case ORC_Q4_1: return 20;
     case ORC_Q5_0: return 22;
@@ -136,6 +137,14 @@ ORC_API int orc_block_bytes(int type) {
 static void deq_q8_0(const uint8_t *b, float *y) {
     float d = orc_h2f(rd_u16(b));
     const int8_t *qs = (const int8_t *)(b + 2);
+    for (int i = 0; i < 32; i++) y[i] = d * (float)qs[i];
+}
+
+/* Q8_1: { f16 d; f16 s; i8 qs[32] }   y[i] = d * qs[i]; s = d * sum(qs) is carried for integer dot products and is not
+ * part of any value (type id 9 of example-cli/src/model/formats/gguf.rs:89, 36 bytes at :136) */
+static void deq_q8_1(const uint8_t *b, float *y) {
+    float d = orc_h2f(rd_u16(b));
+    const int8_t *qs = (const int8_t *)(b + 4);
     for (int i = 0; i < 32; i++) y[i] = d * (float)qs[i];
 }
 
@@ -317,6 +326,7 @@ static void deq_q6_k(const uint8_t *b, float *y) {
 static void deq_row(int type, const uint8_t *row, size_t n_cols, float *y) {
     switch (type) {
     case ORC_Q8_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q8_0(row + 34 * b, y + 32 * b); break;
+    case ORC_Q8_1: for (size_t b = 0; b < n_cols / 32; b++) deq_q8_1(row + 36 * b, y + 32 * b); break;
     case ORC_Q4_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q4_0(row + 18 * b, y + 32 * b); break;
     case ORC_Q4_1: for (size_t b = 0; b < n_cols / 32; b++) deq_q4_1(row + 20 * b, y + 32 * b); break;
     case ORC_Q5_0: for (size_t b = 0; b < n_cols / 32; b++) deq_q5_0(row + 22 * b, y + 32 * b); break;

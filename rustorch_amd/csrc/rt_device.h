@@ -77,6 +77,11 @@ __device__ inline float deq_elem(int type, const uint8_t *row, size_t col) {
         float d = h2f(ld2u(b));
         return d * (float)(int)(int8_t)b[2 + (col & 31)];
     }
+    case RT_GGML_Q8_1: {       // { f16 d; f16 s; i8 qs[32] }: s = d * sum(qs) serves integer dot products and is not part of a value
+        const uint8_t *b = row + 36 * (col >> 5);
+        float d = h2f(ld2u(b));
+        return d * (float)(int)(int8_t)b[4 + (col & 31)];
+    }
     case RT_GGML_Q4_0: {
         const uint8_t *b = row + 18 * (col >> 5);
         float d = h2f(ld2u(b));

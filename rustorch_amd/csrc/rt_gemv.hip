@@ -13,8 +13,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
     RT_DYN_LDS(uint4, lds4);
     __shared__ float red[THREADS / 64];
     const int wg = blockIdx.x;
-    RT_GEMV_PICK_PROBLEM(a, wg, pi);
-    const GemvProb &P = a.p[pi];
+    RT_GEMV_PICK_PROBLEM(a, wg, P);
     gemv_dispatch<false, true>(P, wg - P.tile0, P.rows_per_tile, blockIdx.y, r2 != 0, reinterpret_cast<uint32_t *>(lds4), red);
 }
 
@@ -25,8 +24,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
     RT_DYN_LDS(uint4, lds4);
     __shared__ float red[THREADS / 64];
     const int wg = blockIdx.x;
-    RT_GEMV_PICK_PROBLEM(a, wg, pi);
-    const GemvProb &P = a.p[pi];
+    RT_GEMV_PICK_PROBLEM(a, wg, P);
     lean_dispatch<R>(P, wg - P.tile0, P.rows_per_tile, blockIdx.y, reinterpret_cast<uint32_t *>(lds4), red);
 }
 

@@ -67,7 +67,7 @@ __device__ __forceinline__ void stage_store(int type, int K, int U, uint32_t *ld
             int u = 2 * (i16 >> 3) + (i16 & 1), r = (i16 >> 1) & 3;
             S[2 * U + 4 * u + r] = bsum16;
         }
-    } else if (type == RT_GGML_Q8_0) {
+    } else if (type == RT_GGML_Q8_0 || type == RT_GGML_Q8_1) {
         if ((e & 31) == 0) S[e >> 5] = s;
     } else {
         if ((e & 31) == 0) {
@@ -154,6 +154,9 @@ template <> struct XRegs<RT_GGML_Q6_K> { uint4 h[4], l[4]; float4 xs, xb; };
 template <> struct WRegs<RT_GGML_Q8_0> { uint4 a, b; uint32_t d; };
 template <> struct XRegs<RT_GGML_Q8_0> { uint4 h[2], l[2]; float s; };
 template <> struct WRegs<RT_GGML_Q4_0> { uint4 a; uint32_t d; };
+// Q8_1: a Q8_0 block with a second half word (d * sum of the quants) between the scale and the quants: same registers, same x slice
+template <> struct WRegs<RT_GGML_Q8_1> : WRegs<RT_GGML_Q8_0> {};
+template <> struct XRegs<RT_GGML_Q8_1> : XRegs<RT_GGML_Q8_0> {};
 template <> struct XRegs<RT_GGML_Q4_0> { uint4 h[2], l[2]; float2 sv; };
 // Q3_K: a unit is, as for Q6_K, 16 byte positions x 4 runs of one half of a super-block (element 128 n + 32 j + 16 c + i):
 // the same x slice; 16 bytes of 2-bit fields, 16 bytes of third bits, the 12 scale bytes, d
@@ -240,6 +243,12 @@ __device__ __forceinline__ void load_w(WRegs<RT_GGML_Q8_0> &w, WRow row, int u) 
     w.a = bld16(row, off + 2u);
     w.b = bld16(row, off + 18u);
 }
+__device__ __forceinline__ void load_w(WRegs<RT_GGML_Q8_1> &w, WRow row, int u) {
+    uint32_t off = (uint32_t)u * 36u;
+    w.d = bld2(row, off);
+    w.a = bld16(row, off + 4u);
+    w.b = bld16(row, off + 20u);
+}
 __device__ __forceinline__ void load_w(WRegs<RT_GGML_Q4_0> &w, WRow row, int u) {
     uint32_t off = (uint32_t)u * 18u;
     w.d = bld2(row, off);
@@ -296,6 +305,9 @@ __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q8_0> &x, const uint32_t *l
     const uint4 *XL = XH + K / 16;
     x.h[0] = XH[u]; x.h[1] = XH[U + u]; x.l[0] = XL[u]; x.l[1] = XL[U + u];
     x.s = reinterpret_cast<const float *>(lds + K / 2)[u];
+}
+__device__ __forceinline__ void load_x(XRegs<RT_GGML_Q8_1> &x, const uint32_t *lds, int u, int U, int K) {
+    load_x(static_cast<XRegs<RT_GGML_Q8_0> &>(x), lds, u, U, K);
 }
 __device__ __forceinline__ void load_x(XRegs<RT_GGML_Q4_0> &x, const uint32_t *lds, int u, int U, int K) {
     const uint4 *XH = reinterpret_cast<const uint4 *>(lds);
@@ -509,6 +521,9 @@ __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q8_0> &w, const XR
     return h2f(w.d) * (x.s * __builtin_fmaf((float)dh, 128.f, (float)dl));
 }
 
+__device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q8_1> &w, const XRegs<RT_GGML_Q8_1> &x, int u) {
+    return dot_unit(static_cast<const WRegs<RT_GGML_Q8_0> &>(w), static_cast<const XRegs<RT_GGML_Q8_0> &>(x), u);
+}
 __device__ __forceinline__ float dot_unit(const WRegs<RT_GGML_Q4_0> &w, const XRegs<RT_GGML_Q4_0> &x, int) {
     const uint32_t q[4] = RT_W4(w.a);
     const uint32_t hlo[4] = RT_W4(x.h[0]), hhi[4] = RT_W4(x.h[1]), llo[4] = RT_W4(x.l[0]), lhi[4] = RT_W4(x.l[1]);
@@ -720,6 +735,7 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
         case RT_GGML_Q4_K: gemv_problem<RT_GGML_Q4_K, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q6_K: gemv_problem<RT_GGML_Q6_K, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q8_1: gemv_problem<RT_GGML_Q8_1, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_1: gemv_problem<RT_GGML_Q4_1, 2, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q5_0: gemv_problem<RT_GGML_Q5_0, 2, COH>(P, wg, n_wg, m, lds, red); break;
@@ -732,6 +748,7 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
         case RT_GGML_Q4_K: gemv_problem<RT_GGML_Q4_K, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q6_K: gemv_problem<RT_GGML_Q6_K, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q8_0: gemv_problem<RT_GGML_Q8_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
+        case RT_GGML_Q8_1: gemv_problem<RT_GGML_Q8_1, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_0: gemv_problem<RT_GGML_Q4_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q4_1: gemv_problem<RT_GGML_Q4_1, 1, COH>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q5_0: gemv_problem<RT_GGML_Q5_0, 1, COH>(P, wg, n_wg, m, lds, red); break;
@@ -742,11 +759,13 @@ __device__ __forceinline__ void gemv_dispatch(const GemvProb &P, int wg, int n_w
     }
 }
 
-// The problem a workgroup of the grouped launch belongs to.  A macro, so that the kernel indexes its argument structure
-// where it lies (handing the structure to a function by reference makes the compiler copy all of it to private memory).
-#define RT_GEMV_PICK_PROBLEM(args, wg, pi)                   \
-    int pi = 0;                                              \
-    _Pragma("unroll") for (int i_ = 1; i_ < rt::kMaxGemvProbs; i_++) \
-        if (i_ < (args).n && (wg) >= (args).p[i_].tile0) pi = i_
+// The problem a workgroup of the grouped launch belongs to, as a local copy chosen by a chain of selects over the argument
+// structure's fixed slots.  (Indexing the by-value argument with a run-time index, or handing it to a function by
+// reference, makes the compiler copy all of it to private memory as soon as the kernel grows past some size; a private
+// frame in this kernel slows every launch of it.)
+#define RT_GEMV_PICK_PROBLEM(args, wg, P)                             \
+    rt::GemvProb P = (args).p[0];                                     \
+    _Pragma("unroll") for (int i_ = 1; i_ < rt::kMaxGemvProbs; i_++)  \
+        if (i_ < (args).n && (wg) >= (args).p[i_].tile0) P = (args).p[i_]
 
 }  // namespace rt

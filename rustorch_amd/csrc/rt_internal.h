@@ -194,6 +194,7 @@ inline size_t type_block_bytes(int t) {
     case RT_GGML_Q5_0: return 22;
     case RT_GGML_Q5_1: return 24;
     case RT_GGML_Q8_0: return 34;
+    case RT_GGML_Q8_1: return 36;
     case RT_GGML_Q2_K: return 84;      // 16 scale bytes + 64 + two f16: the public ggml block (the reference's size table lists 82)
     case RT_GGML_Q3_K: return 110;
     case RT_GGML_Q4_K: return 144;
@@ -205,7 +206,7 @@ inline size_t type_block_bytes(int t) {
 inline size_t type_block_elems(int t) {
     switch (t) {
     case RT_GGML_F32: case RT_GGML_F16: return 1;
-    case RT_GGML_Q4_0: case RT_GGML_Q4_1: case RT_GGML_Q5_0: case RT_GGML_Q5_1: case RT_GGML_Q8_0: return 32;
+    case RT_GGML_Q4_0: case RT_GGML_Q4_1: case RT_GGML_Q5_0: case RT_GGML_Q5_1: case RT_GGML_Q8_0: case RT_GGML_Q8_1: return 32;
     case RT_GGML_Q2_K: case RT_GGML_Q3_K: case RT_GGML_Q4_K: case RT_GGML_Q5_K: case RT_GGML_Q6_K: return 256;
     default: return 0;
     }

@@ -192,7 +192,7 @@ int enqueue_step(rt_hip_ctx *ctx, rt_hip_llama *m, bool want_logits) {
 }
 
 bool gemv_type_ok(int t) {
-    return t == RT_GGML_F32 || t == RT_GGML_F16 || t == RT_GGML_Q8_0 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_1 || t == RT_GGML_Q5_0 ||
+    return t == RT_GGML_F32 || t == RT_GGML_F16 || t == RT_GGML_Q8_0 || t == RT_GGML_Q8_1 || t == RT_GGML_Q4_0 || t == RT_GGML_Q4_1 || t == RT_GGML_Q5_0 ||
            t == RT_GGML_Q5_1 || t == RT_GGML_Q2_K || t == RT_GGML_Q3_K || t == RT_GGML_Q4_K || t == RT_GGML_Q5_K || t == RT_GGML_Q6_K;
 }
 

@@ -5,7 +5,7 @@
 // with mix = the splitmix64 finaliser applied to (z + 0x9E3779B97F4A7C15).
 // Field maps (u24(v) = (v & 0xFFFFFF) / 2^24 in double; a scale is
 // f16_rne((float)(lo + (hi - lo) * u))):
-//   Q8_0 : w0 -> d from u24(r);  w1..w8 -> 32 x u16 v, qs = ((v * 255) >> 16) - 127
+//   Q8_0 : w0 -> d from u24(r);  w1..w8 -> 32 x u16 v, qs = ((v * 255) >> 16) - 127        Q8_1 : the same draw, plus s = f16(d * sum qs)
 //   Q4_0 : w0 -> d;  w1,w2 -> the 16 qs bytes verbatim
 //   Q4_1 : w0 -> d from u24(r), m = -8 d' with d' from u24(r >> 32);  w1,w2 -> qs
 //   Q5_0 : w0 -> d, qh = bits 32..63 of r;  w1,w2 -> qs        Q5_1 : w0 -> d, m = -16 d';  w1,w2 -> qs;  w3 -> qh (low 32 bits)
@@ -58,6 +58,25 @@ inline uint16_t f32_to_f16(float f) {
     return (uint16_t)(sign | h);
 }
 
+// binary16 -> binary32 (exact).
+inline float f16_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu;
+    uint32_t x;
+    if (exp == 0) {
+        if (man == 0) x = sign;
+        else {                                     // subnormal: renormalise
+            int e = -1;
+            uint32_t m = man;
+            do { e++; m <<= 1; } while ((m & 0x400u) == 0);
+            x = sign | ((uint32_t)(112 - e) << 23) | ((m & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) x = sign | 0x7F800000u | (man << 13);
+    else x = sign | ((exp + 112u) << 23) | (man << 13);
+    float f;
+    std::memcpy(&f, &x, 4);
+    return f;
+}
+
 inline uint16_t scale_f16(double lo, double hi, double u) { return f32_to_f16((float)(lo + (hi - lo) * u)); }
 
 inline void put16(uint8_t *p, uint16_t v) { p[0] = (uint8_t)v; p[1] = (uint8_t)(v >> 8); }
@@ -84,6 +103,22 @@ void gen_block(int type, uint64_t key, uint64_t b, double lo, double hi, uint8_t
                 o[2 + 4 * w + i] = (uint8_t)(int8_t)((int)((v * 255u) >> 16) - 127);
             }
         }
+        break;
+    }
+    case RT_GGML_Q8_1: {       // the Q8_0 draw with the format's second field, d * sum of the quants (rounded to fp16), filled in
+        const uint16_t dh = scale_f16(lo, hi, u24(mix(base)));
+        put16(o, dh);
+        int sum = 0;
+        for (int w = 0; w < 8; w++) {
+            uint64_t r = mix(base + 1 + w);
+            for (int i = 0; i < 4; i++) {
+                uint32_t v = (uint32_t)((r >> (16 * i)) & 0xFFFFu);
+                const int q = (int)((v * 255u) >> 16) - 127;
+                o[4 + 4 * w + i] = (uint8_t)(int8_t)q;
+                sum += q;
+            }
+        }
+        put16(o + 2, f32_to_f16(f16_to_f32(dh) * (float)sum));
         break;
     }
     case RT_GGML_Q4_0: {

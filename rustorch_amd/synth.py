@@ -16,6 +16,7 @@ from .gguf import GGMLType
 
 D_RANGE = {
     GGMLType.Q8_0: (1e-4, 2e-3),
+    GGMLType.Q8_1: (1e-4, 2e-3),
     GGMLType.Q4_0: (1e-3, 2e-2),
     GGMLType.Q4_1: (1e-3, 2e-2),      # offsets m are drawn from -8 * this range (Q5_1: -16 *)
     GGMLType.Q5_0: (5e-4, 1e-2),

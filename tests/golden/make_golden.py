@@ -43,7 +43,7 @@ def main() -> None:
         payload = [i for i in range(bb) if all(not (o <= i < o + 2) for o in d_off)]
         raw[4, payload] = 0x00
         raw[5, payload] = 0xFF
-        if t == 8:
+        if t in (8, 9):
             raw[5, payload] = 0x81  # -127: keep away from the unused -128 only in this block
         vals = np.stack([fn(b) for b in raw])
         out["raw_%d" % t] = raw

@@ -25,6 +25,13 @@ def decode_q8_0(blk: np.ndarray) -> np.ndarray:
     return (d * q).astype(F32)
 
 
+def decode_q8_1(blk: np.ndarray) -> np.ndarray:
+    """{ f16 d; f16 s; i8 qs[32] }: the values are d * qs; the second half word (d * sum of qs) is not part of them."""
+    d = _f16(blk, 0)
+    q = blk[4:36].view(np.int8)
+    return np.array([F32(d * F32(int(v))) for v in q], dtype=np.float32)
+
+
 def decode_q4_0(blk: np.ndarray) -> np.ndarray:
     d = _f16(blk, 0)
     out = np.empty(32, dtype=F32)
@@ -159,7 +166,7 @@ def decode_q6_k(blk: np.ndarray) -> np.ndarray:
 
 DECODERS = {8: (34, 32, decode_q8_0), 2: (18, 32, decode_q4_0), 12: (144, 256, decode_q4_k), 14: (210, 256, decode_q6_k),
             13: (176, 256, decode_q5_k), 3: (20, 32, decode_q4_1), 6: (22, 32, decode_q5_0), 7: (24, 32, decode_q5_1),
-            11: (110, 256, decode_q3_k), 10: (84, 256, decode_q2_k)}
+            11: (110, 256, decode_q3_k), 10: (84, 256, decode_q2_k), 9: (36, 32, decode_q8_1)}
 
 
 def decode(ggml_type: int, raw: np.ndarray) -> np.ndarray:
@@ -178,6 +185,15 @@ def encode_q8_0(d, q) -> np.ndarray:
     blk = np.zeros(34, dtype=np.uint8)
     _put_f16(blk, 0, d)
     blk[2:] = np.asarray(q, dtype=np.int8).view(np.uint8)
+    return blk
+
+
+def encode_q8_1(d, q, s=None) -> np.ndarray:
+    blk = np.zeros(36, dtype=np.uint8)
+    _put_f16(blk, 0, d)
+    q = np.asarray(q, dtype=np.int8)
+    _put_f16(blk, 2, np.float32(np.float16(d)) * np.float32(int(q.astype(np.int64).sum())) if s is None else s)
+    blk[4:] = q.view(np.uint8)
     return blk
 
 

@@ -60,7 +60,7 @@ def test_static_archive_holds_the_same_entry_points(lib):
 def test_type_table_matches_reference_type_size(lib):
     # example-cli/src/model/formats/gguf.rs:78-99,125-144
     from rustorch_amd import GGMLType
-    for t, size, elems in ((0, 4, 1), (1, 2, 1), (2, 18, 32), (3, 20, 32), (6, 22, 32), (7, 24, 32), (8, 34, 32), (10, 84, 256), (11, 110, 256), (12, 144, 256), (13, 176, 256),
+    for t, size, elems in ((0, 4, 1), (1, 2, 1), (2, 18, 32), (3, 20, 32), (6, 22, 32), (7, 24, 32), (8, 34, 32), (9, 36, 32), (10, 84, 256), (11, 110, 256), (12, 144, 256), (13, 176, 256),
                            (14, 210, 256)):
         assert lib.rt_hip_type_block_bytes(t) == size and lib.rt_hip_type_block_elems(t) == elems
         assert GGMLType(t).type_size() == size and GGMLType(t).block_elems() == elems

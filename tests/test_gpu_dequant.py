@@ -12,7 +12,7 @@ def bits(a):
     return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
 
 
-@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 10, 11, 12, 13, 14])
+@pytest.mark.parametrize("t", [8, 9, 2, 3, 6, 7, 10, 11, 12, 13, 14])
 def test_golden_vectors_bit_exact(ex, t):
     g = np.load(GOLDEN)
     raw, val = g["raw_%d" % t], g["val_%d" % t]
@@ -23,7 +23,7 @@ def test_golden_vectors_bit_exact(ex, t):
 
 
 @pytest.mark.parametrize("t,rows,cols", [(8, 64, 4096), (2, 33, 11008), (12, 48, 4096), (12, 17, 11008), (14, 40, 4096), (14, 9, 11008), (13, 48, 4096), (13, 5, 11008),
-                                         (3, 33, 4096), (6, 33, 11008), (7, 20, 4096), (1, 9, 4096), (0, 5, 1024), (11, 40, 4096), (11, 7, 11008), (10, 40, 4096), (10, 7, 11008)])
+                                         (9, 33, 4096), (9, 7, 11008), (3, 33, 4096), (6, 33, 11008), (7, 20, 4096), (1, 9, 4096), (0, 5, 1024), (11, 40, 4096), (11, 7, 11008), (10, 40, 4096), (10, 7, 11008)])
 def test_synthetic_tensors_bit_exact(ex, orc, t, rows, cols):
     from rustorch_amd import synth
     print("dequant synthetic", t, rows, cols, flush=True)

@@ -65,7 +65,7 @@ def test_gemv_config_shapes_batch1_and_8(ex, orc, name):
     check(yo, y64[:2], wn, x[:2], name + " oracle f32 vs f64")
 
 
-@pytest.mark.parametrize("t", [8, 2, 3, 6, 7, 10, 11, 12, 13, 14, 1, 0])
+@pytest.mark.parametrize("t", [8, 9, 2, 3, 6, 7, 10, 11, 12, 13, 14, 1, 0])
 def test_gemv_edge_inputs(ex, orc, t):
     from rustorch_amd import synth
     be = 256 if t in (10, 11, 12, 13, 14) else 32                  # unquantized rows: any multiple of 32 columns

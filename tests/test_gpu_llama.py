@@ -301,7 +301,7 @@ def test_short_prompts_take_the_batched_pass(ex, orc):
         assert d <= (0.25 if n < 16 else 1.0) and r <= 1.0 and r2 <= 1.0
 
 
-@pytest.mark.parametrize("fmt", ["Q5_K", "Q8_0", "Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q2_K", "Q3_K", "F16", "F32"])
+@pytest.mark.parametrize("fmt", ["Q5_K", "Q8_0", "Q8_1", "Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q2_K", "Q3_K", "F16", "F32"])
 def test_model_in_a_format_without_matrix_core_path(ex, orc, fmt):
     """All seven matrices of every layer in one format that the dense contraction does not serve.  Decode: the GEMV
     kernels (Q5_K: one row per step, gate and up as two problems of one launch followed by the separate SwiGLU).

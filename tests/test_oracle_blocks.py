@@ -9,7 +9,7 @@ import pytest
 import np_blocks as nb
 
 GOLDEN = Path(__file__).resolve().parent / "golden" / "blocks_golden.npz"
-TYPES = [8, 2, 3, 6, 7, 10, 11, 12, 13, 14]
+TYPES = [8, 9, 2, 3, 6, 7, 10, 11, 12, 13, 14]
 
 
 def bits(a):
@@ -48,8 +48,8 @@ def test_f32_to_fp16_rne(orc):
 
 def test_block_geometry_matches_reference_type_size(orc):
     # example-cli/src/model/formats/gguf.rs:125-144
-    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 3, 6, 7, 8, 10, 11, 12, 13, 14)] == [4, 2, 18, 20, 22, 24, 34, 84, 110, 144, 176, 210]
-    assert [orc.load().orc_block_elems(t) for t in (2, 3, 6, 7, 8, 10, 11, 12, 13, 14)] == [32, 32, 32, 32, 32, 256, 256, 256, 256, 256]
+    assert [orc.load().orc_block_bytes(t) for t in (0, 1, 2, 3, 6, 7, 8, 9, 10, 11, 12, 13, 14)] == [4, 2, 18, 20, 22, 24, 34, 36, 84, 110, 144, 176, 210]
+    assert [orc.load().orc_block_elems(t) for t in (2, 3, 6, 7, 8, 9, 10, 11, 12, 13, 14)] == [32, 32, 32, 32, 32, 32, 256, 256, 256, 256, 256]
     assert orc.load().orc_row_bytes(12, 4096) == 2304 and orc.load().orc_row_bytes(14, 11008) == 9030
     assert orc.load().orc_row_bytes(12, 100) == 0
 
@@ -66,6 +66,29 @@ def test_q8_0_closed_forms(orc):
         raw = np.concatenate([nb.encode_q8_0(d, allq[i:i + 32]) for i in range(0, 256, 32)])
         y = orc.dequant(8, raw, 1, 256)[0]
         assert np.array_equal(bits(y), bits(np.float16(d).astype(np.float32) * allq.astype(np.float32)))
+
+
+def test_q8_1_closed_forms(orc):
+    """Q8_1 is Q8_0 with a second half word between scale and quants: y = d * q whatever that word holds, the quants sit at
+    byte 4, and a block is 36 bytes (example-cli/src/model/formats/gguf.rs:89,136)."""
+    q = np.arange(-16, 16)
+    for s in (None, 0.0, 123.0, np.float16(np.nan)):            # the carried sum is not read by the decode
+        y = orc.dequant(9, nb.encode_q8_1(1.0, q, s), 1, 32)[0]
+        assert np.array_equal(y, q.astype(np.float32))
+    y = orc.dequant(9, nb.encode_q8_1(2.0 ** -9, q), 1, 32)[0]
+    assert np.array_equal(y, q.astype(np.float32) * np.float32(2.0 ** -9))
+    for v in (-128, -127, -1, 0, 1, 127):
+        for pos in (0, 1, 15, 16, 31):
+            qq = np.zeros(32, np.int8); qq[pos] = v
+            want = np.zeros(32, np.float32); want[pos] = np.float32(np.float16(0.375)) * np.float32(v)
+            assert np.array_equal(orc.dequant(9, nb.encode_q8_1(0.375, qq), 1, 32)[0], want)
+    # the same values as the Q8_0 block with the same scale and quants
+    rng = np.random.default_rng(5)
+    qq = rng.integers(-127, 128, 32).astype(np.int8)
+    assert np.array_equal(orc.dequant(9, nb.encode_q8_1(0.0123, qq), 1, 32), orc.dequant(8, nb.encode_q8_0(0.0123, qq), 1, 32))
+    # two blocks in a row: the second starts at byte 36
+    two = np.concatenate([nb.encode_q8_1(1.0, q), nb.encode_q8_1(2.0, q)])
+    assert np.array_equal(orc.dequant(9, two, 1, 64)[0], np.concatenate([q, 2 * q]).astype(np.float32))
 
 
 def test_reference_affine_dequant_kat(orc):
@@ -278,7 +301,7 @@ def test_golden_vectors(orc, t):
 @pytest.mark.parametrize("t", TYPES)
 def test_oracle_equals_numpy_decoder_on_synthetic_blocks(orc, lib, t):
     from rustorch_amd import synth
-    be = 32 if t in (8, 2) else 256
+    be = 256 if t in (10, 11, 12, 13, 14) else 32
     raw = synth.blocks(t, 11, 3, 6, 2 * be)
     got = orc.dequant(t, raw, 6, 2 * be)
     assert np.array_equal(bits(got.reshape(-1)), bits(nb.decode(t, raw)))
