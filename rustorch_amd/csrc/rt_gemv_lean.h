@@ -388,9 +388,115 @@ __device__ __forceinline__ void lean_problem_t(const GemvProb &P, int wg, int n_
     }
 }
 
+// Rows of more than one pass with the planner's ksplit: the unit of work is one pass of one row.  The workgroup owns the
+// rows wg, wg + n_wg, ...; their passes, in row order, are dealt out round-robin to its waves (so neighbouring waves read
+// neighbouring pieces of one row at the same time); every pass is reduced over its wave on its own and left in LDS behind
+// x; at the end the workgroup adds the passes of each row in pass order and stores.  A wave's work is then a multiple of
+// a third of a long row instead of whole rows -- a launch ends with its slowest wave, and a wave streams a 9 KB row in
+// about 6 us -- and a row's result does not depend on how the launch was cut: each (row, pass) sum is the same 64 lanes.
+template <int TYPE, bool EXACT>
+__device__ __forceinline__ void lean_problem_split(const GemvProb &P, int wg, int n_wg, int m, uint32_t *lds, float *red) {
+    const int lane = (int)(threadIdx.x & 63);
+    const int waves = (int)(blockDim.x >> 6);
+    const int U = units_of(TYPE, P.K), n_iter = (U + 63) >> 6;
+    const int N = P.N;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int rows_wg = wg < N ? (N - wg + n_wg - 1) / n_wg : 0;
+    const int items = rows_wg * n_iter;
+    const int steps = w < items ? (items - w + waves - 1) / waves : 0;
+    const uint32_t row_bytes = (uint32_t)P.row_bytes;
+    const __amdgpu_buffer_rsrc_t rsrc = weight_rsrc(P.w);
+    const bool add_to_y = P.res != nullptr;
+    float *y = P.y + (size_t)m * N;
+    float *part = reinterpret_cast<float *>(lds) + ((gemv_lds_bytes(TYPE, (size_t)P.K) + 15) >> 4) * 4;      // [rows_wg][n_iter]
+
+    LeanLane<TYPE> L;
+    L.init(lane);
+
+    // item = (j: which of the workgroup's rows, p: pass); a wave moves on by `waves` items
+    struct Pos { int j, p; };
+    const int dj = waves / n_iter, dp = waves % n_iter;
+    auto next = [&](Pos q) {
+        Pos r{ q.j + dj, q.p + dp };
+        if (r.p >= n_iter) { r.p -= n_iter; r.j++; }
+        return r;
+    };
+    auto request = [&](WRegs<TYPE> &wr, Pos s) {
+        uint32_t so = 0, vo = 0;
+        if (EXACT) so = (uint32_t)s.p * LeanLane<TYPE>::kPassBytes;
+        else vo = (uint32_t)(s.p - ((lane + 64 * s.p >= U) ? 1 : 0)) * LeanLane<TYPE>::kPassBytes;      // n_iter > 1 here: U >= 64
+        const int row = min(wg + n_wg * s.j, N - 1);
+        L.load(wr, WRow{ rsrc, (uint32_t)row * row_bytes + so }, vo);
+    };
+
+    WRegs<TYPE> a, b;
+    Pos pa{ w / n_iter, w % n_iter }, pb = next(pa);
+    // x first, then two steps of weights (both whatever the number of steps: a wave with fewer rereads the first pass of the
+    // workgroup's first row, see lean_problem_t)
+    LeanStage S;
+#ifndef RT_LEAN_NO_STAGE
+    S.issue(P, m);
+#endif
+    request(a, steps > 0 ? pa : Pos{ 0, 0 });
+    request(b, steps > 1 ? pb : (steps > 0 ? pa : Pos{ 0, 0 }));
+#ifndef RT_LEAN_NO_STAGE
+    S.finish<TYPE>(P, m, lds, red);
+#endif
+
+    auto consume = [&](const WRegs<TYPE> &wr, Pos s) {
+        const int u = lane + 64 * s.p;
+        XRegs<TYPE> x;
+        float d;
+        if (EXACT) {
+            load_x(x, lds, u, U, P.K);
+            d = RT_LEAN_DOT(L, wr, x);
+        } else {
+            const float live = u < U ? 1.f : 0.f;
+            load_x(x, lds, min(u, U - 1), U, P.K);
+            d = live * RT_LEAN_DOT(L, wr, x);
+        }
+        d = wave_sum_dpp(d);
+        if (lane == 0) part[s.j * n_iter + s.p] = d;
+    };
+
+    int s = 0;
+    while (s + 3 < steps) {
+        consume(a, pa);
+        pa = next(pb);
+        request(a, pa);
+        consume(b, pb);
+        pb = next(pa);
+        request(b, pb);
+        s += 2;
+    }
+    const int left = steps - s;
+    if (left == 3) {
+        consume(a, pa);
+        pa = next(pb);
+        request(a, pa);
+        consume(b, pb);
+        consume(a, pa);
+    } else if (left > 0) {
+        consume(a, pa);
+        if (left == 2) consume(b, pb);
+    }
+    __syncthreads();
+    for (int j = (int)threadIdx.x; j < rows_wg; j += (int)blockDim.x) {
+        float sum = part[j * n_iter];
+        for (int p = 1; p < n_iter; p++) sum += part[j * n_iter + p];
+        const int row = wg + n_wg * j;
+        if (add_to_y) unsafeAtomicAdd(&y[row], sum);
+        else y[row] = sum;
+    }
+}
+
 template <int TYPE, int R, bool DUAL>
 __device__ __forceinline__ void lean_problem(const GemvProb &P, int wg, int n_wg, int m, uint32_t *lds, float *red) {
-    if ((units_of(TYPE, P.K) & 63) == 0) lean_problem_t<TYPE, R, DUAL, true>(P, wg, n_wg, m, lds, red);
+    const bool exact = (units_of(TYPE, P.K) & 63) == 0;
+    if (!DUAL && R == 1 && P.ksplit) {
+        if (exact) lean_problem_split<TYPE, true>(P, wg, n_wg, m, lds, red);
+        else lean_problem_split<TYPE, false>(P, wg, n_wg, m, lds, red);
+    } else if (exact) lean_problem_t<TYPE, R, DUAL, true>(P, wg, n_wg, m, lds, red);
     else lean_problem_t<TYPE, R, DUAL, false>(P, wg, n_wg, m, lds, red);
 }
 

@@ -61,6 +61,8 @@ struct GemvProb {
     int stage, epi;
     int tile0;           // index of this problem's first tile in the launch
     int rows_per_tile;
+    int ksplit;          // set by the planner (lean path, rows of more than one pass): a wave's unit of work is one pass of one
+                         // row, the passes of a row are summed through LDS at the end of the workgroup
 };
 constexpr int kMaxGemvProbs = 8;
 struct GemvArgs {

@@ -108,10 +108,9 @@ int run_case(const Case &c) {
     orc_qgemv_f64(c.type, w.data, c.N, c.K, xeff.data(), (size_t)c.batch, y64.data(), wn.data(), 0);
     if (c.epi == kEpiSwiglu) orc_qgemv_f64(c.type, w2.data, c.N, c.K, xeff.data(), (size_t)c.batch, y64b.data(), wn2.data(), 0);
 
-    float *out[2] = { nullptr, nullptr };
-    int rc = 0;
-    for (int path = 0; path < (c.lean ? 2 : 1) && !rc; path++) {       // 0: general, 1: lean
-        float *y = (float *)malloc(c.N * (size_t)c.batch * 4);
+    bool split_used = false;
+    // one launch of the case down one path (0: general, 1: lean) with the planner given `budget` workgroups
+    auto run = [&](int path, int budget, float *y, int &rc) {
         for (size_t i = 0; i < c.N * (size_t)c.batch; i++) y[i] = c.residual ? res[i] : -12345.f;
         GemvArgs a;
         memset(&a, 0, sizeof a);
@@ -123,9 +122,11 @@ int run_case(const Case &c) {
         p.row_bytes = w.row_bytes; p.type = c.type; p.N = (int)c.N; p.K = (int)c.K; p.stage = c.stage; p.epi = c.epi;
         GemvPlan pl;
         GemvPlanHints h;
-        h.threads = c.threads; h.r2 = c.r2; h.budget = c.budget;
-        if (!plan_qgemv(a, c.batch, pl, h)) { printf("%s: plan refused\n", c.name); return 1; }
-        if (pl.lean != c.lean) { printf("%s: the planner %s this case down the lean path\n", c.name, pl.lean ? "sends" : "does not send"); return 1; }
+        h.threads = c.threads; h.r2 = c.r2; h.budget = budget;
+        if (!plan_qgemv(a, c.batch, pl, h)) { printf("%s: plan refused\n", c.name); rc = 1; return; }
+        if (pl.lean != c.lean) { printf("%s: the planner %s this case down the lean path\n", c.name, pl.lean ? "sends" : "does not send"); rc = 1; return; }
+        if (path == 0) p.ksplit = 0;      // the general path knows whole rows only
+        split_used = split_used || p.ksplit != 0;
         for (int m = 0; m < c.batch && !rc; m++) {
             static float red[16];
             bool ok = emu::launch((unsigned)pl.wgs, (unsigned)pl.threads, pl.lds, [&] {
@@ -139,7 +140,6 @@ int run_case(const Case &c) {
             });
             if (!ok) { printf("%s: path %d stalled\n", c.name, path); rc = 1; }
         }
-        out[path] = y;
         // against the f64 products
         for (int m = 0; m < c.batch && !rc; m++) {
             double xn = 0;
@@ -158,20 +158,80 @@ int run_case(const Case &c) {
             }
             if (!(worst <= 2e-5)) { printf("%s: path %d row %d: max |delta| / (|w| |x|) = %.3e\n", c.name, path, m, worst); rc = 1; }
         }
+    };
+    const size_t n_out = c.N * (size_t)c.batch;
+    float *out[3] = { (float *)malloc(n_out * 4), (float *)malloc(n_out * 4), (float *)malloc(n_out * 4) };
+    int rc = 0;
+    run(0, c.budget, out[0], rc);
+    if (c.lean && !rc) {
+        run(1, c.budget, out[1], rc);
+        if (!rc) run(1, c.budget + 2, out[2], rc);      // the same rows cut into another number of workgroups
+        if (!rc && memcmp(out[1], out[2], n_out * 4) != 0) { printf("%s: the lean result depends on how the launch is cut\n", c.name); rc = 1; }
+        // whole rows per wave: the general path's bits; passes summed through LDS: another order of additions, same bound
+        if (!rc && !split_used && memcmp(out[0], out[1], n_out * 4) != 0) {
+            size_t bad = 0;
+            for (size_t i = 0; i < n_out; i++) bad += out[0][i] != out[1][i];
+            printf("%s: lean and general results differ in %zu of %zu elements\n", c.name, bad, n_out);
+            rc = 1;
+        }
     }
-    if (!rc && c.lean && memcmp(out[0], out[1], c.N * (size_t)c.batch * 4) != 0) {
-        size_t bad = 0;
-        for (size_t i = 0; i < c.N * (size_t)c.batch; i++) bad += out[0][i] != out[1][i];
-        printf("%s: lean and general results differ in %zu of %zu elements\n", c.name, bad, c.N * (size_t)c.batch);
-        rc = 1;
-    }
-    printf("%-44s %s\n", c.name, rc ? "FAIL" : "ok");
+    printf("%-50s %s%s\n", c.name, rc ? "FAIL" : "ok", split_used ? "  (passes dealt out)" : "");
     fflush(stdout);
-    free(out[0]); free(out[1]); free(xd); free(xqd); free(gd); free(w.data); free(w2.data);
+    free(out[0]); free(out[1]); free(out[2]); free(xd); free(xqd); free(gd); free(w.data); free(w2.data);
     return rc;
 }
 
 }  // namespace
+
+// The planner on the benchmark's own launches (no device code runs): shares are positive, contiguous and within the
+// budget, and the busiest wave of the layer launch streams within 5 % of the mean (31.7 KB), rounding included.
+int check_planner() {
+    using namespace rt;
+    struct M { int type, N, K; size_t rb; };
+    const M layer[7] = { { RT_GGML_Q4_K, 4096, 4096, 2304 }, { RT_GGML_Q4_K, 4096, 4096, 2304 }, { RT_GGML_Q6_K, 4096, 4096, 3360 }, { RT_GGML_Q4_K, 4096, 4096, 2304 },
+                         { RT_GGML_Q4_K, 11008, 4096, 2304 }, { RT_GGML_Q4_K, 11008, 4096, 2304 }, { RT_GGML_Q6_K, 4096, 11008, 9030 } };
+    int rc = 0;
+    for (int which = 0; which < 3; which++) {      // the layer in one launch; q, k, v of the decode step; the down-projection with its residual
+        GemvArgs a;
+        memset(&a, 0, sizeof a);
+        static float dummy;
+        const int first = which == 0 ? 0 : (which == 1 ? 0 : 6), n = which == 0 ? 7 : (which == 1 ? 3 : 1);
+        a.n = n;
+        double bytes = 0;
+        for (int i = 0; i < n; i++) {
+            const M &mm = layer[first + i];
+            GemvProb &p = a.p[i];
+            p.type = mm.type; p.N = mm.N; p.K = mm.K; p.row_bytes = mm.rb; p.y = &dummy; p.res = which == 2 ? &dummy : nullptr;
+            bytes += (double)mm.N * mm.rb;
+        }
+        GemvPlan pl;
+        if (!plan_qgemv(a, 1, pl)) { printf("planner: launch %d refused\n", which); return 1; }
+        const int waves = pl.threads / 64, budget = 256 * (1024 / pl.threads);
+        int next = 0;
+        double busiest = 0;
+        printf("planner launch %d: %d threads, lean %d, lds %zu, shares", which, pl.threads, (int)pl.lean, pl.lds);
+        for (int i = 0; i < n; i++) {
+            const GemvProb &p = a.p[i];
+            printf(" %d%s", p.rows_per_tile, p.ksplit ? "*" : "");
+            if (p.tile0 != next || p.rows_per_tile < 1) rc = 1;
+            next += p.rows_per_tile;
+            const int n_iter = (p.K / 64 + 63) / 64;
+            double wb;
+            if (p.ksplit) {
+                const long rows_wg = (p.N + p.rows_per_tile - 1) / p.rows_per_tile;
+                wb = (double)((rows_wg * n_iter + waves - 1) / waves) * p.row_bytes / n_iter;
+                if (rows_wg * n_iter * 4 + ((gemv_lds_bytes(p.type, (size_t)p.K) + 15) & ~(size_t)15) > pl.lds) rc = 1;
+            } else wb = (double)((p.N + (long)waves * p.rows_per_tile - 1) / ((long)waves * p.rows_per_tile)) * p.row_bytes;
+            busiest = wb > busiest ? wb : busiest;
+        }
+        const double mean = bytes / ((double)next * waves);
+        printf("  (* passes dealt out); busiest wave %.1f KB, mean %.1f KB\n", busiest / 1024, mean / 1024);
+        if (next != pl.wgs || next > budget || !pl.lean) rc = 1;
+        if (which == 0 && busiest > 1.05 * mean) rc = 1;
+    }
+    if (rc) printf("planner: FAIL\n");
+    return rc;
+}
 
 int main(int argc, char **argv) {
     using namespace rt;
@@ -193,12 +253,17 @@ int main(int argc, char **argv) {
         { "q4_0 5x96 rms", Q40, 5, 96, kStageRms, kEpiStore, false, -1, -1, 2, 1 },
         { "q4_0 11x11008 xq (ragged sixth pass), two rows", Q40, 11, 11008, kStageXq, kEpiStore, true, 512, 1, 1, 1 },
         { "q4_0 6x2048 f32, gate/up pair", Q40, 6, 2048, kStageF32, kEpiSwiglu, false, 512, 0, 1, 1 },
+        // one row per step and rows of several passes: the passes of a row go to different waves and meet in LDS
+        { "q6k 21x11008 xq, one row per step", Q6K, 21, 11008, kStageXq, kEpiStore, false, 512, 0, 2, 1 },
+        { "q4k 13x8192 rms, one row per step, residual", Q4K, 13, 8192, kStageRms, kEpiStore, true, 512, 0, 3, 1 },
+        { "q8_0 9x4096 f32, one row per step, two vectors", Q80, 9, 4096, kStageF32, kEpiStore, false, 512, 0, 1, 2 },
+        { "q4_0 5x11008 xq, planner's own choice", Q40, 5, 11008, kStageXq, kEpiStore, false, -1, -1, 2, 1 },
         // formats of the general path alone
         { "q8_1 5x96 f32", Q81, 5, 96, kStageF32, kEpiStore, false, -1, -1, 2, 1, false },
         { "q8_1 13x4096 rms, two rows, residual", Q81, 13, 4096, kStageRms, kEpiStore, true, 512, 1, 1, 1, false },
         { "q8_1 7x11008 xq (ragged), gate/up pair", Q81, 7, 11008, kStageXq, kEpiSwiglu, false, 512, 0, 1, 1, false },
     };
-    int rc = 0;
+    int rc = check_planner();
     const int only = argc > 1 ? atoi(argv[1]) : -1;
     for (size_t i = 0; i < sizeof cases / sizeof cases[0]; i++)
         if (only < 0 || only == (int)i) rc |= run_case(cases[i]);
