@@ -322,6 +322,8 @@ __device__ __forceinline__ void lean_problem_t(const GemvProb &P, int wg, int n_
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
 
+    constexpr bool kPasswise = !DUAL && R == 1;
+    float row_sum = 0.f;
     auto consume = [&](const WRegs<TYPE> *w, Pos s) {
         const int u = lane + 64 * s.p;
         XRegs<TYPE> x;
@@ -335,9 +337,19 @@ __device__ __forceinline__ void lean_problem_t(const GemvProb &P, int wg, int n_
 #pragma unroll
             for (int r = 0; r < R; r++) acc[r] = __builtin_fmaf(live, RT_LEAN_DOT(L, w[r], x), acc[r]);
         }
-        if (s.p != n_iter - 1) return;
+        if (kPasswise) {
+            // One row per step: a row's result is the sum, in pass order, of its passes' wave sums -- the same value, bit
+            // for bit, that the split form builds through LDS, so a launch's shape never changes a result.
+            row_sum += wave_sum_dpp(acc[0]);
+            acc[0] = 0.f;
+            if (s.p != n_iter - 1) return;
+            acc[0] = row_sum;
+            row_sum = 0.f;
+        } else {
+            if (s.p != n_iter - 1) return;
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r] = wave_sum_dpp(acc[r]);
+            for (int r = 0; r < R; r++) acc[r] = wave_sum_dpp(acc[r]);
+        }
         if (DUAL) {
 #pragma unroll
             for (int r = 0; r < RG; r++) {

@@ -110,7 +110,7 @@ int run_case(const Case &c) {
 
     bool split_used = false;
     // one launch of the case down one path (0: general, 1: lean) with the planner given `budget` workgroups
-    auto run = [&](int path, int budget, float *y, int &rc) {
+    auto run = [&](int path, int budget, float *y, int &rc, bool whole_rows = false) {
         for (size_t i = 0; i < c.N * (size_t)c.batch; i++) y[i] = c.residual ? res[i] : -12345.f;
         GemvArgs a;
         memset(&a, 0, sizeof a);
@@ -125,7 +125,7 @@ int run_case(const Case &c) {
         h.threads = c.threads; h.r2 = c.r2; h.budget = budget;
         if (!plan_qgemv(a, c.batch, pl, h)) { printf("%s: plan refused\n", c.name); rc = 1; return; }
         if (pl.lean != c.lean) { printf("%s: the planner %s this case down the lean path\n", c.name, pl.lean ? "sends" : "does not send"); rc = 1; return; }
-        if (path == 0) p.ksplit = 0;      // the general path knows whole rows only
+        if (path == 0 || whole_rows) p.ksplit = 0;      // the general path knows whole rows only
         split_used = split_used || p.ksplit != 0;
         for (int m = 0; m < c.batch && !rc; m++) {
             static float red[16];
@@ -167,7 +167,12 @@ int run_case(const Case &c) {
         run(1, c.budget, out[1], rc);
         if (!rc) run(1, c.budget + 2, out[2], rc);      // the same rows cut into another number of workgroups
         if (!rc && memcmp(out[1], out[2], n_out * 4) != 0) { printf("%s: the lean result depends on how the launch is cut\n", c.name); rc = 1; }
-        // whole rows per wave: the general path's bits; passes summed through LDS: another order of additions, same bound
+        // a launch too tight on LDS to deal passes out keeps whole rows per wave: the same bits all the same
+        if (!rc && split_used) {
+            run(1, c.budget, out[2], rc, true);
+            if (!rc && memcmp(out[1], out[2], n_out * 4) != 0) { printf("%s: whole rows and dealt-out passes give different bits\n", c.name); rc = 1; }
+        }
+        // rows of one pass: the general path's bits; rows of several: pass sums added in order, same bound
         if (!rc && !split_used && memcmp(out[0], out[1], n_out * 4) != 0) {
             size_t bad = 0;
             for (size_t i = 0; i < n_out; i++) bad += out[0][i] != out[1][i];
