@@ -186,6 +186,68 @@ int run_case(const Case &c) {
     return rc;
 }
 
+// Several problems in one launch, as the decode step and the benchmark's layer issue them: every problem's result is, bit
+// for bit, what a launch of that problem alone gives, and within the held tolerance of the oracle's f64 products.
+struct GroupSpec { int type; size_t N, K; };
+int run_group(const char *name, const std::vector<GroupSpec> &specs, int budget) {
+    using namespace rt;
+    const size_t n = specs.size();
+    std::vector<Weights> ws;
+    std::vector<float *> xs, ys, singles;
+    for (size_t i = 0; i < n; i++) {
+        ws.push_back(make_weights(specs[i].type, 20 + i, specs[i].N, specs[i].K));
+        float *x = (float *)malloc(specs[i].K * 4);
+        rt_synth_normal_f32(11, 40 + i, specs[i].K, 0.f, 1.f, x);
+        xs.push_back(x);
+        ys.push_back((float *)malloc(specs[i].N * 4));
+        singles.push_back((float *)malloc(specs[i].N * 4));
+    }
+    int rc = 0;
+    auto launch = [&](size_t first, size_t count, std::vector<float *> &out, int wgs_budget) {
+        GemvArgs a;
+        memset(&a, 0, sizeof a);
+        a.n = (int)count;
+        for (size_t i = 0; i < count; i++) {
+            GemvProb &p = a.p[i];
+            const Weights &w = ws[first + i];
+            p.w = w.data; p.x = xs[first + i]; p.y = out[first + i]; p.eps = 1e-5f;
+            p.row_bytes = w.row_bytes; p.type = w.type; p.N = (int)w.N; p.K = (int)w.K; p.stage = kStageF32; p.epi = kEpiStore;
+            for (size_t r = 0; r < w.N; r++) out[first + i][r] = -12345.f;
+        }
+        GemvPlan pl;
+        GemvPlanHints h;
+        h.budget = wgs_budget;
+        if (!plan_qgemv(a, 1, pl, h) || !pl.lean) { printf("%s: plan refused or not lean\n", name); rc = 1; return; }
+        static float red[16];
+        bool ok = emu::launch((unsigned)pl.wgs, (unsigned)pl.threads, pl.lds, [&] {
+            RT_DYN_LDS(uint4, lds4);
+            uint32_t *lds = reinterpret_cast<uint32_t *>(lds4);
+            const int wg = (int)blockIdx.x;
+            RT_GEMV_PICK_PROBLEM(a, wg, P);
+            if (pl.r2) lean_dispatch<2>(P, wg - P.tile0, P.rows_per_tile, 0, lds, red);
+            else lean_dispatch<1>(P, wg - P.tile0, P.rows_per_tile, 0, lds, red);
+        });
+        if (!ok) { printf("%s: stalled\n", name); rc = 1; }
+    };
+    launch(0, n, ys, budget);
+    for (size_t i = 0; i < n && !rc; i++) {
+        launch(i, 1, singles, 3);
+        if (rc) break;
+        if (memcmp(ys[i], singles[i], specs[i].N * 4) != 0) { printf("%s: problem %zu differs from its own launch\n", name, i); rc = 1; }
+        std::vector<double> y64(specs[i].N), wn(specs[i].N);
+        orc_qgemv_f64(specs[i].type, ws[i].data, specs[i].N, specs[i].K, xs[i], 1, y64.data(), wn.data(), 0);
+        double xn = 0, worst = 0;
+        for (size_t k = 0; k < specs[i].K; k++) xn += (double)xs[i][k] * xs[i][k];
+        xn = sqrt(xn);
+        for (size_t r = 0; r < specs[i].N; r++) worst = fmax(worst, fabs((double)ys[i][r] - y64[r]) / (wn[r] * xn));
+        if (!(worst <= 2e-5)) { printf("%s: problem %zu: max |delta| / (|w| |x|) = %.3e\n", name, i, worst); rc = 1; }
+    }
+    printf("%-50s %s\n", name, rc ? "FAIL" : "ok");
+    fflush(stdout);
+    for (size_t i = 0; i < n; i++) { free(ws[i].data); free(xs[i]); free(ys[i]); free(singles[i]); }
+    return rc;
+}
+
 }  // namespace
 
 // The planner on the benchmark's own launches (no device code runs): shares are positive, contiguous and within the
@@ -272,6 +334,11 @@ int main(int argc, char **argv) {
     const int only = argc > 1 ? atoi(argv[1]) : -1;
     for (size_t i = 0; i < sizeof cases / sizeof cases[0]; i++)
         if (only < 0 || only == (int)i) rc |= run_case(cases[i]);
+    if (only < 0) {
+        rc |= run_group("five problems of mixed formats and row lengths", { { Q4K, 40, 4096 }, { Q4K, 12, 4096 }, { Q6K, 33, 4096 }, { Q6K, 9, 11008 }, { Q80, 10, 4096 } }, 9);
+        rc |= run_group("a layer's seven projections, rows / 128", { { Q4K, 32, 4096 }, { Q4K, 32, 4096 }, { Q6K, 32, 4096 }, { Q4K, 32, 4096 }, { Q4K, 86, 4096 }, { Q4K, 86, 4096 }, { Q6K, 32, 11008 } }, 12);
+        rc |= run_group("more problems than the budget has workgroups", { { Q40, 5, 96 }, { Q4K, 3, 256 }, { Q6K, 7, 768 }, { Q80, 4, 11008 } }, 2);
+    }
     printf(rc ? "EMU FAIL\n" : "EMU OK\n");
     return rc;
 }
