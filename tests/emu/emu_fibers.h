@@ -3,10 +3,10 @@
 #pragma once
 
 #include <sys/mman.h>
-#include <ucontext.h>
 
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <functional>
 #include <vector>
 
@@ -15,35 +15,70 @@
 #if defined(__has_feature)
 #if __has_feature(address_sanitizer)
 #define EMU_ASAN 1
+#include <sanitizer/asan_interface.h>
 #include <sanitizer/common_interface_defs.h>
 #endif
 #endif
 
 // ------------------------------------------------------------------ fiber runtime
+// The switch between two stacks, written out (x86-64, System V): callee-saved registers on the old stack, stack pointers
+// exchanged, the same registers off the new stack.  swapcontext would do, but AddressSanitizer intercepts it and clears
+// the shadow of the whole stack it switches to, every time, which makes a launch of a few hundred thousand fibers take
+// minutes.  The sanitizer is told about every switch through its fiber interface instead.
+extern "C" void emu_switch_stack(void **save_sp, void *new_sp);
+asm(R"(
+    .text
+    .p2align 4
+    .globl emu_switch_stack
+    .hidden emu_switch_stack
+    .type emu_switch_stack,@function
+emu_switch_stack:
+    pushq %rbp
+    pushq %rbx
+    pushq %r12
+    pushq %r13
+    pushq %r14
+    pushq %r15
+    movq %rsp, (%rdi)
+    movq %rsi, %rsp
+    popq %r15
+    popq %r14
+    popq %r13
+    popq %r12
+    popq %rbx
+    popq %rbp
+    ret
+    .size emu_switch_stack, .-emu_switch_stack
+)");
+
 namespace emu {
 
-enum State { RUNNABLE, AT_SYNC, AT_WAVE, SPIN, DONE };
-constexpr size_t kStack = 512 * 1024;
+enum State { RUNNABLE, AT_SYNC, AT_WAVE, AT_GATHER, AT_UNIFORM, SPIN, DONE };
+constexpr size_t kStack = 256 * 1024;      // above one guard page
 
 struct Fiber {
-    ucontext_t ctx;
+    void *sp = nullptr;       // where the fiber's registers lie while it is not running
     char *stack = nullptr;
     State state = RUNNABLE;
     Idx3 tid{ 0, 0, 0 };
+    unsigned linear = 0;      // thread number within the workgroup (x fastest): lanes of a wave are 64 consecutive numbers
     int block = 0;
     uint32_t xval = 0, xres = 0;
     int xsrc = 0;
-    bool started = false;
+    const void *gmine = nullptr;   // wave gather: this lane's contribution ...
+    size_t gbytes = 0;             // ... of this many bytes
+    const void *gall = nullptr;    // ... and, afterwards, the wave's 64 contributions in lane order
 };
 
 struct Block {
     std::vector<Fiber> fibers;
+    std::vector<std::vector<char>> gather;   // one buffer per wave
     Idx3 bid{ 0, 0, 0 };
-    bool done = false;
+    bool started = false, done = false;
 };
 
 Fiber *g_cur = nullptr;
-static ucontext_t g_main;
+static void *g_main_sp = nullptr;
 static const void *g_main_bottom = nullptr;
 static size_t g_main_size = 0;
 static std::vector<Block> g_blocks;
@@ -51,13 +86,15 @@ static Idx3 g_bdim{ 1, 1, 1 }, g_gdim{ 1, 1, 1 };
 static std::vector<char> g_lds;
 static std::function<void()> g_kernel;
 static long g_switches = 0;
+static std::vector<char *> g_stack_pool;
 
 Idx3 &tid() { return g_cur->tid; }
 Idx3 &bid() { return g_blocks[(size_t)g_cur->block].bid; }
 Idx3 &bdim() { return g_bdim; }
 Idx3 &gdim() { return g_gdim; }
 void *dyn_lds() { return g_lds.data(); }
-int lane_id() { return (int)(g_cur->tid.x & 63); }
+size_t dyn_lds_bytes() { return g_lds.size(); }
+int lane_id() { return (int)(g_cur->linear & 63); }
 
 static void to_main() {
     Fiber *f = g_cur;
@@ -65,7 +102,7 @@ static void to_main() {
     void *fake = nullptr;
     __sanitizer_start_switch_fiber(f->state == DONE ? nullptr : &fake, g_main_bottom, g_main_size);
 #endif
-    swapcontext(&f->ctx, &g_main);
+    emu_switch_stack(&f->sp, g_main_sp);
 #ifdef EMU_ASAN
     __sanitizer_finish_switch_fiber(fake, &g_main_bottom, &g_main_size);
 #endif
@@ -79,6 +116,14 @@ uint32_t wave_exchange(uint32_t v, int src) {
     g_cur->state = AT_WAVE;
     to_main();
     return g_cur->xres;
+}
+void uniform_point() { g_cur->state = AT_UNIFORM; to_main(); }
+const void *wave_gather(const void *mine, size_t bytes) {
+    g_cur->gmine = mine;
+    g_cur->gbytes = bytes;
+    g_cur->state = AT_GATHER;
+    to_main();
+    return g_cur->gall;
 }
 
 static void fiber_entry() {
@@ -97,11 +142,54 @@ static void resume(Fiber &f) {
     void *fake = nullptr;
     __sanitizer_start_switch_fiber(&fake, f.stack, kStack);
 #endif
-    swapcontext(&g_main, &f.ctx);
+    emu_switch_stack(&g_main_sp, f.sp);
 #ifdef EMU_ASAN
     __sanitizer_finish_switch_fiber(fake, nullptr, nullptr);
 #endif
     g_cur = nullptr;
+}
+
+static char *take_stack() {
+    if (!g_stack_pool.empty()) {
+        char *s = g_stack_pool.back();
+        g_stack_pool.pop_back();
+#ifdef EMU_ASAN
+        __asan_unpoison_memory_region(s, kStack);      // the frames of the fiber that ran here last never returned
+#endif
+        return s;
+    }
+    char *s = (char *)mmap(nullptr, kStack + 4096, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+    if (s == (char *)MAP_FAILED) { perror("mmap"); exit(2); }
+    mprotect(s, 4096, PROT_NONE);      // a fiber that outgrows its stack stops here instead of writing into another's
+    return s + 4096;
+}
+
+static void start_block(Block &b, int index) {
+    const unsigned n = g_bdim.x * g_bdim.y * g_bdim.z;
+    b.fibers.resize(n);
+    b.gather.assign((n + 63) / 64, std::vector<char>());
+    for (unsigned t = 0; t < n; t++) {
+        Fiber &f = b.fibers[t];
+        f.linear = t;
+        f.tid = Idx3{ t % g_bdim.x, t / g_bdim.x % g_bdim.y, t / (g_bdim.x * g_bdim.y) };
+        f.block = index;
+        f.stack = take_stack();
+        // the first switch to the fiber pops six registers and returns into fiber_entry, the stack then as after a call
+        void **top = reinterpret_cast<void **>(f.stack + kStack);
+        *--top = nullptr;                                   // the return address fiber_entry never uses
+        *--top = reinterpret_cast<void *>(&fiber_entry);
+        for (int r = 0; r < 6; r++) *--top = nullptr;
+        f.sp = top;
+    }
+    b.started = true;
+}
+
+static void finish_block(Block &b) {
+    for (Fiber &f : b.fibers) g_stack_pool.push_back(f.stack);
+    b.fibers.clear();
+    b.fibers.shrink_to_fit();
+    b.gather.clear();
+    b.done = true;
 }
 
 // Runs the workgroup until it is finished or stuck in a spin wait. Returns false on a dead rendezvous.
@@ -114,18 +202,49 @@ static bool run_block(Block &b) {
         // wave rendezvous: exchange among the lanes that are waiting at a wave operation
         for (size_t w0 = 0; w0 < n; w0 += 64) {
             size_t w1 = std::min(n, w0 + 64);
-            bool any = false;
-            for (size_t i = w0; i < w1; i++) any = any || b.fibers[i].state == AT_WAVE;
-            if (!any) continue;
+            bool any = false, any_gather = false, any_uniform = false;
             for (size_t i = w0; i < w1; i++) {
-                Fiber &f = b.fibers[i];
-                if (f.state != AT_WAVE) continue;
-                size_t s = w0 + (size_t)(f.xsrc & 63);
-                f.xres = (f.xsrc >= 0 && s < w1 && b.fibers[s].state == AT_WAVE) ? b.fibers[s].xval : f.xval;
+                any = any || b.fibers[i].state == AT_WAVE;
+                any_gather = any_gather || b.fibers[i].state == AT_GATHER;
+                any_uniform = any_uniform || b.fibers[i].state == AT_UNIFORM;
             }
-            for (size_t i = w0; i < w1; i++)
-                if (b.fibers[i].state == AT_WAVE) b.fibers[i].state = RUNNABLE;
-            progressed = true;
+            // lanes at an instruction every lane executes (a wait, which lanes cannot skip) stay there until the lanes
+            // that are still at wave operations before it have caught up: lanes that skipped a predicated operation
+            // run ahead of the others by that much and no further
+            if (any_uniform && !any && !any_gather) {
+                for (size_t i = w0; i < w1; i++)
+                    if (b.fibers[i].state == AT_UNIFORM) b.fibers[i].state = RUNNABLE;
+                progressed = true;
+            }
+            if (any) {
+                for (size_t i = w0; i < w1; i++) {
+                    Fiber &f = b.fibers[i];
+                    if (f.state != AT_WAVE) continue;
+                    size_t s = w0 + (size_t)(f.xsrc & 63);
+                    f.xres = (f.xsrc >= 0 && s < w1 && b.fibers[s].state == AT_WAVE) ? b.fibers[s].xval : f.xval;
+                }
+                for (size_t i = w0; i < w1; i++)
+                    if (b.fibers[i].state == AT_WAVE) b.fibers[i].state = RUNNABLE;
+                progressed = true;
+            }
+            if (any_gather) {
+                size_t bytes = 0;
+                for (size_t i = w0; i < w1; i++)
+                    if (b.fibers[i].state == AT_GATHER) bytes = std::max(bytes, b.fibers[i].gbytes);
+                std::vector<char> &buf = b.gather[w0 / 64];
+                buf.assign(64 * bytes, 0);      // lanes that are not at the operation contribute zeros
+                for (size_t i = w0; i < w1; i++) {
+                    Fiber &f = b.fibers[i];
+                    if (f.state == AT_GATHER) memcpy(buf.data() + (i - w0) * bytes, f.gmine, f.gbytes);
+                }
+                for (size_t i = w0; i < w1; i++) {
+                    Fiber &f = b.fibers[i];
+                    if (f.state != AT_GATHER) continue;
+                    f.gall = buf.data();
+                    f.state = RUNNABLE;
+                }
+                progressed = true;
+            }
         }
         if (progressed) continue;
         size_t at_sync = 0, done = 0, spin = 0;
@@ -134,7 +253,7 @@ static bool run_block(Block &b) {
             done += f.state == DONE;
             spin += f.state == SPIN;
         }
-        if (done == n) { b.done = true; return true; }
+        if (done == n) { finish_block(b); return true; }
         if (at_sync + done == n) {
             for (Fiber &f : b.fibers)
                 if (f.state == AT_SYNC) f.state = RUNNABLE;
@@ -145,51 +264,44 @@ static bool run_block(Block &b) {
                 if (f.state == SPIN) f.state = RUNNABLE;
             return true;
         }
-        fprintf(stderr, "emu: dead rendezvous in workgroup %u (at_sync=%zu done=%zu)\n", b.bid.x, at_sync, done);
+        fprintf(stderr, "emu: dead rendezvous in workgroup (%u,%u,%u) (at_sync=%zu done=%zu)\n", b.bid.x, b.bid.y, b.bid.z, at_sync, done);
         return false;
     }
 }
 
-// Launch `kernel` on grid x block threads (1-D) with lds_bytes of launch-sized LDS. Returns false on a stall.
-bool launch(unsigned grid, unsigned block, size_t lds_bytes, std::function<void()> kernel) {
+// Launch `kernel` on grid x block threads with lds_bytes of launch-sized LDS.  Returns false on a stall.  A workgroup's
+// fibers exist from its first turn to its end; workgroups that never wait for one another run one after the other.
+bool launch3(Idx3 grid, Idx3 block, size_t lds_bytes, std::function<void()> kernel) {
     g_kernel = std::move(kernel);
-    g_bdim = Idx3{ block, 1, 1 };
-    g_gdim = Idx3{ grid, 1, 1 };
+    g_bdim = block;
+    g_gdim = grid;
     g_lds.assign(lds_bytes, 0);   // a heap buffer of exactly the launch's size: overruns are caught
-    g_blocks.assign(grid, Block());
-    for (unsigned bi = 0; bi < grid; bi++) {
-        Block &b = g_blocks[bi];
-        b.bid = Idx3{ bi, 0, 0 };
-        b.fibers.resize(block);
-        for (unsigned t = 0; t < block; t++) {
-            Fiber &f = b.fibers[t];
-            f.tid = Idx3{ t, 0, 0 };
-            f.block = (int)bi;
-            f.stack = (char *)mmap(nullptr, kStack, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
-            if (f.stack == (char *)MAP_FAILED) { perror("mmap"); exit(2); }
-            getcontext(&f.ctx);
-            f.ctx.uc_stack.ss_sp = f.stack;
-            f.ctx.uc_stack.ss_size = kStack;
-            f.ctx.uc_link = nullptr;
-            makecontext(&f.ctx, fiber_entry, 0);
-        }
-    }
+    const size_t n_blocks = (size_t)grid.x * grid.y * grid.z;
+    g_blocks.assign(n_blocks, Block());
+    for (size_t bi = 0; bi < n_blocks; bi++)
+        g_blocks[bi].bid = Idx3{ (unsigned)(bi % grid.x), (unsigned)(bi / grid.x % grid.y), (unsigned)(bi / ((size_t)grid.x * grid.y)) };
     bool ok = true;
     for (long rounds = 0; ok; rounds++) {
         bool all = true;
-        for (Block &b : g_blocks) {
+        for (size_t bi = 0; bi < n_blocks; bi++) {
+            Block &b = g_blocks[bi];
             if (b.done) continue;
             all = false;
+            if (!b.started) start_block(b, (int)bi);
             if (!run_block(b)) { ok = false; break; }
         }
         if (all) break;
         if (rounds > 100000) { fprintf(stderr, "emu: no progress after %ld rounds\n", rounds); ok = false; }
     }
     for (Block &b : g_blocks)
-        for (Fiber &f : b.fibers) munmap(f.stack, kStack);
+        if (b.started && !b.done) finish_block(b);
     g_blocks.clear();
+    g_kernel = nullptr;
     return ok;
 }
 
-}  // namespace emu
+bool launch(unsigned grid, unsigned block, size_t lds_bytes, std::function<void()> kernel) {
+    return launch3(Idx3{ grid, 1, 1 }, Idx3{ block, 1, 1 }, lds_bytes, std::move(kernel));
+}
 
+}  // namespace emu

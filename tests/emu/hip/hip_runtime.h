@@ -1,6 +1,6 @@
 // CPU stand-in for <hip/hip_runtime.h>: enough of the HIP device vocabulary to compile the kernels of
 // rustorch_amd/csrc as host C++ and run them as fibers (one per GPU thread) under AddressSanitizer.
-// TEST INFRASTRUCTURE: used only by tests/emu/emu_main.cpp.
+// TEST INFRASTRUCTURE: used only by the programs and the emulated library under tests/emu.
 //
 // Execution model: a workgroup's threads are fibers that run one after the other; a fiber runs until it
 // reaches __syncthreads(), a wave operation (shuffle / DPP / readlane), a sleep inside a spin loop, or its
@@ -10,10 +10,14 @@
 #pragma once
 
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstddef>
 #include <cstdint>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <functional>
 
 #define __global__
 #define __device__
@@ -21,23 +25,23 @@
 #define __forceinline__ inline
 #define __shared__ static
 #define __launch_bounds__(...)
-#define __align__(n) alignas(n)
+#define __align__(n) __attribute__((aligned(n)))
 
 struct uint2 { uint32_t x, y; };
 struct alignas(16) uint4 { uint32_t x, y, z, w; };
 struct float2 { float x, y; };
 struct alignas(16) float4 { float x, y, z, w; };
+inline uint2 make_uint2(uint32_t x, uint32_t y) { return uint2{ x, y }; }
+inline uint4 make_uint4(uint32_t x, uint32_t y, uint32_t z, uint32_t w) { return uint4{ x, y, z, w }; }
 inline float2 make_float2(float x, float y) { return float2{ x, y }; }
 inline float4 make_float4(float x, float y, float z, float w) { return float4{ x, y, z, w }; }
 struct dim3 { unsigned x = 1, y = 1, z = 1; dim3() {} dim3(unsigned a, unsigned b = 1, unsigned c = 1) : x(a), y(b), z(c) {} };
 
 typedef int hipError_t;
-typedef void *hipStream_t;
-typedef void *hipEvent_t;
-enum { hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2 };
-inline const char *hipGetErrorString(hipError_t) { return "emu"; }
-inline hipError_t hipGetLastError() { return hipSuccess; }
-inline hipError_t hipSetDevice(int) { return hipSuccess; }
+enum { hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2, hipErrorInvalidDevice = 101, hipErrorNotSupported = 801, hipErrorLaunchFailure = 719 };
+inline const char *hipGetErrorString(hipError_t e) {
+    return e == hipSuccess ? "no error" : (e == hipErrorNotSupported ? "not supported by the emulation" : (e == hipErrorLaunchFailure ? "emulated launch stalled" : "emulated HIP error"));
+}
 
 namespace emu {
 
@@ -49,13 +53,100 @@ Idx3 &bid();
 Idx3 &bdim();
 Idx3 &gdim();
 void *dyn_lds();
+size_t dyn_lds_bytes();
 void sync_threads();
 void spin_yield();
 // 64-lane rendezvous: every live lane of the wave deposits v; returns the value deposited by lane `src`
 uint32_t wave_exchange(uint32_t v, int src);
+// 64-lane rendezvous: every live lane deposits `bytes` bytes; returns the wave's 64 deposits in lane order (valid until
+// the wave's next operation; lanes that are not at the operation count as zeros)
+const void *wave_gather(const void *mine, size_t bytes);
+// An instruction that every lane of a wave executes whatever its predicates (the sources' hand-placed waits): the lanes
+// that arrive first wait here for the rest of their wave.  Lanes that skipped a predicated wave operation would otherwise
+// pair up, from then on, with the others' previous operation.
+void uniform_point();
 int lane_id();
+bool launch3(Idx3 grid, Idx3 block, size_t lds_bytes, std::function<void()> kernel);
+hipError_t &last_error();
 
 }  // namespace emu
+
+// ---- the host API the library uses: one device, synchronous "streams", device memory = exact-size heap blocks
+typedef struct emu_stream *hipStream_t;
+struct emu_event { std::chrono::steady_clock::time_point at; };
+typedef emu_event *hipEvent_t;
+typedef struct emu_graph *hipGraph_t;
+typedef struct emu_graph_exec *hipGraphExec_t;
+enum hipMemcpyKind { hipMemcpyHostToHost, hipMemcpyHostToDevice, hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice, hipMemcpyDefault };
+enum { hipStreamNonBlocking = 1, hipStreamCaptureModeThreadLocal = 1, hipFuncAttributeMaxDynamicSharedMemorySize = 8 };
+constexpr size_t kEmuDeviceBytes = (size_t)8 << 30;      // what the emulated device reports and hands out
+struct hipDeviceProp_t {
+    char name[256];
+    char gcnArchName[256];
+    int multiProcessorCount, warpSize, cooperativeLaunch;
+    size_t totalGlobalMem, sharedMemPerBlock;
+};
+inline hipError_t hipGetLastError() { hipError_t e = emu::last_error(); emu::last_error() = hipSuccess; return e; }
+inline hipError_t hipGetDeviceCount(int *n) { *n = 1; return hipSuccess; }
+inline hipError_t hipSetDevice(int d) { return d == 0 ? hipSuccess : hipErrorInvalidDevice; }
+inline hipError_t hipGetDevice(int *d) { *d = 0; return hipSuccess; }
+inline hipError_t hipGetDeviceProperties(hipDeviceProp_t *p, int d) {
+    if (d != 0) return hipErrorInvalidDevice;
+    memset(p, 0, sizeof *p);
+    snprintf(p->name, sizeof p->name, "CPU emulation of an MI355X");
+    snprintf(p->gcnArchName, sizeof p->gcnArchName, "gfx950 (emulated)");
+    p->multiProcessorCount = 256; p->warpSize = 64; p->cooperativeLaunch = 0;
+    p->totalGlobalMem = kEmuDeviceBytes; p->sharedMemPerBlock = 64 * 1024;
+    return hipSuccess;
+}
+// device memory: exact-size heap blocks (the sanitizer guards their ends), counted against the size the device reports
+hipError_t hipMalloc(void **p, size_t n);
+hipError_t hipFree(void *p);
+inline hipError_t hipMemcpy(void *d, const void *s, size_t n, hipMemcpyKind) { memcpy(d, s, n); return hipSuccess; }
+// Work given to a stream runs at once -- or, while the stream is being captured, is recorded for the graph's replays.
+namespace emu { bool submit(hipStream_t s, std::function<void()> work); }
+inline hipError_t hipMemcpyAsync(void *d, const void *s, size_t n, hipMemcpyKind, hipStream_t st) {
+    emu::submit(st, [=] { memmove(d, s, n); });
+    return hipSuccess;
+}
+inline hipError_t hipMemsetAsync(void *d, int v, size_t n, hipStream_t st) {
+    emu::submit(st, [=] { memset(d, v, n); });
+    return hipSuccess;
+}
+inline hipError_t hipStreamCreate(hipStream_t *s) { *s = (hipStream_t)malloc(1); return hipSuccess; }
+inline hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned) { return hipStreamCreate(s); }
+inline hipError_t hipStreamDestroy(hipStream_t s) { free(s); return hipSuccess; }
+inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+inline hipError_t hipEventCreate(hipEvent_t *e) { *e = new emu_event(); return hipSuccess; }
+inline hipError_t hipEventDestroy(hipEvent_t e) { delete e; return hipSuccess; }
+inline hipError_t hipEventRecord(hipEvent_t e, hipStream_t) { e->at = std::chrono::steady_clock::now(); return hipSuccess; }
+inline hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
+inline hipError_t hipEventElapsedTime(float *ms, hipEvent_t a, hipEvent_t b) {
+    *ms = std::chrono::duration<float, std::milli>(b->at - a->at).count();
+    return hipSuccess;
+}
+template <class F> inline hipError_t hipFuncSetAttribute(F, int, int) { return hipSuccess; }
+// captured graphs: the list of work recorded between begin and end; a launch of the graph runs the list again
+hipError_t hipStreamBeginCapture(hipStream_t s, int mode);
+hipError_t hipStreamEndCapture(hipStream_t s, hipGraph_t *g);
+hipError_t hipGraphInstantiate(hipGraphExec_t *e, hipGraph_t g, void *, void *, size_t);
+hipError_t hipGraphLaunch(hipGraphExec_t e, hipStream_t s);
+hipError_t hipGraphDestroy(hipGraph_t g);
+hipError_t hipGraphExecDestroy(hipGraphExec_t e);
+
+// kernel<<<grid, block, lds, stream>>>(args) of the sources, rewritten by tests/emu/build_emulated.py: runs the grid to its
+// end before it returns (arguments are taken by value, as a launch takes them); a stall -- a barrier that not every
+// thread reaches -- is reported as a failed launch
+inline emu::Idx3 emu_idx3(dim3 d) { return emu::Idx3{ d.x, d.y, d.z }; }
+#define EMU_LAUNCH(kernel, grid, block, lds, stream, ...)                                                                   \
+    do {                                                                                                                    \
+        const emu::Idx3 emu_g = emu_idx3(dim3(grid)), emu_b = emu_idx3(dim3(block));                                        \
+        const size_t emu_l = (size_t)(lds);                                                                                 \
+        emu::submit(stream, [=] {                                                                                           \
+            if (!emu::launch3(emu_g, emu_b, emu_l, [=] { kernel(__VA_ARGS__); })) emu::last_error() = hipErrorLaunchFailure; \
+        });                                                                                                                 \
+    } while (0)
+
 
 #define threadIdx (emu::tid())
 #define blockIdx (emu::bid())
@@ -70,6 +161,7 @@ inline int __float_as_int(float f) { int i; std::memcpy(&i, &f, 4); return i; }
 inline float __int_as_float(int i) { float f; std::memcpy(&f, &i, 4); return f; }
 inline float __uint_as_float(unsigned i) { float f; std::memcpy(&f, &i, 4); return f; }
 inline int __float2int_rn(float f) { return (int)std::nearbyintf(f); }
+inline int __mul24(int a, int b) { return (int)((unsigned)((a << 8) >> 8) * (unsigned)((b << 8) >> 8)); }     // v_mul_i32_i24
 using std::max;
 using std::min;
 inline void sincosf_emu(float a, float *s, float *c) { *s = std::sin(a); *c = std::cos(a); }
@@ -129,7 +221,7 @@ inline short emu_bload16(emu_buffer_rsrc r, unsigned voff, unsigned soff) { shor
 #define __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, aux) emu_bload32(r, voff, soff)
 #define __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, aux) emu_bload16(r, voff, soff)
 #define __builtin_amdgcn_s_sleep(n) emu::spin_yield()
-#define __builtin_amdgcn_s_waitcnt(n) ((void)0)
+#define __builtin_amdgcn_s_waitcnt(n) emu::uniform_point()     // nothing to wait for; see uniform_point
 
 // ---- device-scope atomics: fibers never run concurrently, plain accesses are exact
 #define __HIP_MEMORY_SCOPE_AGENT 0
@@ -139,3 +231,104 @@ template <class T> inline T emu_fetch_add(T *p, T v) { T o = *p; *p = o + v; ret
 #define __hip_atomic_load(p, order, scope) emu_atomic_load(p)
 #define __hip_atomic_store(p, v, order, scope) emu_atomic_store(p, v)
 #define __hip_atomic_fetch_add(p, v, order, scope) emu_fetch_add(p, v)
+
+// ---- workgroup / wave barriers and fences.  The lanes of a wave run one after the other here, in lockstep on the
+// device: where a wave's lanes hand data to one another through LDS without a workgroup barrier, the sources mark the
+// point with a wave barrier, and the emulation makes it a rendezvous of the wave's lanes.
+inline void emu_wave_sync() { (void)emu::wave_exchange(0u, emu::lane_id()); }
+#define __builtin_amdgcn_s_barrier() emu::sync_threads()
+#define __builtin_amdgcn_wave_barrier() emu_wave_sync()
+#define __builtin_amdgcn_fence(order, scope) ((void)0)
+#define __builtin_amdgcn_sched_barrier(mask) ((void)0)
+inline void __threadfence() {}
+
+// ---- matrix-core operations: the 64 lanes deposit their A and B registers, each lane then works out its own part of D.
+// v_mfma_i32_16x16x32_i8: lane l holds A[l % 16][8 (l / 16) .. +7] and B[8 (l / 16) .. +7][l % 16] as eight int8;
+// D register r of lane l is D[4 (l / 16) + r][l % 16].
+typedef int emu_i32x4 __attribute__((ext_vector_type(4)));
+typedef float emu_f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 emu_f16x8 __attribute__((ext_vector_type(8)));
+inline emu_i32x4 emu_mfma_i32_16x16x32_i8(long a, long b, emu_i32x4 c) {
+    struct { long a, b; } mine{ a, b };
+    const auto *all = static_cast<const decltype(mine) *>(emu::wave_gather(&mine, sizeof mine));
+    const int l = emu::lane_id(), col = l % 16;
+    for (int r = 0; r < 4; r++) {
+        const int row = 4 * (l / 16) + r;
+        int acc = c[r];
+        for (int kb = 0; kb < 4; kb++) {
+            const long av = all[16 * kb + row].a, bv = all[16 * kb + col].b;
+            for (int j = 0; j < 8; j++) acc += (int)(int8_t)(av >> (8 * j)) * (int)(int8_t)(bv >> (8 * j));
+        }
+        c[r] = acc;
+    }
+    return c;
+}
+#define __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, c, cbsz, abid, blgp) emu_mfma_i32_16x16x32_i8(a, b, c)
+// v_mfma_f32_32x32x16_f16: lane l holds A[l % 32][8 (l / 32) .. +7] and B[8 (l / 32) .. +7][l % 32] as eight halves;
+// D register r of lane l is D[8 (r / 4) + 4 (l / 32) + r % 4][l % 32].  Products are exact in f32; the sum is taken in
+// double and rounded once (the hardware's own order of additions is not specified).
+inline emu_f32x16 emu_mfma_f32_32x32x16_f16(emu_f16x8 a, emu_f16x8 b, emu_f32x16 c) {
+    struct { emu_f16x8 a, b; } mine{ a, b };
+    const auto *all = static_cast<const decltype(mine) *>(emu::wave_gather(&mine, sizeof mine));
+    const int l = emu::lane_id(), col = l % 32;
+    for (int r = 0; r < 16; r++) {
+        const int row = 8 * (r / 4) + 4 * (l / 32) + r % 4;
+        double acc = c[r];
+        for (int kb = 0; kb < 2; kb++)
+            for (int j = 0; j < 8; j++) acc += (double)((float)all[32 * kb + row].a[j] * (float)all[32 * kb + col].b[j]);
+        c[r] = (float)acc;
+    }
+    return c;
+}
+#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, cbsz, abid, blgp) emu_mfma_f32_32x32x16_f16(a, b, c)
+
+// ---- LDS by 32-bit address (hand-written LDS traffic) and loads that land in LDS: addresses are the low half of the
+// host address of the launch-sized LDS buffer, and every access is checked against that buffer
+inline char *emu_lds_at(uint32_t addr, size_t bytes) {
+    char *base = static_cast<char *>(emu::dyn_lds());
+    const uintptr_t host = ((uintptr_t)base & ~(uintptr_t)0xFFFFFFFFu) | addr;
+    if (host < (uintptr_t)base || host + bytes > (uintptr_t)base + emu::dyn_lds_bytes()) {
+        fprintf(stderr, "emu: LDS access of %zu bytes at offset %ld outside the launch's %zu bytes\n", bytes, (long)(host - (uintptr_t)base), emu::dyn_lds_bytes());
+        abort();
+    }
+    return reinterpret_cast<char *>(host);
+}
+inline void emu_global_load_lds(const void *g, void *lds_wave_base, unsigned size, unsigned offset) {
+    char *dst = static_cast<char *>(lds_wave_base) + offset + (size_t)emu::lane_id() * size;     // lanes land side by side
+    char *base = static_cast<char *>(emu::dyn_lds());
+    if (dst < base || dst + size > base + emu::dyn_lds_bytes()) { fprintf(stderr, "emu: load-to-LDS outside the launch's LDS\n"); abort(); }
+    memcpy(dst, g, size);
+}
+#define __builtin_amdgcn_global_load_lds(g, l, size, offset, aux) emu_global_load_lds((const void *)(g), (void *)(l), size, offset)
+
+// ---- inline assembly of the sources, rewritten by tests/emu/build_emulated.py into emu_asm(template, operands...):
+// outputs first, then inputs, as the template numbers them
+struct emu_operand {
+    void *out;                     // where an output goes (null for an input)
+    alignas(16) char value[16];    // an input's value
+    size_t size;
+};
+template <class T> inline emu_operand emu_out(T &v) { emu_operand o{ &v, {}, sizeof(T) }; memcpy(o.value, &v, sizeof(T) < 16 ? sizeof(T) : 16); return o; }
+template <class T> inline emu_operand emu_in(const T &v) { static_assert(sizeof(T) <= 16, ""); emu_operand o{ nullptr, {}, sizeof(T) }; memcpy(o.value, &v, sizeof(T)); return o; }
+inline uint64_t emu_u64(const emu_operand &o) { uint64_t v = 0; memcpy(&v, o.value, o.size < 8 ? o.size : 8); return v; }
+inline void emu_asm_run(const char *t, emu_operand *op, int n) {
+    auto is = [&](const char *m) { return strncmp(t, m, strlen(m)) == 0; };
+    if (t[0] == 0) return;                                                                        // a register pin
+    if (is("global_load_dwordx4")) { memcpy(op[0].out, (const void *)emu_u64(op[1]), 16); return; }
+    if (is("global_load_ushort")) { uint16_t h; memcpy(&h, (const void *)emu_u64(op[1]), 2); uint32_t w = h; memcpy(op[0].out, &w, 4); return; }
+    // hand-written LDS traffic: a wave's LDS instructions execute in order for all its lanes at once, and the sources rely
+    // on that (a wave writes a tile and reads it back transposed with no barrier between), so each one is a rendezvous
+    if (is("ds_")) emu_wave_sync();
+    if (is("ds_read_b128")) { memcpy(op[0].out, emu_lds_at((uint32_t)emu_u64(op[1]) + (uint32_t)emu_u64(op[2]), 16), 16); return; }
+    if (is("ds_read_b32")) { memcpy(op[0].out, emu_lds_at((uint32_t)emu_u64(op[1]) + (uint32_t)emu_u64(op[2]), 4), 4); return; }
+    if (is("ds_write_b128")) { memcpy(emu_lds_at((uint32_t)emu_u64(op[0]) + (uint32_t)emu_u64(op[2]), 16), op[1].value, 16); return; }
+    if (is("ds_write_b32")) { memcpy(emu_lds_at((uint32_t)emu_u64(op[0]) + (uint32_t)emu_u64(op[2]), 4), op[1].value, 4); return; }
+    if (is("v_and_or_b32")) { uint32_t r = ((uint32_t)emu_u64(op[1]) & (uint32_t)emu_u64(op[2])) | (uint32_t)emu_u64(op[3]); memcpy(op[0].out, &r, 4); return; }
+    if (is("v_mov_b32")) { const char *c = strrchr(t, ','); uint32_t r = (uint32_t)strtoul(c + 1, nullptr, 0); memcpy(op[0].out, &r, 4); return; }
+    fprintf(stderr, "emu: no emulation of the instruction \"%s\" (%d operands)\n", t, n);
+    abort();
+}
+template <class... Ops> inline void emu_asm(const char *t, Ops... ops) {
+    emu_operand op[sizeof...(Ops) + 1] = { ops... };
+    emu_asm_run(t, op, (int)sizeof...(Ops));
+}

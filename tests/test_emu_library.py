@@ -1,0 +1,40 @@
+"""The library's own sources built as host C++ (tests/emu/build_emulated.py: every GPU thread a fiber, device memory as
+exact-size heap blocks, AddressSanitizer on) and a selection of the GPU tests run against that build, through the same
+C-ABI and the same Python layer.  What it adds to the GPU run: an access outside a buffer, a barrier that not every
+thread reaches or a host-side sizing mistake stops this run with a report; on the device it would be a fault.  What it
+does not show: timing, and anything that depends on how the hardware interleaves waves.
+
+The selection keeps to sizes a CPU finishes in a few minutes; `python tests/emu/build_emulated.py OUT_DIR --pytest ...`
+runs any other GPU test the same way."""
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parents[1]
+sys.path.insert(0, str(ROOT / "tests" / "emu"))
+import build_emulated  # noqa: E402
+
+SELECTION = [
+    "tests/test_gpu_ops.py",
+    "tests/test_gpu_dequant.py",
+    "tests/test_gpu_failures.py",
+    "tests/test_gpu_gemv.py::test_gemv_edge_inputs",
+    "tests/test_gpu_gemv.py::test_device_pointer_form_and_errors",
+    "tests/test_gpu_gemv.py::test_dense_matmul_f32_kat",
+    "tests/test_gpu_gemv.py::test_dense_matmul_on_resident_buffers_and_batches",
+]
+
+
+@pytest.mark.skipif(not (Path(build_emulated.CLANG).exists() and shutil.which("gcc")), reason="needs ROCm's clang++ and gcc")
+def test_gpu_tests_pass_on_the_emulated_library_under_asan(tmp_path):
+    so = build_emulated.build(tmp_path / "emulated")
+    r = subprocess.run([sys.executable, "-u", "-m", "pytest", *SELECTION, "-m", "gpu", "-x", "-q", "-n", "4", "-p", "no:cacheprovider"],
+                       cwd=ROOT, env=build_emulated.environment(so), capture_output=True, text=True, timeout=1500)
+    tail = r.stdout[-4000:] + r.stderr[-4000:]
+    assert "AddressSanitizer" not in r.stdout + r.stderr, tail
+    assert r.returncode == 0, tail
+    assert " passed" in r.stdout and "failed" not in r.stdout, tail
