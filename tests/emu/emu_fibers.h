@@ -275,7 +275,9 @@ bool launch3(Idx3 grid, Idx3 block, size_t lds_bytes, std::function<void()> kern
     g_kernel = std::move(kernel);
     g_bdim = block;
     g_gdim = grid;
-    g_lds.assign(lds_bytes, 0);   // a heap buffer of exactly the launch's size: overruns are caught
+    // a heap buffer of exactly the launch's size: overruns are caught; LDS comes up undefined on the device, so it is
+    // filled with NaN patterns here and a kernel that reads what it never wrote does not pass its test by luck
+    g_lds.assign(lds_bytes, (char)0xFF);
     const size_t n_blocks = (size_t)grid.x * grid.y * grid.z;
     g_blocks.assign(n_blocks, Block());
     for (size_t bi = 0; bi < n_blocks; bi++)

@@ -38,7 +38,7 @@ inline float4 make_float4(float x, float y, float z, float w) { return float4{ x
 struct dim3 { unsigned x = 1, y = 1, z = 1; dim3() {} dim3(unsigned a, unsigned b = 1, unsigned c = 1) : x(a), y(b), z(c) {} };
 
 typedef int hipError_t;
-enum { hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2, hipErrorInvalidDevice = 101, hipErrorNotSupported = 801, hipErrorLaunchFailure = 719 };
+enum { hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2, hipErrorInvalidDevice = 101, hipErrorInvalidSymbol = 13, hipErrorNotSupported = 801, hipErrorLaunchFailure = 719 };
 inline const char *hipGetErrorString(hipError_t e) {
     return e == hipSuccess ? "no error" : (e == hipErrorNotSupported ? "not supported by the emulation" : (e == hipErrorLaunchFailure ? "emulated launch stalled" : "emulated HIP error"));
 }
@@ -126,6 +126,9 @@ inline hipError_t hipEventElapsedTime(float *ms, hipEvent_t a, hipEvent_t b) {
     return hipSuccess;
 }
 template <class F> inline hipError_t hipFuncSetAttribute(F, int, int) { return hipSuccess; }
+// a __device__ variable is a host global here: its address is its own
+#define HIP_SYMBOL(x) (x)
+template <class T> inline hipError_t hipGetSymbolAddress(void **p, T &symbol) { *p = (void *)&symbol; return hipSuccess; }
 // captured graphs: the list of work recorded between begin and end; a launch of the graph runs the list again
 hipError_t hipStreamBeginCapture(hipStream_t s, int mode);
 hipError_t hipStreamEndCapture(hipStream_t s, hipGraph_t *g);
