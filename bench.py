@@ -265,6 +265,24 @@ def bench_prefill(ex, reps=20):
     return out
 
 
+def bench_dense_f32(ex, reps=5):
+    """The dense f32 product on resident buffers (the executor the reference's unquantized callers use): 2 m n k flops against
+    the f32 matrix-core peak.  Not a benchmark configuration; reported beside the others."""
+    from rustorch_amd import synth
+    F32_PEAK = 157.3e12
+    out = []
+    for m, n, k in ((4096, 4096, 4096), (512, 4096, 4096), (512, 11008, 4096)):
+        a = ex.to_device(synth.normal(SEED, 7300 + m, m * k)); b = ex.to_device(synth.normal(SEED, 7301 + n, k * n))
+        c = ex.buffer(4 * m * n)
+        ex.matmul_f32_dev(a, b, c, m, n, k)
+        ms = timed_regions(ex, lambda: [ex.matmul_f32_dev(a, b, c, m, n, k) for _ in range(reps)])[0] / reps
+        flops = 2.0 * m * n * k
+        out.append({"m": m, "n": n, "k": k, "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "mfma_f32_frac": round(flops / (ms * 1e-3) / F32_PEAK, 4)})
+        for buf in (a, b, c):
+            buf.free()
+    return out
+
+
 def cpu_baseline(reps, gpu_results=None):
     """Reference CPU path for one layer: dequantize each tensor to dense f32, then x . W^T with sequential k-sums.
     With `gpu_results` (what the benchmarked launch left for this layer) also the correctness gate of the timing: the
@@ -370,6 +388,7 @@ def main():
         out["prefill"] = bench_prefill(ex)
         out["batch8"] = bench_batch8(ex)
         out["layer_batch8"] = bench_layer_batch8(ex)
+        out["dense_f32"] = bench_dense_f32(ex)
     if not args.no_decode:
         out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen, args.decode_shape)
     ex.close()

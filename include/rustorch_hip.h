@@ -126,7 +126,10 @@ RT_HIP_API int rt_hip_matmul_f32(rt_hip_ctx *ctx, const float *a, const float *b
 /* The same product on resident buffers (the GpuBuffer idiom, src/gpu/memory_ops/buffer.rs:22-48), enqueue only, and for a
  * batch of products laid out one after the other: c_dev[i] = a_dev[i] . b_dev[i], i < batch -- what
  * GpuLinearAlgebra::{gpu_matmul, gpu_batch_matmul, gpu_matvec} (src/gpu/matrix_ops.rs:562-595) and
- * GpuBatchMatrixExecutor::batch_matmul (:308-343) ask of a device; a matrix-vector product is n = 1. */
+ * GpuBatchMatrixExecutor::batch_matmul (:308-343) ask of a device; a matrix-vector product is n = 1.
+ * Both forms run the f32 matrix-core kernel when m, n >= 64, k >= 16, n and k are multiples of 4 and the bases are
+ * 16-byte aligned (f32 in, f32 accumulate; the order of the k additions is the hardware's), and a plain tiled kernel
+ * that adds k in ascending order otherwise. */
 RT_HIP_API int rt_hip_matmul_f32_dev(rt_hip_ctx *ctx, const float *a_dev, const float *b_dev, float *c_dev, size_t m,
                                      size_t n, size_t k, size_t batch);
 

@@ -647,7 +647,8 @@ __global__ void step_advance_kernel(int *pos_dev, int *token_dev, const int *pic
 }
 
 // Dense row-major f32 C[m,n] = A[m,k] . B[k,n], 32x32 tiles through LDS, k summed in ascending order; grid.z walks a batch
-// of such products laid out one after the other (batch_matmul: src/gpu/matrix_ops.rs:308-343).
+// of such products laid out one after the other (batch_matmul: src/gpu/matrix_ops.rs:308-343).  The kernel of small and
+// odd-shaped products; larger ones go to the matrix cores (below).
 __global__ __launch_bounds__(1024) void matmul_f32_kernel(const float *a, const float *b, float *c, size_t m, size_t n,
                                                           size_t k) {
     __shared__ float as[32][33];
@@ -666,6 +667,89 @@ __global__ __launch_bounds__(1024) void matmul_f32_kernel(const float *a, const 
         __syncthreads();
     }
     if (row < m && col < n) c[row * n + col] = acc;
+}
+
+// The same product on the matrix cores, for operands whose rows are whole 16-byte pieces (n % 4 == 0, k % 4 == 0, 16-byte
+// aligned bases): v_mfma_f32_32x32x2f32, f32 in and out.  Workgroup = 4 waves = a 128 x 128 tile of C, a wave a 64 x 64
+// quarter of it as 2 x 2 blocks of 32 x 32 (64 accumulator registers).  k goes by in slices of 16 through a double-buffered
+// LDS pair: A transposed to [k][m] (rows padded to 132 floats: a lane reads 32 consecutive m of one k), B as it lies,
+// [k][n].  The slice after the current one is in flight in registers while the 32 matrix instructions of the current one
+// run; a slice is 16 KB of global reads per 128 x 128 x 16 x 2 flop, so the kernel is bound by the matrix pipe
+// (157 TFLOP/s dense f32), not by HBM.  Lane l of a wave gives A[l % 32][l / 32] and B[l / 32][l % 32] of a k pair;
+// accumulator r holds C[8 (r / 4) + 4 (l / 32) + r % 4][l % 32] of the block.  Rows and columns past the matrix are
+// loaded as zeros and not stored.
+typedef float float16v __attribute__((ext_vector_type(16)));
+constexpr int kMmTile = 128, kMmK = 16, kMmLda = kMmTile + 4;
+__global__ __launch_bounds__(256) void matmul_f32_mfma_kernel(const float *a, const float *b, float *c, size_t m, size_t n, size_t k) {
+    __shared__ __align__(16) float as[2][kMmK][kMmLda];
+    __shared__ __align__(16) float bs[2][kMmK][kMmTile];
+    a += (size_t)blockIdx.z * m * k;
+    b += (size_t)blockIdx.z * k * n;
+    c += (size_t)blockIdx.z * m * n;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, l32 = lane & 31, lh = lane >> 5;
+    const size_t m0 = (size_t)blockIdx.y * kMmTile, n0 = (size_t)blockIdx.x * kMmTile;
+    float16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    // a thread's two 16-byte pieces of each operand's slice: A piece (row, 4 k), B piece (k row, 4 columns)
+    float4 ra[2], rb[2];
+    auto fetch = [&](size_t k0) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            const int idx = tid + 256 * p;
+            const size_t row = m0 + (size_t)(idx >> 2), ka = k0 + 4 * (size_t)(idx & 3);
+            ra[p] = (row < m && ka < k) ? *reinterpret_cast<const float4 *>(a + row * k + ka) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const size_t kb = k0 + (size_t)(idx >> 5), col = n0 + 4 * (size_t)(idx & 31);
+            rb[p] = (kb < k && col < n) ? *reinterpret_cast<const float4 *>(b + kb * n + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto park = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            const int idx = tid + 256 * p, row = idx >> 2, kq = 4 * (idx & 3);
+            as[buf][kq + 0][row] = ra[p].x;
+            as[buf][kq + 1][row] = ra[p].y;
+            as[buf][kq + 2][row] = ra[p].z;
+            as[buf][kq + 3][row] = ra[p].w;
+            *reinterpret_cast<float4 *>(&bs[buf][idx >> 5][4 * (idx & 31)]) = rb[p];
+        }
+    };
+    fetch(0);
+    park(0);
+    __syncthreads();
+    int buf = 0;
+    for (size_t k0 = 0; k0 < k; k0 += kMmK) {
+        const bool more = k0 + kMmK < k;
+        if (more) fetch(k0 + kMmK);
+#pragma unroll
+        for (int kp = 0; kp < kMmK / 2; kp++) {
+            const int kk = 2 * kp + lh;
+            const float a0 = as[buf][kk][wm * 64 + l32], a1 = as[buf][kk][wm * 64 + 32 + l32];
+            const float b0 = bs[buf][kk][wn * 64 + l32], b1 = bs[buf][kk][wn * 64 + 32 + l32];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+        if (more) park(buf ^ 1);      // the other buffer: its last readers passed the barrier at the end of the previous slice
+        __syncthreads();
+        buf ^= 1;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const size_t col = n0 + (size_t)(wn * 64 + j * 32 + l32);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const size_t row = m0 + (size_t)(wm * 64 + i * 32 + 8 * (r / 4) + 4 * lh + r % 4);
+                if (row < m && col < n) c[row * n + col] = acc[i][j][r];
+            }
+        }
 }
 
 // Per-tensor affine int8 matmul (QuantizedOps::qmatmul, src/quantization/operations.rs:195-260):
@@ -911,6 +995,14 @@ hipError_t launch_embed_rows(hipStream_t s, int type, const uint8_t *w, size_t r
 hipError_t launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *c, size_t m, size_t n, size_t k, size_t batch) {
     if (m == 0 || n == 0 || batch == 0) return hipSuccess;
     if (batch > 65535 || (m + 31) / 32 > 65535) return hipErrorInvalidValue;
+    // the matrix cores take products large enough to fill tiles and laid out in whole 16-byte pieces; the rest (the
+    // reference's 2 x 2 known answer, odd widths, matrix-vector products) goes through the plain kernel
+    const bool pieces = n % 4 == 0 && k % 4 == 0 && (((uintptr_t)a | (uintptr_t)b) & 15) == 0;
+    if (pieces && m >= 64 && n >= 64 && k >= kMmK) {
+        dim3 grid((unsigned)((n + kMmTile - 1) / kMmTile), (unsigned)((m + kMmTile - 1) / kMmTile), (unsigned)batch);
+        matmul_f32_mfma_kernel<<<grid, 256, 0, s>>>(a, b, c, m, n, k);
+        return hipGetLastError();
+    }
     dim3 grid((unsigned)((n + 31) / 32), (unsigned)((m + 31) / 32), (unsigned)batch);
     matmul_f32_kernel<<<grid, dim3(32, 32), 0, s>>>(a, b, c, m, n, k);
     return hipGetLastError();

@@ -285,6 +285,21 @@ inline emu_f32x16 emu_mfma_f32_32x32x16_f16(emu_f16x8 a, emu_f16x8 b, emu_f32x16
 }
 #define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, cbsz, abid, blgp) emu_mfma_f32_32x32x16_f16(a, b, c)
 
+// v_mfma_f32_32x32x2f32: lane l holds A[l % 32][l / 32] and B[l / 32][l % 32]; D as for the other 32 x 32 shapes
+inline emu_f32x16 emu_mfma_f32_32x32x2f32(float a, float b, emu_f32x16 c) {
+    struct { float a, b; } mine{ a, b };
+    const auto *all = static_cast<const decltype(mine) *>(emu::wave_gather(&mine, sizeof mine));
+    const int l = emu::lane_id(), col = l % 32;
+    for (int r = 0; r < 16; r++) {
+        const int row = 8 * (r / 4) + 4 * (l / 32) + r % 4;
+        float acc = c[r];
+        for (int kb = 0; kb < 2; kb++) acc = fmaf(all[32 * kb + row].a, all[32 * kb + col].b, acc);
+        c[r] = acc;
+    }
+    return c;
+}
+#define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, cbsz, abid, blgp) emu_mfma_f32_32x32x2f32(a, b, c)
+
 // ---- LDS by 32-bit address (hand-written LDS traffic) and loads that land in LDS: addresses are the low half of the
 // host address of the launch-sized LDS buffer, and every access is checked against that buffer
 inline char *emu_lds_at(uint32_t addr, size_t bytes) {

@@ -33,6 +33,7 @@ SELECTION = [
     "tests/test_gpu_gemv.py::test_device_pointer_form_and_errors",
     "tests/test_gpu_gemv.py::test_dense_matmul_f32_kat",
     "tests/test_gpu_gemv.py::test_dense_matmul_on_resident_buffers_and_batches",
+    "tests/test_gpu_gemv.py::test_dense_matmul_on_the_matrix_cores",
     "tests/test_gpu_gemv.py::test_batches_of_two_to_eight_on_the_matrix_cores[37-256-12]",
     "tests/test_gpu_gemv.py::test_batches_of_two_to_eight_on_the_matrix_cores[16-768-14]",
     "tests/test_gpu_gemv.py::test_batches_of_two_to_eight_on_the_matrix_cores[1-4096-12]",
