@@ -195,10 +195,14 @@ def environment(so: Path) -> dict:
 
 if __name__ == "__main__":
     if len(sys.argv) < 2:
-        sys.exit("usage: python tests/emu/build_emulated.py OUT_DIR [--pytest PYTEST_ARGS...]\n"
-                 "  builds the emulated library into OUT_DIR; with --pytest, then runs `pytest -m gpu PYTEST_ARGS` against it")
-    lib = build(Path(sys.argv[1]), verbose="--pytest" not in sys.argv)
+        sys.exit("usage: python tests/emu/build_emulated.py OUT_DIR [--pytest PYTEST_ARGS... | --run SCRIPT ARGS...]\n"
+                 "  builds the emulated library into OUT_DIR; with --pytest, then runs `pytest -m gpu PYTEST_ARGS` against it;\n"
+                 "  with --run, a Python script (tests/emu/fuzz_shapes.py for one)")
+    lib = build(Path(sys.argv[1]), verbose="--pytest" not in sys.argv and "--run" not in sys.argv)
     print(lib)
+    if "--run" in sys.argv:
+        args = sys.argv[sys.argv.index("--run") + 1:]
+        sys.exit(subprocess.run([sys.executable, "-u", *args], cwd=ROOT, env=environment(lib)).returncode)
     if "--pytest" in sys.argv:
         args = sys.argv[sys.argv.index("--pytest") + 1:]
         sys.exit(subprocess.run([sys.executable, "-u", "-m", "pytest", "-m", "gpu", *args], cwd=ROOT, env=environment(lib)).returncode)
