@@ -147,13 +147,18 @@ __global__ __launch_bounds__(64 * kAttnWaves) void attn_causal_kernel(const floa
             mt = fmaxf(mt, s[r]);
         }
         mt = fmaxf(mt, __shfl_xor(mt, 32));
-        const float m_new = fmaxf(m_run, mt);                 // finite from the first tile on: key 0 is visible to every query
-        const float alpha = expf(m_run - m_new);
+        // Finite from wave 0's first tile on (key 0 is visible to every query), but not in every wave: with pos0 off a
+        // multiple of 32 the first tile of a later wave can lie wholly beyond an early query.  Such a query keeps
+        // max = -inf, sum = 0 and a zero accumulator in that wave (exp(-inf - (-inf)) would make them NaN), and the
+        // fold below gives the wave the factor 0.
+        const float m_new = fmaxf(m_run, mt);
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = expf(m_run - m_ref);
         float psum = 0.f;
         half8v phi[2], plo[2];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const float p = expf(s[r] - m_new);
+            const float p = expf(s[r] - m_ref);
             psum += p;
             const float ps = p * 16384.0f;
             const _Float16 hi = (_Float16)ps;

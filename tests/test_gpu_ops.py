@@ -69,7 +69,10 @@ def test_kv_append_and_attention(ex, orc):
 
 
 @pytest.mark.parametrize("nh,nkv,hd,pos0,m", [(4, 4, 64, 0, 37), (32, 32, 128, 0, 70), (8, 2, 128, 100, 45), (2, 1, 128, 1000, 33),
-                                               (6, 3, 64, 31, 1), (3, 3, 128, 0, 129)])
+                                               (6, 3, 64, 31, 1), (3, 3, 128, 0, 129),
+                                               # a batch that starts off a multiple of 32 among the first positions: the first tile
+                                               # of a later wave lies wholly beyond the early queries
+                                               (1, 1, 64, 24, 28), (6, 3, 128, 23, 41), (2, 2, 128, 3, 48), (4, 2, 64, 1, 95)])
 def test_causal_attention_of_a_batch(ex, orc, nh, nkv, hd, pos0, m):
     """Row i of the batch (position pos0 + i) against the single-query oracle over cache rows [0, pos0 + i]."""
     from rustorch_amd import synth
