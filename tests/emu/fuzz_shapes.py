@@ -17,7 +17,8 @@ from rustorch_amd.executor import HipKernelExecutor
 
 TYPES = [0, 1, 2, 3, 6, 7, 8, 9, 10, 11, 12, 13, 14]
 BLOCK = {0: 1, 1: 1, 2: 32, 3: 32, 6: 32, 7: 32, 8: 32, 9: 32, 10: 256, 11: 256, 12: 256, 13: 256, 14: 256}
-TOL = 2e-5            # of ||w_row|| ||x||: what the GEMV tests hold the kernels to
+TOL = 2e-5            # of ||w_row|| ||x||: what the GEMV tests hold the kernels to at the benchmark's row lengths
+TOL_SHORT = 6e-5      # rows of a few blocks: one element's 15-bit rounding is not averaged away (the benchmark's bound is 1e-3)
 TOL_GEMM = 3e-4       # the fp16 contractions (the emulation rounds after every fp16 operation)
 
 
@@ -39,7 +40,7 @@ def gemv_case(ex, rng, i):
     y = np.atleast_2d(ex.qgemv(w, x if batch > 1 else x[0]))
     y64, wn = orc.qgemv_f64(t, raw, rows, cols, x)
     ratio = np.abs(y - np.atleast_2d(y64)) / (wn[None, :] * np.linalg.norm(x.astype(np.float64), axis=1)[:, None] + 1e-30)
-    assert np.isfinite(y).all() and ratio.max() <= TOL, ratio.max()
+    assert np.isfinite(y).all() and ratio.max() <= (TOL if cols >= 1024 else TOL_SHORT), ratio.max()
     w.free()
 
 
