@@ -1,8 +1,9 @@
 // The decode GEMV's own code path for the four block formats of the benchmark (Q4_K, Q6_K, Q8_0, Q4_0).
 //
-// Same work split, x layout in LDS, dot-product arithmetic and rounding as the general path in
-// rt_gemv_device.h (a row's result is bit-identical whichever of the two computed it), with everything that
-// does not depend on the row taken out of the loop:
+// Same x layout in LDS and the same dot-product arithmetic per unit as the general path in rt_gemv_device.h.  A row of one
+// pass (up to 4096 elements of the K-quants) has the general path's bits; a longer row is the sum, in pass order, of
+// its passes' wave sums (the general path sums each lane's passes first), whichever way the launch deals the passes out.
+// Everything that does not depend on the row is taken out of the loop:
 //   * what a lane needs to decode its unit -- the byte selector of its two 6-bit scales and minima, the
 //     masks of the two packings of a Q4_K header, the scale bytes of its Q6_K runs -- is a lane constant
 //     (a lane's unit index changes by 64 from pass to pass, so u & 3 never changes), and the decode is
