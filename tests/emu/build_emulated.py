@@ -1,5 +1,6 @@
 """Builds the library's own sources as host C++ against the stand-in HIP headers of tests/emu: every GPU thread a fiber,
-every device allocation an exact-size heap block under AddressSanitizer.  TEST INFRASTRUCTURE: the result is loaded by
+every device allocation an exact-size heap block under AddressSanitizer (and the alignment check of the undefined-behaviour
+sanitizer: a 16-byte access through a pointer that is not 16-byte aligned stops the run).  TEST INFRASTRUCTURE: the result is loaded by
 tests only (RUSTORCH_HIP_LIBRARY names it), to run the same tests that run on the GPU -- at small sizes -- where an access
 outside a buffer stops the run with a report instead of faulting a device.
 
@@ -149,7 +150,7 @@ def build(out_dir: Path, verbose: bool = False) -> Path:
     out_dir.mkdir(parents=True, exist_ok=True)
     gen = out_dir / "src"
     gen.mkdir(exist_ok=True)
-    flags = ["-std=c++17", "-O2", "-g", "-fPIC", "-fsanitize=address", "-shared-libasan", "-fno-omit-frame-pointer", "-DRT_EMULATED=1",
+    flags = ["-std=c++17", "-O2", "-g", "-fPIC", "-fsanitize=address,alignment", "-fno-sanitize-recover=alignment", "-shared-libasan", "-fno-omit-frame-pointer", "-DRT_EMULATED=1",
              "-Wno-unknown-attributes", "-Wno-unused-value", "-I", str(EMU), "-I", str(CSRC), "-I", str(ROOT / "include")]
     jobs = []
     for name in SOURCES:
@@ -171,7 +172,7 @@ def build(out_dir: Path, verbose: bool = False) -> Path:
     with ThreadPoolExecutor(max_workers=min(4, os.cpu_count() or 1)) as pool:
         list(pool.map(compile_one, jobs))
     so = out_dir / "librustorch_hip_emulated.so"
-    r = subprocess.run([CLANG, "-shared", "-fsanitize=address", "-shared-libasan", *[str(o) for _, o in jobs], "-o", str(so)], capture_output=True, text=True)
+    r = subprocess.run([CLANG, "-shared", "-fsanitize=address,alignment", "-shared-libasan", *[str(o) for _, o in jobs], "-o", str(so)], capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link of the emulated library failed:\n" + r.stderr[-6000:])
     return so
