@@ -352,6 +352,48 @@ def test_model_in_a_format_without_matrix_core_path(ex, orc, fmt):
     assert np.median(ratios) <= 0.1 and (ratios <= 1).mean() >= 0.9
 
 
+@pytest.mark.parametrize("fmts", [
+    dict(attn_q="Q4_K", attn_k="Q8_0", attn_v="Q6_K", ffn_gate="Q4_K", ffn_up="Q5_K"),      # fused, fp16, fused contraction in one group
+    dict(attn_q="Q5_K", attn_k="Q4_K", attn_v="Q4_K", ffn_gate="Q8_0", ffn_up="Q6_K"),      # fp16 first, then two that share a prepared X
+    dict(attn_q="Q6_K", attn_k="F16", attn_v="Q4_0", attn_output="Q2_K", ffn_down="Q5_1")])
+def test_prefill_with_mixed_formats_inside_a_group(ex, orc, fmts):
+    """The matrices that meet one activation matrix (q / k / v; gate / up) in different formats: some take the fused
+    matrix-core contraction, which shares a prepared copy of X in the workspace, some the fp16 contraction, which uses
+    the same workspace for its own operands.  A batched prefill of 36 tokens has to give what feeding the tokens one by
+    one gives, and both the oracle's logits."""
+    from rustorch_amd import llama, synth, GGMLType
+    cfg = dict(n_layers=2, hidden=512, n_heads=4, ffn=1024, vocab=400, max_pos=40)
+    print("llama mixed formats", fmts, cfg, flush=True)
+    gm = llama.HipLlama(ex, **cfg)
+    om = orc.OracleLlama(**cfg)
+    head = {}
+    for slot, layer, t, r, c, raw in llama.synthetic_tensors(41, cfg["n_layers"], cfg["hidden"], cfg["ffn"], cfg["vocab"]):
+        if slot in fmts:
+            t = getattr(GGMLType, fmts[slot])
+            raw = synth.blocks(t, 41, synth.layer_tid(layer, slot), r, c)
+        gm.upload(slot, layer, t, r, c, raw)
+        om.set_tensor(slot, layer, t, r, c, raw)
+        if slot == "output":
+            head["wn"] = np.linalg.norm(orc.dequant(t, raw, r, c).astype(np.float64), axis=1)
+    toks = synth.tokens(41, synth.TID_PROMPT, 38, cfg["vocab"])
+    want = om.forward(toks, 0)
+    tol = logit_tol(head["wn"], cfg["hidden"])
+    for p, t in enumerate(toks[:36]):
+        gm.step(int(t), p, want_token=False)
+    stepped = gm.logits().copy()
+    gm.reset()
+    gm.prefill(toks[:36], 0)
+    batched = gm.logits().copy()
+    r_step, r_batch = float((np.abs(stepped - want[35]) / tol).max()), float((np.abs(batched - want[35]) / tol).max())
+    between = float((np.abs(batched - stepped) / tol).max())
+    print("position 35, ratio to the tolerance: token by token %.3f, batched %.3f, between the two %.3f" % (r_step, r_batch, between), flush=True)
+    # the fp16 contraction rounds weights and activations to fp16: about half the bound at this size, the fused one a tenth
+    assert np.isfinite(batched).all() and between <= 1.0 and r_batch <= 1.0 and r_step <= 0.2
+    gm.step(int(toks[36]), 36)                                  # the cache the batched pass left serves the next step
+    assert float((np.abs(gm.logits() - want[36]) / tol).max()) <= 1.0
+    gm.close()
+
+
 def test_graph_replay_equals_eager_launches(ex, orc):
     """Mode 2 replays the step from a captured graph.  Every replay is checked against the eager launches of mode 1:
     same kernels, same arguments, so logits and picks are equal bit for bit -- with eager work (a cache reset, a
