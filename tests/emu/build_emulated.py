@@ -146,11 +146,21 @@ def to_host_cpp(src: str) -> str:
     return rewrite_asm(rewrite_launches(src))
 
 
-def build(out_dir: Path, verbose: bool = False) -> Path:
+# The two instrumented builds.  "address": out-of-bounds and misaligned accesses.  "thread": a wave is a thread of the race
+# detector (emu_fibers.h); function entry / exit hooks are off because the 64 lanes of a wave share one detector context
+# while each has a call stack of its own.
+SANITIZERS = {
+    "address": ["-fsanitize=address,alignment", "-fno-sanitize-recover=alignment", "-shared-libasan"],
+    "thread": ["-fsanitize=thread", "-shared-libsan", "-mllvm", "-tsan-instrument-func-entry-exit=0"],
+}
+
+
+def build(out_dir: Path, verbose: bool = False, sanitizer: str = "address") -> Path:
     out_dir.mkdir(parents=True, exist_ok=True)
     gen = out_dir / "src"
     gen.mkdir(exist_ok=True)
-    flags = ["-std=c++17", "-O2", "-g", "-fPIC", "-fsanitize=address,alignment", "-fno-sanitize-recover=alignment", "-shared-libasan", "-fno-omit-frame-pointer", "-DRT_EMULATED=1",
+    san = SANITIZERS[sanitizer]
+    flags = ["-std=c++17", "-O2", "-g", "-fPIC", *san, "-fno-omit-frame-pointer", "-DRT_EMULATED=1",
              "-Wno-unknown-attributes", "-Wno-unused-value", "-I", str(EMU), "-I", str(CSRC), "-I", str(ROOT / "include")]
     jobs = []
     for name in SOURCES:
@@ -162,7 +172,11 @@ def build(out_dir: Path, verbose: bool = False) -> Path:
 
     def compile_one(job):
         src, obj = job
-        cmd = [CLANG, *flags, "-x", "c++", "-c", str(src), "-o", str(obj)]
+        mine = list(flags)
+        if sanitizer == "thread" and src.name == "emu_library.cpp":
+            # the fiber scheduler tells the race detector what it does (EMU_TSAN) but is not itself watched
+            mine = [f for f in mine if f not in san] + ["-DEMU_TSAN=1"]
+        cmd = [CLANG, *mine, "-x", "c++", "-c", str(src), "-o", str(obj)]
         if verbose:
             print("[emu build]", " ".join(cmd), flush=True)
         r = subprocess.run(cmd, capture_output=True, text=True)
@@ -172,38 +186,46 @@ def build(out_dir: Path, verbose: bool = False) -> Path:
     with ThreadPoolExecutor(max_workers=min(4, os.cpu_count() or 1)) as pool:
         list(pool.map(compile_one, jobs))
     so = out_dir / "librustorch_hip_emulated.so"
-    r = subprocess.run([CLANG, "-shared", "-fsanitize=address,alignment", "-shared-libasan", *[str(o) for _, o in jobs], "-o", str(so)], capture_output=True, text=True)
+    r = subprocess.run([CLANG, "-shared", *[f for f in san if not f.startswith("-mllvm") and not f.startswith("-tsan")], *[str(o) for _, o in jobs], "-o", str(so)],
+                       capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link of the emulated library failed:\n" + r.stderr[-6000:])
     return so
 
 
-def asan_runtime() -> str:
-    return subprocess.run([CLANG, "-print-file-name=libclang_rt.asan-x86_64.so"], capture_output=True, text=True, check=True).stdout.strip()
+def sanitizer_runtime(sanitizer: str = "address") -> str:
+    name = {"address": "asan", "thread": "tsan"}[sanitizer]
+    return subprocess.run([CLANG, "-print-file-name=libclang_rt.%s-x86_64.so" % name], capture_output=True, text=True, check=True).stdout.strip()
 
 
-def environment(so: Path) -> dict:
+def environment(so: Path, sanitizer: str = "address") -> dict:
     """The environment of a Python process that is to load the emulated library instead of the GPU one."""
     env = dict(os.environ)
     env["RUSTORCH_HIP_LIBRARY"] = str(so)
     # the sanitizer's runtime has to be in the process before the library is; whatever is preloaded already stays
-    env["LD_PRELOAD"] = ":".join(x for x in (asan_runtime(), env.get("LD_PRELOAD", "")) if x)
+    env["LD_PRELOAD"] = ":".join(x for x in (sanitizer_runtime(sanitizer), env.get("LD_PRELOAD", "")) if x)
     # a fake stack per fiber (the default's use-after-return check) costs more than the kernels themselves
     env["ASAN_OPTIONS"] = "detect_leaks=0:detect_stack_use_after_return=0:verify_asan_link_order=0"
+    # a race is a failure of the run, reported once per place
+    env["TSAN_OPTIONS"] = "halt_on_error=0:exitcode=66:report_signal_unsafe=0:history_size=4"
     env["PYTHONPATH"] = os.pathsep.join(x for x in (str(ROOT), env.get("PYTHONPATH", "")) if x)
     return env
 
 
 if __name__ == "__main__":
     if len(sys.argv) < 2:
-        sys.exit("usage: python tests/emu/build_emulated.py OUT_DIR [--pytest PYTEST_ARGS... | --run SCRIPT ARGS...]\n"
+        sys.exit("usage: python tests/emu/build_emulated.py OUT_DIR [--races] [--pytest PYTEST_ARGS... | --run SCRIPT ARGS...]\n"
+                 "  --races: the ThreadSanitizer build (a wave is a thread: unordered accesses of two waves are reported)\n"
                  "  builds the emulated library into OUT_DIR; with --pytest, then runs `pytest -m gpu PYTEST_ARGS` against it;\n"
                  "  with --run, a Python script (tests/emu/fuzz_shapes.py for one)")
-    lib = build(Path(sys.argv[1]), verbose="--pytest" not in sys.argv and "--run" not in sys.argv)
+    kind = "thread" if "--races" in sys.argv else "address"
+    if "--races" in sys.argv:
+        sys.argv.remove("--races")
+    lib = build(Path(sys.argv[1]), verbose="--pytest" not in sys.argv and "--run" not in sys.argv, sanitizer=kind)
     print(lib)
     if "--run" in sys.argv:
         args = sys.argv[sys.argv.index("--run") + 1:]
-        sys.exit(subprocess.run([sys.executable, "-u", *args], cwd=ROOT, env=environment(lib)).returncode)
+        sys.exit(subprocess.run([sys.executable, "-u", *args], cwd=ROOT, env=environment(lib, kind)).returncode)
     if "--pytest" in sys.argv:
         args = sys.argv[sys.argv.index("--pytest") + 1:]
-        sys.exit(subprocess.run([sys.executable, "-u", "-m", "pytest", "-m", "gpu", *args], cwd=ROOT, env=environment(lib)).returncode)
+        sys.exit(subprocess.run([sys.executable, "-u", "-m", "pytest", "-m", "gpu", *args], cwd=ROOT, env=environment(lib, kind)).returncode)

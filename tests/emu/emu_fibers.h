@@ -19,6 +19,11 @@
 #include <sanitizer/common_interface_defs.h>
 #endif
 #endif
+// EMU_TSAN is given on the command line of the race-detecting build: this file itself is compiled without the
+// instrumentation there (the scheduler's own bookkeeping is touched from every context by design).
+#ifdef EMU_TSAN
+#include <sanitizer/tsan_interface.h>
+#endif
 
 // ------------------------------------------------------------------ fiber runtime
 // The switch between two stacks, written out (x86-64, System V): callee-saved registers on the old stack, stack pointers
@@ -51,6 +56,11 @@ emu_switch_stack:
     .size emu_switch_stack, .-emu_switch_stack
 )");
 
+// the scheduler's own bookkeeping is touched from every context by design: never watched by the race detector, whether
+// this file is compiled into a translation unit with the instrumentation (a self-contained test program) or without
+#ifdef EMU_TSAN
+#pragma clang attribute push(__attribute__((no_sanitize("thread"))), apply_to = function)
+#endif
 namespace emu {
 
 enum State { RUNNABLE, AT_SYNC, AT_WAVE, AT_GATHER, AT_UNIFORM, SPIN, DONE };
@@ -88,6 +98,20 @@ static std::function<void()> g_kernel;
 static long g_switches = 0;
 static std::vector<char *> g_stack_pool;
 
+// Under ThreadSanitizer a wave is a thread of the race detector: its 64 lanes share one context (they run in lockstep
+// on the device, so what one lane writes another may read), different waves of a workgroup are different contexts
+// with no order between them except at a workgroup barrier, and workgroups and launches follow one another.  A
+// write by one wave and an access by another with no barrier between is then reported as a data race.
+#ifdef EMU_TSAN
+static void *g_tsan_main = nullptr;
+static std::vector<void *> g_tsan_wave;
+static char g_tsan_barrier, g_tsan_order;      // addresses the happens-before edges hang on
+static void *tsan_wave(unsigned wave) {
+    while (g_tsan_wave.size() <= wave) g_tsan_wave.push_back(__tsan_create_fiber(0));
+    return g_tsan_wave[wave];
+}
+#endif
+
 Idx3 &tid() { return g_cur->tid; }
 Idx3 &bid() { return g_blocks[(size_t)g_cur->block].bid; }
 Idx3 &bdim() { return g_bdim; }
@@ -98,6 +122,9 @@ int lane_id() { return (int)(g_cur->linear & 63); }
 
 static void to_main() {
     Fiber *f = g_cur;
+#ifdef EMU_TSAN
+    __tsan_switch_to_fiber(g_tsan_main, __tsan_switch_to_fiber_no_sync);
+#endif
 #ifdef EMU_ASAN
     void *fake = nullptr;
     __sanitizer_start_switch_fiber(f->state == DONE ? nullptr : &fake, g_main_bottom, g_main_size);
@@ -108,7 +135,16 @@ static void to_main() {
 #endif
 }
 
-void sync_threads() { g_cur->state = AT_SYNC; to_main(); }
+void sync_threads() {
+#ifdef EMU_TSAN
+    __tsan_release(&g_tsan_barrier);       // every lane arrives before any leaves
+#endif
+    g_cur->state = AT_SYNC;
+    to_main();
+#ifdef EMU_TSAN
+    __tsan_acquire(&g_tsan_barrier);
+#endif
+}
 void spin_yield() { g_cur->state = SPIN; to_main(); }
 uint32_t wave_exchange(uint32_t v, int src) {
     g_cur->xval = v;
@@ -130,7 +166,13 @@ static void fiber_entry() {
 #ifdef EMU_ASAN
     __sanitizer_finish_switch_fiber(nullptr, &g_main_bottom, &g_main_size);
 #endif
+#ifdef EMU_TSAN
+    __tsan_acquire(&g_tsan_order);         // after the host's writes and the workgroups that ran before this one
+#endif
     g_kernel();
+#ifdef EMU_TSAN
+    __tsan_release(&g_tsan_order);
+#endif
     g_cur->state = DONE;
     to_main();
 }
@@ -138,6 +180,9 @@ static void fiber_entry() {
 static void resume(Fiber &f) {
     g_cur = &f;
     g_switches++;
+#ifdef EMU_TSAN
+    __tsan_switch_to_fiber(tsan_wave(f.linear >> 6), __tsan_switch_to_fiber_no_sync);
+#endif
 #ifdef EMU_ASAN
     void *fake = nullptr;
     __sanitizer_start_switch_fiber(&fake, f.stack, kStack);
@@ -167,7 +212,7 @@ static char *take_stack() {
 static void start_block(Block &b, int index) {
     const unsigned n = g_bdim.x * g_bdim.y * g_bdim.z;
     b.fibers.resize(n);
-    b.gather.assign((n + 63) / 64, std::vector<char>());
+    b.gather.assign((n + 63) / 64, std::vector<char>(64 * 64));      // room for 64 bytes per lane, sized here once
     for (unsigned t = 0; t < n; t++) {
         Fiber &f = b.fibers[t];
         f.linear = t;
@@ -182,9 +227,15 @@ static void start_block(Block &b, int index) {
         f.sp = top;
     }
     b.started = true;
+#ifdef EMU_TSAN
+    __tsan_release(&g_tsan_order);         // the lanes read what was set up here (their indices)
+#endif
 }
 
 static void finish_block(Block &b) {
+#ifdef EMU_TSAN
+    __tsan_acquire(&g_tsan_order);         // the host continues after the workgroup's last access (and frees what its lanes read)
+#endif
     for (Fiber &f : b.fibers) g_stack_pool.push_back(f.stack);
     b.fibers.clear();
     b.fibers.shrink_to_fit();
@@ -231,11 +282,17 @@ static bool run_block(Block &b) {
                 size_t bytes = 0;
                 for (size_t i = w0; i < w1; i++)
                     if (b.fibers[i].state == AT_GATHER) bytes = std::max(bytes, b.fibers[i].gbytes);
+                // (byte loops, not memset / memcpy: the race-detecting build intercepts those and would book them as
+                // accesses of the host, while this is the wave handing its own registers round)
                 std::vector<char> &buf = b.gather[w0 / 64];
-                buf.assign(64 * bytes, 0);      // lanes that are not at the operation contribute zeros
+                if (buf.size() < 64 * bytes) buf.resize(64 * bytes);
+                volatile char *dst = buf.data();
+                for (size_t k = 0; k < 64 * bytes; k++) dst[k] = 0;      // lanes that are not at the operation contribute zeros
                 for (size_t i = w0; i < w1; i++) {
                     Fiber &f = b.fibers[i];
-                    if (f.state == AT_GATHER) memcpy(buf.data() + (i - w0) * bytes, f.gmine, f.gbytes);
+                    if (f.state != AT_GATHER) continue;
+                    const volatile char *src = static_cast<const char *>(f.gmine);
+                    for (size_t k = 0; k < f.gbytes; k++) dst[(i - w0) * bytes + k] = src[k];
                 }
                 for (size_t i = w0; i < w1; i++) {
                     Fiber &f = b.fibers[i];
@@ -278,6 +335,10 @@ bool launch3(Idx3 grid, Idx3 block, size_t lds_bytes, std::function<void()> kern
     // a heap buffer of exactly the launch's size: overruns are caught; LDS comes up undefined on the device, so it is
     // filled with NaN patterns here and a kernel that reads what it never wrote does not pass its test by luck
     g_lds.assign(lds_bytes, (char)0xFF);
+#ifdef EMU_TSAN
+    g_tsan_main = __tsan_get_current_fiber();
+    __tsan_release(&g_tsan_order);
+#endif
     const size_t n_blocks = (size_t)grid.x * grid.y * grid.z;
     g_blocks.assign(n_blocks, Block());
     for (size_t bi = 0; bi < n_blocks; bi++)
@@ -307,3 +368,6 @@ bool launch(unsigned grid, unsigned block, size_t lds_bytes, std::function<void(
 }
 
 }  // namespace emu
+#ifdef EMU_TSAN
+#pragma clang attribute pop
+#endif

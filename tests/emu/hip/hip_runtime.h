@@ -207,7 +207,16 @@ inline unsigned emu_perm(unsigned s0, unsigned s1, unsigned sel) {
     return r;
 }
 #define __builtin_amdgcn_perm(a, b, sel) emu_perm(a, b, sel)
-inline void unsafeAtomicAdd(float *p, float v) { *p += v; }
+inline void unsafeAtomicAdd(float *p, float v) {
+    uint32_t seen, want;
+    __atomic_load(reinterpret_cast<uint32_t *>(p), &seen, __ATOMIC_RELAXED);
+    do {
+        float f;
+        memcpy(&f, &seen, 4);
+        f += v;
+        memcpy(&want, &f, 4);
+    } while (!__atomic_compare_exchange(reinterpret_cast<uint32_t *>(p), &seen, &want, false, __ATOMIC_RELAXED, __ATOMIC_RELAXED));
+}
 // buffer resources: base pointer only (the emulation neither checks ranges nor strides), loads at base + voffset + soffset
 struct emu_buffer_rsrc { const unsigned char *base; };
 typedef emu_buffer_rsrc __amdgpu_buffer_rsrc_t;
@@ -226,11 +235,12 @@ inline short emu_bload16(emu_buffer_rsrc r, unsigned voff, unsigned soff) { shor
 #define __builtin_amdgcn_s_sleep(n) emu::spin_yield()
 #define __builtin_amdgcn_s_waitcnt(n) emu::uniform_point()     // nothing to wait for; see uniform_point
 
-// ---- device-scope atomics: fibers never run concurrently, plain accesses are exact
+// ---- device-scope atomics: fibers never run concurrently, so any access would be exact; they go through the
+// compiler's atomics so that the race detector of the ThreadSanitizer build knows them for what they are
 #define __HIP_MEMORY_SCOPE_AGENT 0
-template <class T> inline T emu_atomic_load(const T *p) { return *p; }
-template <class T> inline void emu_atomic_store(T *p, T v) { *p = v; }
-template <class T> inline T emu_fetch_add(T *p, T v) { T o = *p; *p = o + v; return o; }
+template <class T> inline T emu_atomic_load(const T *p) { T v; __atomic_load(p, &v, __ATOMIC_RELAXED); return v; }
+template <class T> inline void emu_atomic_store(T *p, T v) { __atomic_store(p, &v, __ATOMIC_RELAXED); }
+template <class T> inline T emu_fetch_add(T *p, T v) { return __atomic_fetch_add(p, v, __ATOMIC_RELAXED); }
 #define __hip_atomic_load(p, order, scope) emu_atomic_load(p)
 #define __hip_atomic_store(p, v, order, scope) emu_atomic_store(p, v)
 #define __hip_atomic_fetch_add(p, v, order, scope) emu_fetch_add(p, v)
