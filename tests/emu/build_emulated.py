@@ -207,7 +207,7 @@ def environment(so: Path, sanitizer: str = "address") -> dict:
     # a fake stack per fiber (the default's use-after-return check) costs more than the kernels themselves
     env["ASAN_OPTIONS"] = "detect_leaks=0:detect_stack_use_after_return=0:verify_asan_link_order=0"
     # a race is a failure of the run, reported once per place
-    env["TSAN_OPTIONS"] = "halt_on_error=0:exitcode=66:report_signal_unsafe=0:history_size=4"
+    env["TSAN_OPTIONS"] = "halt_on_error=0:exitcode=66:report_signal_unsafe=0:history_size=4:suppressions=%s" % (EMU / "tsan.supp")
     env["PYTHONPATH"] = os.pathsep.join(x for x in (str(ROOT), env.get("PYTHONPATH", "")) if x)
     return env
 

@@ -4,8 +4,6 @@
 // kernel (no barrier time-out, no dead rendezvous), and the logits agree with the CPU oracle.
 //
 // usage: emu_main [n_wg]        (n_wg: number of workgroups, a multiple of 8 and >= n_heads; default 8)
-#include <sys/mman.h>
-#include <ucontext.h>
 
 #include <cstdio>
 #include <cstdlib>

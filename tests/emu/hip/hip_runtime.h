@@ -1,12 +1,14 @@
-// CPU stand-in for <hip/hip_runtime.h>: enough of the HIP device vocabulary to compile the kernels of
-// rustorch_amd/csrc as host C++ and run them as fibers (one per GPU thread) under AddressSanitizer.
-// TEST INFRASTRUCTURE: used only by the programs and the emulated library under tests/emu.
+// CPU stand-in for <hip/hip_runtime.h>: the HIP device vocabulary the sources of rustorch_amd/csrc use (thread indices,
+// LDS, wave operations, matrix-core and LDS-DMA builtins, buffer loads, atomics, the few hand-written instructions) and the
+// part of the host API they call (memory, streams, events, captured graphs), so that the same sources compile as host C++
+// and run under AddressSanitizer or ThreadSanitizer.  TEST INFRASTRUCTURE: used only by the programs and the emulated
+// library under tests/emu.
 //
-// Execution model: a workgroup's threads are fibers that run one after the other; a fiber runs until it
-// reaches __syncthreads(), a wave operation (shuffle / DPP / readlane), a sleep inside a spin loop, or its
-// end.  Workgroups take turns; a workgroup is left only when it is spinning in the grid barrier, at which
-// point its LDS contents are dead, so one LDS buffer serves all workgroups.  Wave operations are executed by
-// whole waves in the kernels here, so they are modelled as a 64-lane rendezvous with value exchange.
+// Execution model (tests/emu/emu_fibers.h): a GPU thread is a fiber; a workgroup's fibers run one after the other, each
+// until it reaches __syncthreads(), a wave operation (shuffle / DPP / readlane / a matrix instruction / a wave barrier /
+// a hand-written LDS instruction / a wait), a sleep inside a spin loop, or its end.  Workgroups run one after the other; a
+// workgroup is left before its end only while it spins on another one (a grid barrier), at which point its LDS contents
+// are dead, so one launch-sized LDS buffer serves all workgroups.  Wave operations are a rendezvous of the wave's lanes.
 #pragma once
 
 #include <algorithm>

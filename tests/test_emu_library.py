@@ -55,3 +55,30 @@ def test_gpu_tests_pass_on_the_emulated_library_under_asan(tmp_path):
     assert "AddressSanitizer" not in r.stdout + r.stderr, tail
     assert r.returncode == 0, tail
     assert " passed" in r.stdout and "failed" not in r.stdout, tail
+
+
+# the race detector's share of the same selection: what passes data between waves through LDS
+RACE_SELECTION = [
+    "tests/test_gpu_ops.py",
+    "tests/test_gpu_gemv.py::test_gemv_edge_inputs",
+    "tests/test_gpu_gemv.py::test_gemv_config_shapes_batch1_and_8[C3_down]",       # rows of three passes dealt out over the waves
+    "tests/test_gpu_gemv.py::test_grouped_launch_equals_single_launches",
+    "tests/test_gpu_gemv.py::test_batches_of_two_to_eight_on_the_matrix_cores[300-11008-14]",
+    "tests/test_gpu_gemv.py::test_dense_matmul_on_the_matrix_cores",
+    "tests/test_gpu_gemm.py::test_single_superblock_odd_counts_and_tiny_matrices",
+    "tests/test_gpu_gemm.py::test_three_to_fifteen_rows_go_eight_at_a_time[100-11008-12]",
+]
+
+
+@pytest.mark.skipif(not (Path(build_emulated.CLANG).exists() and shutil.which("gcc")), reason="needs ROCm's clang++ and gcc")
+def test_gpu_tests_show_no_race_between_waves_on_the_emulated_library(tmp_path):
+    """The same sources under ThreadSanitizer with a wave as a thread of the detector (tests/emu/emu_fibers.h): an access of
+    one wave to what another wrote, with no workgroup barrier between, ends the run with the detector's exit code."""
+    so = build_emulated.build(tmp_path / "emulated", sanitizer="thread")
+    # one process, output not captured by pytest: the detector's reports reach stderr and its exit code is the run's
+    r = subprocess.run([sys.executable, "-u", "-m", "pytest", *RACE_SELECTION, "-m", "gpu", "-x", "-q", "-s", "-p", "no:cacheprovider"],
+                       cwd=ROOT, env=build_emulated.environment(so, "thread"), capture_output=True, text=True, timeout=1500)
+    tail = r.stdout[-4000:] + r.stderr[-4000:]
+    assert "ThreadSanitizer" not in r.stdout + r.stderr, tail
+    assert r.returncode == 0, tail
+    assert " passed" in r.stdout and "failed" not in r.stdout, tail
