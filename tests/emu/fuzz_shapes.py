@@ -4,7 +4,8 @@
     python tests/emu/build_emulated.py OUT_DIR --run tests/emu/fuzz_shapes.py [seed [rounds]]
 
 Each round draws one case of each kind -- a GEMV (any format, 1..8 rows, ragged row counts, rows of one to several
-passes), a grouped launch of several such problems, a prefill contraction (rows on and off the matrix cores, ragged
+passes), a grouped launch of several such problems, several weights against one batch (also from ready-made quantized
+activations), a block decode, the greedy pick, the int8 affine product, a prefill contraction (rows on and off the matrix cores, ragged
 tiles), the dense f32 product, the decode and prefill attention, RMSNorm / SwiGLU / RoPE -- sized so that the emulation
 finishes a round in about a minute.  It prints every case before running it, so the last line names the culprit."""
 import sys
@@ -126,6 +127,58 @@ def small_ops_case(ex, rng, i):
     assert np.allclose(ex.rope(v, nh, hd, pos, 10000.0), orc.rope(v, nh, hd, pos, 10000.0), rtol=1e-4, atol=1e-4)
 
 
+def shared_x_case(ex, rng, i):
+    """Several weights against one batch (the q / k / v and gate / up launches), also from ready-made quantized activations."""
+    cols = 256 * int(rng.integers(1, 12)); batch = int(rng.integers(1, 9)); n = int(rng.integers(1, 8))
+    specs = [(int(rng.choice([12, 14, 8, 2, 13])), int(rng.integers(1, 150))) for _ in range(n)]
+    say("shared-x gemv, %d columns, batch %d:" % (cols, batch), specs)
+    x = synth.normal(600 + i, 1, batch * cols).reshape(batch, cols)
+    dx = ex.to_device(x)
+    ws, ys, raws = [], [], []
+    for j, (t, r) in enumerate(specs):
+        raw = synth.blocks(t, 600 + i, 10 + j, r, cols)
+        raws.append(raw); ws.append(ex.upload_qweight(t, r, cols, raw)); ys.append(ex.buffer(4 * batch * r))
+    ex.qgemv_shared_x_dev(ws, dx, ys, batch)
+    xn = np.linalg.norm(x.astype(np.float64), axis=1)[:, None]
+    for (t, r), raw, y in zip(specs, raws, ys):
+        y64, wn = orc.qgemv_f64(t, raw, r, cols, x)
+        got = y.download(np.float32).reshape(batch, r)
+        assert np.isfinite(got).all() and (np.abs(got - np.atleast_2d(y64)) / (wn[None, :] * xn)).max() <= TOL_SHORT
+    if batch == 1:
+        # the same launch from activations quantized once by their own kernel: one problem per weight
+        xq = ex.buffer(ex.xq_bytes(cols))
+        ex.quantize_act_dev([dx], [cols], [xq])
+        ex.qgemv_xq_grouped_dev(ws, [xq] * n, ys)
+        for (t, r), raw, y in zip(specs, raws, ys):
+            y64, wn = orc.qgemv_f64(t, raw, r, cols, x)
+            got = y.download(np.float32).reshape(1, r)
+            assert (np.abs(got - np.atleast_2d(y64)) / (wn[None, :] * xn)).max() <= TOL_SHORT
+        xq.free()
+    for b in ws + ys + [dx]:
+        b.free()
+
+
+def misc_case(ex, rng, i):
+    t = int(rng.choice(TYPES)); rows = int(rng.integers(1, 40)); cols = cols_for(rng, t)
+    say("dequant type %d, %d x %d" % (t, rows, cols))
+    raw = synth.blocks(t, 700 + i, 1, rows, cols)
+    w = ex.upload_qweight(t, rows, cols, raw)
+    assert np.array_equal(ex.dequant(w).view(np.uint32), orc.dequant(t, raw, rows, cols).view(np.uint32))
+    w.free()
+    n = int(rng.integers(1, 70000))
+    say("argmax over %d" % n)
+    v = synth.normal(700 + i, 2, n)
+    v[int(rng.integers(0, n))] = v.max()              # a tie now and then: the lowest index wins
+    assert ex.argmax(v) == orc.argmax(v)
+    m, k, nn = int(rng.integers(1, 90)), int(rng.integers(1, 200)), int(rng.integers(1, 90))
+    say("int8 affine matmul %d x %d x %d" % (m, k, nn))
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8); b = rng.integers(-128, 128, (k, nn), dtype=np.int8)
+    za, zb = int(rng.integers(-20, 20)), int(rng.integers(-20, 20))
+    got = ex.qmatmul_i8(a, 0.02, za, b, 0.03, zb)
+    want = orc.qmatmul_i8(a, 0.02, za, b, 0.03, zb)
+    assert np.array_equal(got[0], want[0]) and got[1:] == want[1:]
+
+
 def main():
     seed = int(sys.argv[1]) if len(sys.argv) > 1 else 1
     rounds = int(sys.argv[2]) if len(sys.argv) > 2 else 10
@@ -135,7 +188,7 @@ def main():
     say("device:", ex.device_info())
     for i in range(rounds):
         say("-- round %d of seed %d" % (i, seed))
-        for case in (gemv_case, grouped_case, gemm_case, dense_case, attention_case, small_ops_case):
+        for case in (gemv_case, grouped_case, shared_x_case, gemm_case, dense_case, attention_case, small_ops_case, misc_case):
             case(ex, rng, 1000 * seed + i)
     ex.close()
     say("FUZZ OK: %d rounds" % rounds)
