@@ -4,9 +4,10 @@ the emulated library (an access outside a buffer stops the run with an AddressSa
     python tests/emu/build_emulated.py OUT_DIR --run tests/emu/fuzz_models.py [seed [cases]]
 
 A case draws the widths (head size 64 or 128, grouped-query layouts, feed-forward width), a format per matrix slot (so
-the q / k / v and gate / up groups mix formats with and without a matrix-core path), and a way to cut a prompt into
-prefill calls (lengths that take the batched pass, the grid-slice pass and the token-by-token pass, starting off
-multiples of 32), then steps a few tokens.  After every call the logits must be finite and within a loose multiple of
+the q / k / v and gate / up groups mix formats with and without a matrix-core path), a context length (from 512 on the
+decode attention splits a head's positions over workgroups) and a way to cut a prompt into prefill calls (lengths that
+take the batched pass, the grid-slice pass and the token-by-token pass, starting off multiples of 32), then steps a few
+tokens.  After every call the logits must be finite and within a loose multiple of
 the benchmark's bound of the oracle's -- the tiny models are ill conditioned in places, so this hunts for faults, NaNs and
 gross errors, not for the last bit -- and a second model fed token by token must agree with the first."""
 import sys
@@ -34,6 +35,8 @@ def one_case(ex, rng, seed):
     hidden = nh * hd
     ffn = 256 * int(rng.integers(1, 5)); vocab = int(rng.integers(40, 200)); n_layers = int(rng.integers(1, 3))
     n_tok = int(rng.integers(20, 60)); max_pos = n_tok + 4
+    if rng.random() < 0.3:
+        max_pos = int(rng.integers(512, 700))      # from 512 positions on the decode attention is split over several workgroups
     uniform = rng.random() < 0.4
     fmts = {}
     base = str(rng.choice(MATRIX_FORMATS))
