@@ -1,6 +1,6 @@
 """Builds the library's own sources as host C++ against the stand-in HIP headers of tests/emu: every GPU thread a fiber,
-every device allocation an exact-size heap block under AddressSanitizer (and the alignment check of the undefined-behaviour
-sanitizer: a 16-byte access through a pointer that is not 16-byte aligned stops the run).  TEST INFRASTRUCTURE: the result is loaded by
+every device allocation an exact-size heap block under AddressSanitizer (with the undefined-behaviour sanitizer's checks of
+alignment, array bounds, shifts, signed overflow and conversions beside it: any of them stops the run).  TEST INFRASTRUCTURE: the result is loaded by
 tests only (RUSTORCH_HIP_LIBRARY names it), to run the same tests that run on the GPU -- at small sizes -- where an access
 outside a buffer stops the run with a report instead of faulting a device.
 
@@ -146,11 +146,13 @@ def to_host_cpp(src: str) -> str:
     return rewrite_asm(rewrite_launches(src))
 
 
-# The two instrumented builds.  "address": out-of-bounds and misaligned accesses.  "thread": a wave is a thread of the race
+# The two instrumented builds.  "address": out-of-bounds and misaligned accesses, indices outside fixed-size arrays, shifts by
+# too much, signed overflow, float-to-int conversions out of range, integer division by zero (each ends the run).  "thread": a wave is a thread of the race
 # detector (emu_fibers.h); function entry / exit hooks are off because the 64 lanes of a wave share one detector context
 # while each has a call stack of its own.
 SANITIZERS = {
-    "address": ["-fsanitize=address,alignment", "-fno-sanitize-recover=alignment", "-shared-libasan"],
+    "address": ["-fsanitize=address,alignment,bounds,shift-exponent,signed-integer-overflow,float-cast-overflow,integer-divide-by-zero",
+                "-fno-sanitize-recover=all", "-shared-libasan"],
     "thread": ["-fsanitize=thread", "-shared-libsan", "-mllvm", "-tsan-instrument-func-entry-exit=0"],
 }
 
