@@ -10,6 +10,10 @@ hipError_t &last_error() {
     static hipError_t e = hipSuccess;
     return e;
 }
+bool trace_launches() {
+    static const bool on = getenv("EMU_TRACE_LAUNCHES") != nullptr;
+    return on;
+}
 }  // namespace emu
 
 // ---- device memory
@@ -22,6 +26,7 @@ hipError_t hipMalloc(void **p, size_t n) {
     if (n > kEmuDeviceBytes - g_mem_bytes) return hipErrorOutOfMemory;
     *p = malloc(n ? n : 1);
     if (!*p) return hipErrorOutOfMemory;
+    memset(*p, 0xFF, n ? n : 1);      // undefined on the device; NaN patterns here, so that a read of it does not pass by luck
     g_mem[*p] = n;
     g_mem_bytes += n;
     return hipSuccess;

@@ -69,6 +69,7 @@ const void *wave_gather(const void *mine, size_t bytes);
 void uniform_point();
 int lane_id();
 bool launch3(Idx3 grid, Idx3 block, size_t lds_bytes, std::function<void()> kernel);
+bool trace_launches();      // EMU_TRACE_LAUNCHES=1 in the environment: every launch is named on stderr (a report then has its context)
 hipError_t &last_error();
 
 }  // namespace emu
@@ -147,6 +148,7 @@ inline emu::Idx3 emu_idx3(dim3 d) { return emu::Idx3{ d.x, d.y, d.z }; }
     do {                                                                                                                    \
         const emu::Idx3 emu_g = emu_idx3(dim3(grid)), emu_b = emu_idx3(dim3(block));                                        \
         const size_t emu_l = (size_t)(lds);                                                                                 \
+        if (emu::trace_launches()) fprintf(stderr, "emu: launch %s at %s:%d\n", #kernel, __FILE__, __LINE__);                \
         emu::submit(stream, [=] {                                                                                           \
             if (!emu::launch3(emu_g, emu_b, emu_l, [=] { kernel(__VA_ARGS__); })) emu::last_error() = hipErrorLaunchFailure; \
         });                                                                                                                 \
@@ -165,7 +167,12 @@ inline void __syncthreads() { emu::sync_threads(); }
 inline int __float_as_int(float f) { int i; std::memcpy(&i, &f, 4); return i; }
 inline float __int_as_float(int i) { float f; std::memcpy(&f, &i, 4); return f; }
 inline float __uint_as_float(unsigned i) { float f; std::memcpy(&f, &i, 4); return f; }
-inline int __float2int_rn(float f) { return (int)std::nearbyintf(f); }
+// v_cvt_i32_f32: NaN gives 0, values beyond the range saturate (a plain C++ conversion of those is undefined)
+inline int __float2int_rn(float f) {
+    if (f != f) return 0;
+    const float r = std::nearbyintf(f);
+    return r >= 2147483648.0f ? 2147483647 : (r <= -2147483648.0f ? (-2147483647 - 1) : (int)r);
+}
 inline int __mul24(int a, int b) { return (int)((unsigned)((a << 8) >> 8) * (unsigned)((b << 8) >> 8)); }     // v_mul_i32_i24
 using std::max;
 using std::min;
