@@ -231,6 +231,8 @@ __device__ __forceinline__ Q4Pack quantize4(float4 v) {
     amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
     amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
     amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    // (a block whose largest magnitude is below 16383 / FLT_MAX makes inv infinite: its zeros then give NaN, which the
+    // conversion below turns into 0, its other elements saturate and are clamped; the scale is as tiny as the values)
     float inv = amax > 0.f ? 16383.0f / amax : 0.f;
     Q4Pack r;
     r.s = amax / 16383.0f;
