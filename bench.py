@@ -30,10 +30,11 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK = 8.0e12
-# HBM bytes one launch of the GEMV kernel moves on this workload, from the FETCH_SIZE and WRITE_SIZE hardware
-# counters (each scaled by what the same counter reads for a plain x += y kernel of known size); measured
-# offline with the profiler, since counters cannot be read from inside this process.
-GEMV_TRAFFIC_BYTES = 131_800_000
+PARITY_BOUND = 1e-3     # max |y - y_f64| / (||w_row|| ||x||) a benchmarked launch may show
+# HBM bytes one launch moves on the headline workload, per kernel, from the FETCH_SIZE and WRITE_SIZE hardware counters
+# (each scaled by what the same counter reads for a plain x += y kernel of known size); measured offline with the
+# profiler, since counters cannot be read from inside this process.  A kernel without a measurement reports null.
+GEMV_TRAFFIC_BYTES = {"qgemv_kernel<512>": 131_800_000}
 SEED = 20250127
 H, F, V, NH, NL = 4096, 11008, 32000, 32, 32
 
@@ -79,6 +80,8 @@ def bench_layer_gemv(ex, steps, warmup, n_layers):
         ws = [ex.upload_qweight(t, r, c, synth.blocks(t, SEED, synth.layer_tid(l, slot), r, c)) for slot, t, r, c in specs]
         layers.append(ws)
     log("[bench] %d layers (%.2f GB) generated and uploaded in %.1f s" % (n_layers, n_layers * wbytes / 1e9, time.time() - t0))
+    plan = ex.qgemv_describe(layers[0])       # the kernel the timed launch runs and how the planner cuts it
+    log("[bench] headline launch:", plan)
     xs = [ex.to_device(synth.normal(SEED, 1000 + i, c)) for i, (_, _, _, c) in enumerate(specs)]
     xqs = [ex.buffer(ex.xq_bytes(c)) for _, _, _, c in specs]
     ys = [ex.buffer(4 * r) for _, _, r, _ in specs]
@@ -110,7 +113,7 @@ def bench_layer_gemv(ex, steps, warmup, n_layers):
         for w in ws:
             w.free()
     return dict(wbytes=wbytes, abytes=abytes, wall_s=wall, event_ms=ev_ms, kernel_ms=kern_ms, hot_ms=hot_ms, fused_ms=fused_ms, regions=n_regions,
-                results=results)
+                results=results, plan=plan)
 
 
 def bench_read_probe(ex, nbytes, steps):
@@ -277,30 +280,40 @@ def bench_dense_f32(ex, reps=5):
         ex.matmul_f32_dev(a, b, c, m, n, k)
         ms = timed_regions(ex, lambda: [ex.matmul_f32_dev(a, b, c, m, n, k) for _ in range(reps)])[0] / reps
         flops = 2.0 * m * n * k
-        out.append({"m": m, "n": n, "k": k, "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "mfma_f32_frac": round(flops / (ms * 1e-3) / F32_PEAK, 4)})
+        out.append({"m": m, "n": n, "k": k, "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "mfma_f32_frac": round(flops / (ms * 1e-3) / F32_PEAK, 4),
+                    "kernel": "matmul_f32_mfma_kernel" if ex.get_option(ex.OPT_DENSE_MFMA) else "matmul_f32_kernel"})
         for buf in (a, b, c):
             buf.free()
     return out
 
 
-def cpu_baseline(reps, gpu_results=None):
-    """Reference CPU path for one layer: dequantize each tensor to dense f32, then x . W^T with sequential k-sums.
-    With `gpu_results` (what the benchmarked launch left for this layer) also the correctness gate of the timing: the
-    worst |y_gpu - y_f64| / (||w_row|| ||x||) over the seven projections, against the f64 products of the same blocks."""
-    from oracle import oracle as orc
+def layer_inputs():
+    """Blocks and activation vectors of layer 0 of the headline workload, as the GPU legs generate them."""
     from rustorch_amd import synth
     specs = synth.layer_tensor_specs(H, F)
-    wbytes, _ = layer_bytes_algorithmic(specs)
-    tensors = [(t, r, c, synth.blocks(t, SEED, synth.layer_tid(0, slot), r, c), synth.normal(SEED, 1000 + i, c))
-               for i, (slot, t, r, c) in enumerate(specs)]
+    return [(t, r, c, synth.blocks(t, SEED, synth.layer_tid(0, slot), r, c), synth.normal(SEED, 1000 + i, c))
+            for i, (slot, t, r, c) in enumerate(specs)]
+
+
+def parity_of_launch(tensors, gpu_results):
+    """The correctness gate of the timing: the worst |y_gpu - y_f64| / (||w_row|| ||x||) over the seven projections of the
+    benchmarked launch, against the oracle's f64 products of the same blocks.  Computed outside the timed regions."""
+    from oracle import oracle as orc
+    worst = 0.0
+    for (t, r, c, raw, x), got in zip(tensors, gpu_results):
+        y64, wn = orc.qgemv_f64(t, raw, r, c, x)
+        yard = wn * np.linalg.norm(x.astype(np.float64))
+        if not np.isfinite(got).all():
+            return float("inf")
+        worst = max(worst, float((np.abs(got.astype(np.float64) - np.asarray(y64).reshape(-1)) / yard).max()))
+    return worst
+
+
+def cpu_baseline(tensors, reps):
+    """Reference CPU path for one layer: dequantize each tensor to dense f32, then x . W^T with sequential k-sums."""
+    from oracle import oracle as orc
+    wbytes = sum(t.row_bytes(c) * r for t, r, c, _, _ in tensors)
     ncores = orc.num_threads()
-    worst = None
-    if gpu_results is not None:
-        worst = 0.0
-        for (t, r, c, raw, x), got in zip(tensors, gpu_results):
-            y64, wn = orc.qgemv_f64(t, raw, r, c, x)
-            yard = wn * np.linalg.norm(x.astype(np.float64))
-            worst = max(worst, float((np.abs(got.astype(np.float64) - np.asarray(y64).reshape(-1)) / yard).max()))
     best = {}
     for threads in (1, ncores):
         ts = []
@@ -311,7 +324,7 @@ def cpu_baseline(reps, gpu_results=None):
                 orc.matmul_xwt(x, W, threads)
             ts.append(time.perf_counter() - t0)
         best[threads] = min(ts)
-    return wbytes, best[1], best[ncores], ncores, worst
+    return wbytes, best[1], best[ncores], ncores
 
 
 def main():
@@ -328,6 +341,9 @@ def main():
     ap.add_argument("--decode-prompt", type=int, default=128)
     ap.add_argument("--decode-gen", type=int, default=128)
     ap.add_argument("--decode-shape", choices=sorted(SHAPES), default="7b", help="model shape of the decode measurement (the benchmark's is 7b)")
+    ap.add_argument("--gemv-path", choices=("default", "general", "lean"), default="default",
+                    help="decode GEMV kernel of every leg: the library's default, the general kernel, or the lean one (rt_hip_set_option)")
+    ap.add_argument("--dense-mfma", action="store_true", help="dense f32 leg on the f32 matrix-core kernel (rt_hip_set_option)")
     ap.add_argument("--calibrate", action="store_true",
                     help="run only a plain x += y kernel over 2 x 128 MiB (reads 256 MiB, writes 128 MiB per launch): "
                          "the known-size launch that hardware traffic counters are scaled by")
@@ -339,6 +355,11 @@ def main():
     ex = HipKernelExecutor(0)
     info = ex.device_info()
     log("[bench] device:", info)
+
+    if args.gemv_path != "default":
+        ex.set_option(ex.OPT_GEMV_LEAN, 1 if args.gemv_path == "lean" else 0)
+    if args.dense_mfma:
+        ex.set_option(ex.OPT_DENSE_MFMA, 1)
 
     if args.calibrate:
         n = 32 << 20
@@ -361,6 +382,17 @@ def main():
         return
 
     g = bench_layer_gemv(ex, args.steps, args.warmup, args.layers)
+    kernel = g["plan"].split(" ")[0]
+    # the gate before anything is reported: a launch outside the bound has no rate
+    tensors = None if args.no_cpu else layer_inputs()
+    parity = None if args.no_cpu else parity_of_launch(tensors, g["results"])
+    if parity is not None and not parity <= PARITY_BOUND:
+        log("[bench] the benchmarked launch (%s) is outside the bound: worst |y - y_f64| / (||w_row|| ||x||) = %.3e > %.0e" % (g["plan"], parity, PARITY_BOUND))
+        print(json.dumps({"metric": "Q4_K/Q6_K GEMV weight GB/s, one Llama-7B decoder layer at batch 1 (plus decode tokens/s), 1xMI355X", "value": None,
+                          "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
+                          "error": "parity gate failed", "config": {"workload": "C3", "parity_worst": parity, "kernel": g["plan"]}}), flush=True)
+        ex.close()
+        sys.exit(1)
     # wall_s, event_ms: the median region of `steps` steps (timed_regions)
     ms_per_step = 1e3 * g["wall_s"] / args.steps
     value = g["wbytes"] / (g["wall_s"] / args.steps) / 1e9
@@ -374,9 +406,11 @@ def main():
                    "weight_bytes_per_step": g["wbytes"], "layers_rotated": args.layers, "hbm_frac_of_value": round(value * 1e9 / HBM_PEAK, 4),
                    "event_ms_per_step": round(g["event_ms"] / args.steps, 5),
                    "timing": "every figure is the median over %d repeats of a region of `steps` launches (repeated until 10 ms of device time are covered)" % g["regions"],
-                   "tolerance": "max |y - y_f64| <= 1e-3 * ||w_row|| * ||x|| per element", "parity_worst": None},
+                   "tolerance": "max |y - y_f64| <= 1e-3 * ||w_row|| * ||x|| per element",
+                   # of the benchmarked launch on one layer, in units of ||w_row|| ||x||; the run ends without a rate when it exceeds the bound
+                   "parity_worst": parity},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": GEMV_TRAFFIC_BYTES, "kernel": "qgemv_lean_kernel<512,1>",
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": GEMV_TRAFFIC_BYTES.get(kernel), "kernel": kernel, "launch": g["plan"],
                      "bytes_per_launch": g["abytes"], "avg_launch_ms": round(g["kernel_ms"], 5),
                      "cache_resident_launch_ms": round(g["hot_ms"], 5),
                      "fused_quantize_launch_ms": round(g["fused_ms"], 5)},
@@ -393,8 +427,7 @@ def main():
         out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen, args.decode_shape)
     ex.close()
     if not args.no_cpu:
-        wbytes, t1, tn, ncores, worst = cpu_baseline(3, g["results"])
-        out["config"]["parity_worst"] = worst       # of the benchmarked launch on one layer, in units of ||w_row|| ||x||; the bound is 1e-3
+        wbytes, t1, tn, ncores = cpu_baseline(tensors, 3)
         out["cpu_baseline"] = {"value": round(wbytes / t1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": "one of the 32 layers (seven projections, batch 1): dequantize to dense f32, then naive x.W^T; best of 3",
                                "all_cores_value": round(wbytes / tn / 1e9, 4), "all_cores": ncores}

@@ -25,7 +25,8 @@
  *     serialised internally; distinct contexts are independent.  There is no
  *     global mutable state (contrast src/gpu/mod.rs:757-772) apart from atomic
  *     per-device flags that record that a kernel's LDS limit has been raised
- *     (setting it twice is harmless, so they need no lock).
+ *     (setting it twice is harmless, so they need no lock) and the atomic
+ *     code-path switches of rt_hip_set_option.
  */
 #ifndef RUSTORCH_HIP_H
 #define RUSTORCH_HIP_H
@@ -98,6 +99,18 @@ RT_HIP_API const char *rt_hip_last_error(rt_hip_ctx *ctx);
 /* bytes per block / elements per block of a GGML type: GGMLType::type_size (gguf.rs:125-144); 0 if unsupported. */
 RT_HIP_API size_t rt_hip_type_block_bytes(int ggml_type);
 RT_HIP_API size_t rt_hip_type_block_elems(int ggml_type);
+
+/* ---- code-path switches (no reference counterpart; the nearest thing is the cargo feature set that picks a backend,
+ *      Cargo.toml:166).  Where two kernels serve one call, the one with the longer record on the device is the default and
+ *      the other is opt-in: process-wide, atomic, read at every launch, so a caller can run one call each way and compare.
+ *      Initial values come from the environment (RUSTORCH_HIP_GEMV_LEAN, RUSTORCH_HIP_DENSE_MFMA: "1" switches on).
+ *      Unknown options and values are refused with RT_HIP_ERR_INVALID_ARG. */
+typedef enum {
+    RT_HIP_OPT_GEMV_LEAN = 1,  /* 1: decode GEMV launches whose problems are all Q4_K / Q6_K / Q8_0 / Q4_0 take the lean kernel; 0 (default): the general one */
+    RT_HIP_OPT_DENSE_MFMA = 2  /* 1: dense f32 products in whole 16-byte pieces take the f32 matrix-core kernel; 0 (default): the LDS-tiled one */
+} rt_hip_option;
+RT_HIP_API int rt_hip_set_option(rt_hip_ctx *ctx, int option, int value);
+RT_HIP_API int rt_hip_get_option(rt_hip_ctx *ctx, int option, int *value);
 
 /* ---- resident buffers: the GpuBuffer<T> idiom (src/gpu/memory_ops/buffer.rs:22-48). */
 RT_HIP_API int rt_hip_malloc(rt_hip_ctx *ctx, size_t nbytes, void **out_dev);
@@ -188,6 +201,11 @@ RT_HIP_API int rt_hip_quantize_act_dev(rt_hip_ctx *ctx, int n, const float *cons
                                        void *const *xqs_dev);
 RT_HIP_API int rt_hip_qgemv_xq_grouped_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const *ws,
                                            const void *const *xqs_dev, float *const *ys_dev);
+/* Report aid (no reference counterpart): which kernel the grouped launches above would run for these n weights at this
+ * batch size, and how the launch would be cut, as text in out (at most out_bytes - 1 characters and a NUL).  Launches
+ * nothing.  The bench names the kernel it measured with this instead of assuming one. */
+RT_HIP_API int rt_hip_qgemv_describe(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const *ws, int batch, char *out,
+                                     size_t out_bytes);
 /* Y[M, n_rows] = X[M, n_cols] . dequant(W)^T for prefill (any M >= 1; MFMA path for M >= 16). */
 RT_HIP_API int rt_hip_qgemm(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *X, size_t M, float *Y);
 RT_HIP_API int rt_hip_qgemm_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *X_dev, size_t M,

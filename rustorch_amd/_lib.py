@@ -46,6 +46,8 @@ SIGNATURES = {
     "rt_hip_event_record": (C.c_int, [C.c_void_p, C.c_void_p]),
     "rt_hip_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, c_float_p]),
     "rt_hip_event_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "rt_hip_set_option": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
+    "rt_hip_get_option": (C.c_int, [C.c_void_p, C.c_int, c_int_p]),
     "rt_hip_stream_read_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "rt_hip_matmul_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]),
     "rt_hip_matmul_f32_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t]),
@@ -63,6 +65,7 @@ SIGNATURES = {
     "rt_hip_xq_bytes": (C.c_size_t, [C.c_size_t]),
     "rt_hip_quantize_act_dev": (C.c_int, [C.c_void_p, C.c_int, c_void_pp, C.POINTER(C.c_size_t), c_void_pp]),
     "rt_hip_qgemv_xq_grouped_dev": (C.c_int, [C.c_void_p, C.c_int, c_void_pp, c_void_pp, c_void_pp]),
+    "rt_hip_qgemv_describe": (C.c_int, [C.c_void_p, C.c_int, c_void_pp, C.c_int, C.c_char_p, C.c_size_t]),
     "rt_hip_qgemm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rt_hip_qgemm_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rt_hip_rmsnorm_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_float]),

@@ -4,8 +4,10 @@
 // status code and leaves the failure text in the context.
 #include "rt_internal.h"
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -29,6 +31,36 @@ int hip_fail(rt_hip_ctx *ctx, hipError_t e, const char *what) {
     int code = (e == hipErrorOutOfMemory) ? RT_HIP_ERR_OOM : RT_HIP_ERR_HIP;
     (void)hipGetLastError();
     return fail(ctx, code, "%s: %s", what, hipGetErrorString(e));
+}
+
+// Code-path switches: one atomic per option, -1 until the environment has been consulted.
+namespace {
+constexpr int kOptions = 3;      // option ids 1 .. kOptions - 1
+std::atomic<int> g_option[kOptions] = { { 0 }, { -1 }, { -1 } };
+const char *option_env(int option) {
+    switch (option) {
+    case RT_HIP_OPT_GEMV_LEAN: return "RUSTORCH_HIP_GEMV_LEAN";
+    case RT_HIP_OPT_DENSE_MFMA: return "RUSTORCH_HIP_DENSE_MFMA";
+    default: return nullptr;
+    }
+}
+}  // namespace
+int path_option(int option) {
+    const char *env = option_env(option);
+    if (!env) return -1;
+    int v = g_option[option].load(std::memory_order_relaxed);
+    if (v < 0) {
+        const char *e = getenv(env);
+        v = (e && e[0] == '1' && e[1] == 0) ? 1 : 0;
+        int expected = -1;
+        if (!g_option[option].compare_exchange_strong(expected, v, std::memory_order_relaxed)) v = expected;      // a set_option got there first
+    }
+    return v;
+}
+bool set_path_option(int option, int value) {
+    if (!option_env(option) || (value != 0 && value != 1)) return false;
+    g_option[option].store(value, std::memory_order_relaxed);
+    return true;
 }
 
 // Grow the context scratch to at least `bytes` (contents are not preserved).
@@ -540,6 +572,23 @@ int rt_hip_qgemv_xq_grouped_dev(rt_hip_ctx *ctx, int n, const rt_hip_qweight *co
     return RT_HIP_OK;
 }
 
+int rt_hip_qgemv_describe(rt_hip_ctx *ctx, int n, const rt_hip_qweight *const *ws, int batch, char *out, size_t out_bytes) {
+    if (!ctx || !ws || !out || out_bytes == 0) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_qgemv_describe: NULL argument");
+    RT_REQUIRE(ctx, n >= 1 && n <= rt::kMaxGemvProbs, RT_HIP_ERR_INVALID_ARG, "grouped GEMV takes 1..%d problems, got %d", rt::kMaxGemvProbs, n);
+    rt::GemvArgs a;
+    memset(&a, 0, sizeof a);
+    a.n = n;
+    for (int i = 0; i < n; i++) {
+        if (!ws[i]) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_qgemv_describe: weight %d is NULL", i);
+        int rc = qgemv_check(ctx, ws[i], batch);
+        if (rc) return rc;
+        a.p[i].w = ws[i]->dev; a.p[i].row_bytes = ws[i]->row_bytes; a.p[i].type = ws[i]->type; a.p[i].N = (int)ws[i]->n_rows; a.p[i].K = (int)ws[i]->n_cols;
+    }
+    out[0] = 0;
+    if (!rt::describe_qgemv(a, batch, out, out_bytes)) return fail(ctx, RT_HIP_ERR_SHAPE, "rt_hip_qgemv_describe: no launch takes these problems");
+    return RT_HIP_OK;
+}
+
 int rt_hip_qgemm_dev(rt_hip_ctx *ctx, const rt_hip_qweight *w, const float *X_dev, size_t M, float *Y_dev) {
     if (!ctx || !w || !X_dev || !Y_dev) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_qgemm_dev: NULL argument");
     RT_REQUIRE(ctx, gemv_type_ok(w->type), RT_HIP_ERR_UNSUPPORTED_TYPE, "qgemm: GGML type id %d has no kernel", w->type);
@@ -641,6 +690,19 @@ int rt_hip_add_dev(rt_hip_ctx *ctx, float *x, const float *y, size_t n) {
     if (!ctx || !x || !y) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_add_dev: NULL argument");
     Guard g(ctx);
     RT_TRY_HIP(ctx, rt::launch_add(ctx->stream, x, y, n));
+    return RT_HIP_OK;
+}
+
+int rt_hip_set_option(rt_hip_ctx *ctx, int option, int value) {
+    if (!rt::set_path_option(option, value)) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_set_option: option %d, value %d", option, value);
+    return RT_HIP_OK;
+}
+
+int rt_hip_get_option(rt_hip_ctx *ctx, int option, int *value) {
+    if (!value) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_get_option: NULL argument");
+    const int v = rt::path_option(option);
+    if (v < 0) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_get_option: option %d", option);
+    *value = v;
     return RT_HIP_OK;
 }
 

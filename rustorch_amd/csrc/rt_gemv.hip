@@ -4,6 +4,8 @@
 #include "rt_gemv_lean.h"
 #include "rt_gemv_plan.h"
 
+#include <cstdio>
+
 namespace rt {
 
 namespace {
@@ -30,10 +32,30 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
 
 }  // namespace
 
+// The plan of a launch as the launcher makes it: the lean path is opt-in (rt_hip_set_option), the general kernel serves
+// every launch otherwise.
+static bool plan_launch(GemvArgs &a, int batch, GemvPlan &pl) {
+    GemvPlanHints hints;
+    hints.lean = path_option(RT_HIP_OPT_GEMV_LEAN) == 1 ? 1 : 0;
+    return plan_qgemv(a, batch, pl, hints);
+}
+
+// Which kernel launch_qgemv would run for these problems and how it would cut the launch, as text (for reports).
+bool describe_qgemv(GemvArgs &a, int batch, char *out, size_t out_bytes) {
+    GemvPlan pl;
+    if (!plan_launch(a, batch, pl)) return false;
+    int n = pl.lean ? snprintf(out, out_bytes, "qgemv_lean_kernel<%d,1>", pl.threads) : snprintf(out, out_bytes, "qgemv_kernel<%d>", pl.threads);
+    if (n < 0 || (size_t)n >= out_bytes) return true;
+    n += snprintf(out + n, out_bytes - n, " grid %dx%d lds %zu%s shares", pl.wgs, batch, pl.lds, pl.lean ? "" : (pl.r2 ? " two rows per step" : " one row per step"));
+    for (int i = 0; i < a.n && (size_t)n < out_bytes; i++)
+        n += snprintf(out + n, out_bytes - n, " %d%s", a.p[i].rows_per_tile, a.p[i].ksplit ? "k" : "");
+    return true;
+}
+
 // One grid over all problems (grid.y = batch row).  Workgroups of a problem stage x once and deal its rows out round-robin.
 hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
     GemvPlan pl;
-    if (!plan_qgemv(a, batch, pl)) return hipErrorInvalidValue;
+    if (!plan_launch(a, batch, pl)) return hipErrorInvalidValue;
     dim3 grid((unsigned)pl.wgs, (unsigned)batch);
     const size_t lds = pl.lds;
     if (lds > 64 * 1024) {

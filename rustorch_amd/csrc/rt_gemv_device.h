@@ -178,15 +178,27 @@ template <> struct XRegs<RT_GGML_Q4_1> : XRegs<RT_GGML_Q4_0> {};
 template <> struct XRegs<RT_GGML_Q5_0> : XRegs<RT_GGML_Q4_0> {};
 template <> struct XRegs<RT_GGML_Q5_1> : XRegs<RT_GGML_Q4_0> {};
 
-// Weight loads go through a buffer resource: the matrix is the buffer, the row (wave-uniform) a scalar byte
-// offset, the lane's place in the row a 32-bit vector offset -- no 64-bit address arithmetic per load.
+// Weight loads go through a buffer resource made for the piece of the matrix a wave step may read (a row, or one pass of
+// a row): the resource starts at the piece's first byte and its num_records is the piece's length, so the hardware's range
+// check holds every lane inside the piece whatever its 32-bit vector offset turns out to be -- a lane that is out of range
+// reads zeros (a failed comparison in a test) instead of touching memory that may not be mapped.  The piece itself is
+// placed by wave-uniform scalar arithmetic and clamped to the tensor, so no load of these kernels can leave the tensor.
+// No 64-bit address arithmetic per load: the lane's place in the piece is the vector offset.
+//
+// The start is rounded down to a multiple of four bytes (rows of Q6_K at K = 11008 are 9030 bytes: only 2-byte aligned)
+// and the remainder goes into the scalar offset, with num_records lengthened by it: whether the range check counts the
+// scalar offset or not, every in-range lane passes it, and no lane gets more than 3 bytes past the piece.
 struct WRow {
     __amdgpu_buffer_rsrc_t rsrc;
-    uint32_t soff;      // row * row_bytes
+    uint32_t soff;      // 0..3: what the rounding of the start took off
 };
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t weight_rsrc(const uint8_t *w) {
-    // raw buffer (stride 0), no range limit of its own (rows and units are clamped by the caller), dword 3 as for 32-bit data
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w), 0, 0xFFFFFFFFu, 0x00020000);
+// w: the tensor; nbytes: its size (N * row_bytes < 4 GB, checked at launch); start: byte offset of the piece; span: its length
+// (nbytes >= span).  All arguments wave-uniform.
+__device__ __forceinline__ WRow weight_window(const uint8_t *w, uint32_t nbytes, uint32_t start, uint32_t span) {
+    start = min(start, nbytes - span);      // unsigned: a start that went wrong in any direction lands inside the tensor
+    const uint32_t rem = start & 3u;
+    // raw buffer (stride 0), dword 3 as for 32-bit data
+    return WRow{ __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w) + (start - rem), 0, (int)(span + rem), 0x00020000), rem };
 }
 __device__ __forceinline__ uint4 bld16(WRow r, uint32_t off) {
     return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r.rsrc, off, r.soff, 0));
@@ -603,7 +615,8 @@ struct Walker {
     const uint32_t *lds;
     int m, U, n_iter, lane, gw, n_gw, n_groups, rows_per_group;
     bool dual;
-    __amdgpu_buffer_rsrc_t rsrc, rsrc2;
+    const uint8_t *w1, *w2;     // the matrix, and the second one of the gate / up pair form (else the same)
+    uint32_t nbytes;            // size of a matrix
 
     // A step is (row group g, unit pass p); steps are walked in order, so the position is advanced, not divided out.
     struct Pos { int g, p; };
@@ -621,8 +634,8 @@ struct Walker {
         for (int r = 0; r < R; r++) {
             int row = dual ? g * rows_per_group + (r >> 1) : g * rows_per_group + r;
             row = min(row, P.N - 1);  // ragged tail: reread the last row, the store is skipped
-            // a tensor is below 4 GB (checked at launch), so the row offset fits the 32-bit scalar offset of the load
-            load_w(w[r], WRow{ (dual && (r & 1)) ? rsrc2 : rsrc, (uint32_t)row * (uint32_t)P.row_bytes }, u);
+            // a tensor is below 4 GB (checked at launch), so the row's byte offset fits 32 bits
+            load_w(w[r], weight_window((dual && (r & 1)) ? w2 : w1, nbytes, (uint32_t)row * (uint32_t)P.row_bytes, (uint32_t)P.row_bytes), u);
             if (!dual && P.res) rv[r] = ld_f<COH>(&P.res[(size_t)m * P.N + row]);
         }
     }
@@ -670,7 +683,7 @@ template <int TYPE, int R, bool COH>
 __device__ __forceinline__ void gemv_problem(const GemvProb &P, int wg, int n_wg, int m, uint32_t *lds, float *red) {
     const int waves = (int)(blockDim.x >> 6);
     Walker<TYPE, R, COH> W{ P, lds, m, units_of(TYPE, P.K), 0, (int)(threadIdx.x & 63), 0, 0, 0, 0, P.epi == kEpiSwiglu,
-                            weight_rsrc(P.w), weight_rsrc(P.epi == kEpiSwiglu ? P.w2 : P.w) };
+                            P.w, P.epi == kEpiSwiglu ? P.w2 : P.w, (uint32_t)P.N * (uint32_t)P.row_bytes };
     W.n_iter = (W.U + 63) / 64;
     W.rows_per_group = W.dual ? R / 2 : R;
     W.n_groups = (P.N + W.rows_per_group - 1) / W.rows_per_group;

@@ -275,8 +275,8 @@ __device__ __forceinline__ void lean_problem_t(const GemvProb &P, int wg, int n_
     const int n_gw = n_wg * waves;
     const int my_groups = gw < n_groups ? (n_groups - gw + n_gw - 1) / n_gw : 0;
     const int steps = my_groups * n_iter;
-    const uint32_t row_bytes = (uint32_t)P.row_bytes;
-    const __amdgpu_buffer_rsrc_t rsrc = weight_rsrc(P.w), rsrc2 = weight_rsrc(DUAL ? P.w2 : P.w);
+    const uint32_t row_bytes = (uint32_t)P.row_bytes, nbytes = (uint32_t)N * row_bytes;
+    const uint8_t *const w1 = P.w, *const w2 = DUAL ? P.w2 : P.w;
     // a residual is taken only in place (res == y; the launcher sends other cases to the general path): the row end is then
     // one returnless floating-point add to memory, with no load to wait for and no register held for it
     const bool add_to_y = !DUAL && P.res != nullptr;
@@ -288,10 +288,11 @@ __device__ __forceinline__ void lean_problem_t(const GemvProb &P, int wg, int n_
     // position of a step: row group g, pass p
     struct Pos { int g, p; };
     auto next = [&](Pos q) { return q.p + 1 == n_iter ? Pos{ q.g + n_gw, 0 } : Pos{ q.g, q.p + 1 }; };
-    // EXACT: the row is a whole number of passes, every lane has a unit in every pass and the pass is part of the scalar
-    // offset.  Otherwise the pass is part of the lane's offset, and the lanes past the end of the row in its last pass
-    // reread the unit 64 before theirs (same u & 3, so the lane constants hold; U >= 64 whenever a row has more than one
-    // pass); their products are masked.  Offsets are unsigned: nothing here may go below the start of the row.
+    // EXACT: the row is a whole number of passes, every lane has a unit in every pass, and the window the loads go
+    // through (weight_window) is the pass.  Otherwise the window is the row, the pass is part of the lane's offset, and the
+    // lanes past the end of the row in its last pass reread the unit 64 before theirs (same u & 3, so the lane constants
+    // hold; U >= 64 whenever a row has more than one pass); their products are masked.  Offsets are unsigned: nothing here
+    // may go below the start of the row -- and if it did, the window's range check would turn the load into zeros.
     auto request = [&](WRegs<TYPE> *w, Pos s) {
         uint32_t so = 0, vo = 0;
         if (EXACT) so = (uint32_t)s.p * LeanLane<TYPE>::kPassBytes;
@@ -300,7 +301,8 @@ __device__ __forceinline__ void lean_problem_t(const GemvProb &P, int wg, int n_
         for (int r = 0; r < R; r++) {
             int row = s.g * RG + (DUAL ? (r >> 1) : r);
             row = min(row, N - 1);                                         // ragged tail: reread the last row, the store is skipped
-            L.load(w[r], WRow{ (DUAL && (r & 1)) ? rsrc2 : rsrc, (uint32_t)row * row_bytes + so }, vo);
+            L.load(w[r], weight_window((DUAL && (r & 1)) ? w2 : w1, nbytes, (uint32_t)row * row_bytes + so,
+                                       EXACT ? LeanLane<TYPE>::kPassBytes : row_bytes), vo);
         }
     };
 
@@ -417,8 +419,7 @@ __device__ __forceinline__ void lean_problem_split(const GemvProb &P, int wg, in
     const int rows_wg = wg < N ? (N - wg + n_wg - 1) / n_wg : 0;
     const int items = rows_wg * n_iter;
     const int steps = w < items ? (items - w + waves - 1) / waves : 0;
-    const uint32_t row_bytes = (uint32_t)P.row_bytes;
-    const __amdgpu_buffer_rsrc_t rsrc = weight_rsrc(P.w);
+    const uint32_t row_bytes = (uint32_t)P.row_bytes, nbytes = (uint32_t)N * row_bytes;
     const bool add_to_y = P.res != nullptr;
     float *y = P.y + (size_t)m * N;
     float *part = reinterpret_cast<float *>(lds) + ((gemv_lds_bytes(TYPE, (size_t)P.K) + 15) >> 4) * 4;      // [rows_wg][n_iter]
@@ -439,7 +440,7 @@ __device__ __forceinline__ void lean_problem_split(const GemvProb &P, int wg, in
         if (EXACT) so = (uint32_t)s.p * LeanLane<TYPE>::kPassBytes;
         else vo = (uint32_t)(s.p - ((lane + 64 * s.p >= U) ? 1 : 0)) * LeanLane<TYPE>::kPassBytes;      // n_iter > 1 here: U >= 64
         const int row = min(wg + n_wg * s.j, N - 1);
-        L.load(wr, WRow{ rsrc, (uint32_t)row * row_bytes + so }, vo);
+        L.load(wr, weight_window(P.w, nbytes, (uint32_t)row * row_bytes + so, EXACT ? LeanLane<TYPE>::kPassBytes : row_bytes), vo);
     };
 
     WRegs<TYPE> a, b;

@@ -27,6 +27,7 @@ struct GemvPlan {
 // code paths that large launches take.
 struct GemvPlanHints {
     int threads = -1, r2 = -1, budget = -1;
+    int lean = -1;        // 0: never the lean path; 1 or -1: wherever every problem of the launch qualifies
 };
 
 // Gives every problem a share of the workgroups in proportion to its weight bytes (tile0 = first workgroup,
@@ -45,7 +46,7 @@ inline bool plan_qgemv(GemvArgs &a, int batch, GemvPlan &pl, const GemvPlanHints
     }
     if (total_bytes <= 0) return false;
     if (lds > kGemvLdsMax) return false;    // x of the longest row must fit the workgroup's LDS
-    bool lean = lds <= 64 * 1024;
+    bool lean = hints.lean != 0 && lds <= 64 * 1024;
     for (int i = 0; i < a.n; i++) {
         const GemvProb &p = a.p[i];
         lean = lean && (p.res == nullptr || p.res == p.y) &&

@@ -77,11 +77,17 @@ struct QuantGroupArgs {
     int n;
 };
 
+// ---- code-path switches (rt_hip_set_option): process-wide atomics, initial value from the environment.
+// index = rt_hip_option; value -1 until first read.
+int path_option(int option);
+bool set_path_option(int option, int value);
+
 // ---- launchers (all enqueue on `s`, return hipError_t of the launch)
 hipError_t launch_set_state(hipStream_t s, int *state, int pos, int token, int step);
 hipError_t launch_quantize_x(hipStream_t s, const float *x, uint8_t *xq, size_t K, size_t batch);
 hipError_t launch_quantize_group(hipStream_t s, const QuantGroupArgs &a);
 hipError_t launch_qgemv(hipStream_t s, GemvArgs &args, int batch);  // fills tile0 / rows_per_tile
+bool describe_qgemv(GemvArgs &args, int batch, char *out, size_t out_bytes);   // the kernel and cut launch_qgemv would choose, as text
 
 // 2..8 activation rows against Q4_K / Q6_K weights in one pass over the weights, on the integer matrix cores
 // (rt_gemv_mb.hip).  work: qgemv_mb_scratch_bytes(K) bytes, 256-byte aligned; res (optional) is added to y.

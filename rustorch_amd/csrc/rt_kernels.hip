@@ -998,7 +998,7 @@ hipError_t launch_matmul_f32(hipStream_t s, const float *a, const float *b, floa
     // the matrix cores take products large enough to fill tiles and laid out in whole 16-byte pieces; the rest (the
     // reference's 2 x 2 known answer, odd widths, matrix-vector products) goes through the plain kernel
     const bool pieces = n % 4 == 0 && k % 4 == 0 && (((uintptr_t)a | (uintptr_t)b) & 15) == 0;
-    if (pieces && m >= 64 && n >= 64 && k >= kMmK) {
+    if (pieces && m >= 64 && n >= 64 && k >= kMmK && path_option(RT_HIP_OPT_DENSE_MFMA) == 1) {      // opt-in (rt_hip_set_option)
         dim3 grid((unsigned)((n + kMmTile - 1) / kMmTile), (unsigned)((m + kMmTile - 1) / kMmTile), (unsigned)batch);
         matmul_f32_mfma_kernel<<<grid, 256, 0, s>>>(a, b, c, m, n, k);
         return hipGetLastError();

@@ -166,6 +166,18 @@ class HipKernelExecutor:
                 "wavefront_size": info.wavefront_size, "hbm_bytes": info.hbm_bytes,
                 "lds_bytes_per_block": info.lds_bytes_per_block}
 
+    # -- code-path switches (rt_hip_set_option): process-wide, read at every launch
+    OPT_GEMV_LEAN = 1
+    OPT_DENSE_MFMA = 2
+
+    def set_option(self, option: int, value: int) -> None:
+        _lib.check(self.lib.rt_hip_set_option(self.ctx, int(option), int(value)), self.ctx)
+
+    def get_option(self, option: int) -> int:
+        v = C.c_int(0)
+        _lib.check(self.lib.rt_hip_get_option(self.ctx, int(option), C.byref(v)), self.ctx)
+        return v.value
+
     def event(self) -> Event:
         return Event(self)
 
@@ -291,6 +303,14 @@ class HipKernelExecutor:
         arr = C.c_void_p * n
         wa = arr(*[w.handle for w in ws]); qa = arr(*[q.ptr for q in xqs]); ya = arr(*[y.ptr for y in ys])
         _lib.check(self.lib.rt_hip_qgemv_xq_grouped_dev(self.ctx, n, wa, qa, ya), self.ctx)
+
+    def qgemv_describe(self, ws: Sequence[QWeight], batch: int = 1) -> str:
+        """The kernel a grouped launch over these weights would run and how it would be cut (rt_hip_qgemv_describe)."""
+        n = len(ws)
+        wa = (C.c_void_p * n)(*[w.handle for w in ws])
+        buf = C.create_string_buffer(256)
+        _lib.check(self.lib.rt_hip_qgemv_describe(self.ctx, n, wa, batch, buf, len(buf)), self.ctx)
+        return buf.value.decode()
 
     # -- decode-step operators (host arrays in, host arrays out; each call goes through device buffers)
     def rmsnorm(self, x, gamma, eps: float) -> np.ndarray:

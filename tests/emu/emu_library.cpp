@@ -42,6 +42,16 @@ hipError_t hipFree(void *p) {
     return hipSuccess;
 }
 
+// Whether [p, p + n) lies inside one live device allocation (the buffer loads of the stand-in header ask).
+extern "C" int emu_device_owns(const void *p, size_t n) {
+    std::lock_guard<std::mutex> lock(g_mem_mu);
+    auto it = g_mem.upper_bound(const_cast<void *>(p));
+    if (it == g_mem.begin()) return 0;
+    --it;
+    const char *b = static_cast<const char *>(it->first);
+    return static_cast<const char *>(p) + n <= b + it->second;
+}
+
 // ---- streams and captured graphs
 struct emu_graph { std::vector<std::function<void()>> work; };
 struct emu_graph_exec { std::vector<std::function<void()>> work; };

@@ -1,4 +1,4 @@
-// CPU run of the persistent decode-step kernel (rustorch_amd/csrc/rt_mega_device.h) under AddressSanitizer.
+// CPU run of the persistent decode-step kernel (tests/emu/rt_mega_device.h) under AddressSanitizer.
 // TEST INFRASTRUCTURE.  Every GPU thread is a fiber; see tests/emu/hip/hip_runtime.h for the execution model.
 // What it checks: no out-of-bounds access to any buffer the kernel is handed, every workgroup leaves the
 // kernel (no barrier time-out, no dead rendezvous), and the logits agree with the CPU oracle.

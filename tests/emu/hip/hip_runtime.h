@@ -226,17 +226,34 @@ inline void unsafeAtomicAdd(float *p, float v) {
         memcpy(&want, &f, 4);
     } while (!__atomic_compare_exchange(reinterpret_cast<uint32_t *>(p), &seen, &want, false, __ATOMIC_RELAXED, __ATOMIC_RELAXED));
 }
-// buffer resources: base pointer only (the emulation neither checks ranges nor strides), loads at base + voffset + soffset
-struct emu_buffer_rsrc { const unsigned char *base; };
+// buffer resources (raw, stride 0): base pointer and num_records.  A load must lie inside the resource -- the sources never
+// rely on the zeros the hardware returns for an out-of-range lane, so here such a lane ends the run, which is stricter than
+// the device and than the address sanitizer (a wild offset can land inside another live block).  The check is made both
+// ways the range check may be defined (with and without the scalar offset), and the bytes must belong to one allocation of
+// the emulated device where the runtime that tracks them is linked in.
+struct emu_buffer_rsrc { const unsigned char *base; unsigned num; };
 typedef emu_buffer_rsrc __amdgpu_buffer_rsrc_t;
 typedef unsigned int emu_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int emu_u32x2 __attribute__((ext_vector_type(2)));
-inline emu_buffer_rsrc emu_make_rsrc(const void *p) { return emu_buffer_rsrc{ (const unsigned char *)p }; }
-inline emu_u32x4 emu_bload128(emu_buffer_rsrc r, unsigned voff, unsigned soff) { emu_u32x4 v; __builtin_memcpy(&v, r.base + voff + soff, 16); return v; }
-inline emu_u32x2 emu_bload64(emu_buffer_rsrc r, unsigned voff, unsigned soff) { emu_u32x2 v; __builtin_memcpy(&v, r.base + voff + soff, 8); return v; }
-inline unsigned int emu_bload32(emu_buffer_rsrc r, unsigned voff, unsigned soff) { unsigned int v; __builtin_memcpy(&v, r.base + voff + soff, 4); return v; }
-inline short emu_bload16(emu_buffer_rsrc r, unsigned voff, unsigned soff) { short v; __builtin_memcpy(&v, r.base + voff + soff, 2); return v; }
-#define __builtin_amdgcn_make_buffer_rsrc(p, stride, num, flags) emu_make_rsrc(p)
+extern "C" int emu_device_owns(const void *p, size_t n) __attribute__((weak));      // emu_library.cpp; absent in stand-alone drivers
+inline emu_buffer_rsrc emu_make_rsrc(const void *p, int num) { return emu_buffer_rsrc{ (const unsigned char *)p, (unsigned)num }; }
+inline void emu_bload(void *dst, emu_buffer_rsrc r, unsigned voff, unsigned soff, unsigned size) {
+    if ((unsigned long long)voff + soff + size > r.num) {
+        fprintf(stderr, "emu: buffer load out of range: voffset %u + soffset %u + %u bytes > num_records %u\n", voff, soff, size, r.num);
+        abort();
+    }
+    if (emu_device_owns && !emu_device_owns(r.base + voff + soff, size)) {
+        fprintf(stderr, "emu: buffer load of %u bytes at %p (voffset %u, soffset %u) is not inside one device allocation\n", size,
+                (const void *)(r.base + voff + soff), voff, soff);
+        abort();
+    }
+    __builtin_memcpy(dst, r.base + voff + soff, size);
+}
+inline emu_u32x4 emu_bload128(emu_buffer_rsrc r, unsigned voff, unsigned soff) { emu_u32x4 v; emu_bload(&v, r, voff, soff, 16); return v; }
+inline emu_u32x2 emu_bload64(emu_buffer_rsrc r, unsigned voff, unsigned soff) { emu_u32x2 v; emu_bload(&v, r, voff, soff, 8); return v; }
+inline unsigned int emu_bload32(emu_buffer_rsrc r, unsigned voff, unsigned soff) { unsigned int v; emu_bload(&v, r, voff, soff, 4); return v; }
+inline short emu_bload16(emu_buffer_rsrc r, unsigned voff, unsigned soff) { short v; emu_bload(&v, r, voff, soff, 2); return v; }
+#define __builtin_amdgcn_make_buffer_rsrc(p, stride, num, flags) emu_make_rsrc(p, num)
 #define __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, aux) emu_bload128(r, voff, soff)
 #define __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, aux) emu_bload64(r, voff, soff)
 #define __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, aux) emu_bload32(r, voff, soff)

@@ -33,7 +33,7 @@ SELECTION = [
     "tests/test_gpu_gemv.py::test_device_pointer_form_and_errors",
     "tests/test_gpu_gemv.py::test_dense_matmul_f32_kat",
     "tests/test_gpu_gemv.py::test_dense_matmul_on_resident_buffers_and_batches",
-    "tests/test_gpu_gemv.py::test_dense_matmul_on_the_matrix_cores",
+    "tests/test_z_optin_paths.py",                                                  # the lean GEMV and the dense matrix-core kernel, switched on per test
     "tests/test_gpu_gemv.py::test_batches_of_two_to_eight_on_the_matrix_cores[37-256-12]",
     "tests/test_gpu_gemv.py::test_batches_of_two_to_eight_on_the_matrix_cores[16-768-14]",
     "tests/test_gpu_gemv.py::test_batches_of_two_to_eight_on_the_matrix_cores[1-4096-12]",
@@ -64,7 +64,9 @@ RACE_SELECTION = [
     "tests/test_gpu_gemv.py::test_gemv_config_shapes_batch1_and_8[C3_down]",       # rows of three passes dealt out over the waves
     "tests/test_gpu_gemv.py::test_grouped_launch_equals_single_launches",
     "tests/test_gpu_gemv.py::test_batches_of_two_to_eight_on_the_matrix_cores[300-11008-14]",
-    "tests/test_gpu_gemv.py::test_dense_matmul_on_the_matrix_cores",
+    "tests/test_z_optin_paths.py::test_dense_matmul_on_the_matrix_cores",
+    "tests/test_z_optin_paths.py::test_lean_gemv_edge_inputs",
+    "tests/test_z_optin_paths.py::test_lean_gemv_config_shapes[C3_down]",
     "tests/test_gpu_gemm.py::test_single_superblock_odd_counts_and_tiny_matrices",
     "tests/test_gpu_gemm.py::test_three_to_fifteen_rows_go_eight_at_a_time[100-11008-12]",
 ]

@@ -225,31 +225,3 @@ def test_dense_matmul_on_resident_buffers_and_batches(ex):
         ex.matmul_f32_dev(dA, dB, c, m, n, k, batch)
     for buf in (a, b, c, dA, dB, dC, v, y):
         buf.free()
-
-
-@pytest.mark.parametrize("batch,m,n,k", [(1, 128, 128, 16), (3, 200, 136, 72), (1, 130, 132, 20), (2, 64, 64, 260), (1, 257, 384, 128), (1, 96, 64, 64)])
-def test_dense_matmul_on_the_matrix_cores(ex, batch, m, n, k):
-    """Products whose rows are whole 16-byte pieces and that fill tiles take the f32 matrix-core kernel (whole tiles, ragged
-    edges in m, n and k, batches): against NumPy f64, held to 4 * sqrt(k) roundings of the row and column norms; a
-    product with the identity returns its operand bit for bit (GpuValidator::validate_matrix_multiplication,
-    src/gpu/validation.rs:116-166)."""
-    print("dense matmul on the matrix cores: batch %d, %d x %d x %d" % (batch, m, n, k), flush=True)
-    rng = np.random.default_rng(m + n + k)
-    A = rng.standard_normal((batch, m, k)).astype(np.float32); B = rng.standard_normal((batch, k, n)).astype(np.float32)
-    dA, dB, dC = ex.to_device(A), ex.to_device(B), ex.buffer(4 * batch * m * n)
-    ex.matmul_f32_dev(dA, dB, dC, m, n, k, batch)
-    got = dC.download(np.float32).reshape(batch, m, n)
-    want = A.astype(np.float64) @ B.astype(np.float64)
-    bound = 4 * np.sqrt(k) * 2.0 ** -24 * np.linalg.norm(A.astype(np.float64), axis=2)[:, :, None] * np.linalg.norm(B.astype(np.float64), axis=1)[:, None, :]
-    assert np.isfinite(got).all() and np.all(np.abs(got - want) <= bound)
-    if k == n:
-        eye = np.broadcast_to(np.eye(k, dtype=np.float32), (batch, k, k)).copy()
-        dI = ex.to_device(eye)
-        ex.matmul_f32_dev(dA, dI, dC, m, n, k, batch)
-        assert np.array_equal(dC.download(np.float32).reshape(batch, m, n), A)
-        dI.free()
-    one = np.zeros((m, n), dtype=np.float32)
-    ex.matmul_f32(A[0], B[0], one, m, n, k)                    # the host-slice entry point runs the same kernel
-    assert np.array_equal(one, got[0])
-    for buf in (dA, dB, dC):
-        buf.free()

@@ -33,7 +33,13 @@ def stable_positions(om, toks, want, tol, rel=3e-4, frac=0.02):
     tolerances -- in the oracle just as on the GPU.  To tell those positions from real kernel errors the oracle is run a
     second and a third time with every attention-norm weight multiplied by 1 + rel * N(0, 1) (rel = 3e-4: ten times the relative
     rounding of the GPU's 15-bit activations): a position whose oracle logits move by more than `frac` of the tolerance in either run is
-    ill conditioned and exempt from the bound on the maximum; every other position has to keep the bound itself."""
+    ill conditioned and exempt from the bound on the maximum; every other position has to keep the bound itself.
+
+    The filter depends on the oracle alone, so how much it leaves in is known without a device: 3 to 5 of the 26 checked
+    positions of the grouped-query models, 13 and 20 of 42 of the long-context ones, 2 of 12 after the prefill passes.
+    It is a small subset: what these tests state about every position is the typical-position bound (median and nine in
+    ten inside the tolerance); the bound at every position without exemption is held by the full-size model test.  Each
+    caller asserts the count it was written against, so the exemption cannot quietly grow to cover everything."""
     rng = np.random.default_rng(12345)
     n_layers = len(om.attn_norms)
     hidden = om.attn_norms[0].size
@@ -167,6 +173,7 @@ def test_grouped_query_attention_model(ex, orc, n_heads, n_kv):
     print("ratio to the tolerance: median %.3f, max %.2f, %d of %d above 1; well-conditioned positions: %d, max %.3f"
           % (np.median(ratios), ratios.max(), (ratios > 1).sum(), ratios.size, ok.sum(), ratios[ok].max() if ok.any() else 0.0), flush=True)
     assert np.median(ratios) <= 0.1 and (ratios <= 1).mean() >= 0.9
+    assert ok.sum() >= 3, "the stability filter left %d positions in" % ok.sum()
     assert np.all(ratios[ok] <= 1.0), "positions %s" % [a for a, r, k in zip(at, ratios, ok) if k and r > 1.0]
     with pytest.raises(ShapeMismatch):                           # k must have n_kv * head_dim rows
         gm.upload("attn_k", 0, 12, 512, 512, synth.blocks(12, 1, 1, 512, 512))
@@ -204,6 +211,7 @@ def test_long_context_attention_split_over_workgroups(ex, orc, n_heads, n_kv):
     # with hundreds of positions near-ties of the one-hot softmax are frequent: the typical position is held to the oracle,
     # and so is every position at which the oracle itself is well conditioned
     assert np.median(ratios) <= 0.2
+    assert ok.sum() >= 10, "the stability filter left %d positions in" % ok.sum()
     assert np.all(ratios[ok] <= 1.0), "positions %s" % [a for a, r, k in zip(at, ratios, ok) if k and r > 1.0]
 
 
@@ -268,6 +276,7 @@ def test_prefill_in_several_passes_and_calls(ex, orc):
     print("steps after the passes: median %.3f, max %.2f; well-conditioned positions: %d of 12, max %.3f"
           % (np.median(ratios), ratios.max(), ok.sum(), ratios[ok].max() if ok.any() else 0.0), flush=True)
     assert np.median(ratios) <= 0.2
+    assert ok.sum() >= 2, "the stability filter left %d positions in" % ok.sum()
     assert np.all(ratios[ok] <= 1.0)
     if stable[n - 1]:
         assert r <= 1.0
