@@ -341,8 +341,9 @@ def main():
     ap.add_argument("--decode-prompt", type=int, default=128)
     ap.add_argument("--decode-gen", type=int, default=128)
     ap.add_argument("--decode-shape", choices=sorted(SHAPES), default="7b", help="model shape of the decode measurement (the benchmark's is 7b)")
-    ap.add_argument("--gemv-path", choices=("default", "general", "lean"), default="default",
-                    help="decode GEMV kernel of every leg: the library's default, the general kernel, or the lean one (rt_hip_set_option)")
+    ap.add_argument("--gemv-path", choices=("default", "general", "lean", "lean5"), default="default",
+                    help="decode GEMV kernel of every leg: the library's default, the general kernel, the lean one, or the lean one with "
+                         "five waves per SIMD where the launch allows it (rt_hip_set_option)")
     ap.add_argument("--dense-mfma", action="store_true", help="dense f32 leg on the f32 matrix-core kernel (rt_hip_set_option)")
     ap.add_argument("--calibrate", action="store_true",
                     help="run only a plain x += y kernel over 2 x 128 MiB (reads 256 MiB, writes 128 MiB per launch): "
@@ -357,7 +358,7 @@ def main():
     log("[bench] device:", info)
 
     if args.gemv_path != "default":
-        ex.set_option(ex.OPT_GEMV_LEAN, 1 if args.gemv_path == "lean" else 0)
+        ex.set_option(ex.OPT_GEMV_LEAN, {"general": 0, "lean": 1, "lean5": 2}[args.gemv_path])
     if args.dense_mfma:
         ex.set_option(ex.OPT_DENSE_MFMA, 1)
 

@@ -103,10 +103,12 @@ RT_HIP_API size_t rt_hip_type_block_elems(int ggml_type);
 /* ---- code-path switches (no reference counterpart; the nearest thing is the cargo feature set that picks a backend,
  *      Cargo.toml:166).  Where two kernels serve one call, the one with the longer record on the device is the default and
  *      the other is opt-in: process-wide, atomic, read at every launch, so a caller can run one call each way and compare.
- *      Initial values come from the environment (RUSTORCH_HIP_GEMV_LEAN, RUSTORCH_HIP_DENSE_MFMA: "1" switches on).
+ *      Initial values come from the environment (RUSTORCH_HIP_GEMV_LEAN, RUSTORCH_HIP_DENSE_MFMA: the value as one digit).
  *      Unknown options and values are refused with RT_HIP_ERR_INVALID_ARG. */
 typedef enum {
-    RT_HIP_OPT_GEMV_LEAN = 1,  /* 1: decode GEMV launches whose problems are all Q4_K / Q6_K / Q8_0 / Q4_0 take the lean kernel; 0 (default): the general one */
+    RT_HIP_OPT_GEMV_LEAN = 1,  /* 1: decode GEMV launches whose problems are all Q4_K / Q6_K / Q8_0 / Q4_0 take the lean kernel; 2: the same, and
+                                * launches without a gate / up pair problem run it with five waves per SIMD (640-thread workgroups);
+                                * 0 (default): the general kernel */
     RT_HIP_OPT_DENSE_MFMA = 2  /* 1: dense f32 products in whole 16-byte pieces take the f32 matrix-core kernel; 0 (default): the LDS-tiled one */
 } rt_hip_option;
 RT_HIP_API int rt_hip_set_option(rt_hip_ctx *ctx, int option, int value);

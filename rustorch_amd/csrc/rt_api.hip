@@ -45,20 +45,21 @@ const char *option_env(int option) {
     }
 }
 }  // namespace
+static int option_max(int option) { return option == RT_HIP_OPT_GEMV_LEAN ? 2 : 1; }
 int path_option(int option) {
     const char *env = option_env(option);
     if (!env) return -1;
     int v = g_option[option].load(std::memory_order_relaxed);
     if (v < 0) {
-        const char *e = getenv(env);
-        v = (e && e[0] == '1' && e[1] == 0) ? 1 : 0;
+        const char *e = getenv(env);      // one digit within the option's range, anything else counts as 0
+        v = (e && e[0] >= '0' && e[0] <= '0' + option_max(option) && e[1] == 0) ? e[0] - '0' : 0;
         int expected = -1;
         if (!g_option[option].compare_exchange_strong(expected, v, std::memory_order_relaxed)) v = expected;      // a set_option got there first
     }
     return v;
 }
 bool set_path_option(int option, int value) {
-    if (!option_env(option) || (value != 0 && value != 1)) return false;
+    if (!option_env(option) || value < 0 || value > option_max(option)) return false;
     g_option[option].store(value, std::memory_order_relaxed);
     return true;
 }

@@ -20,14 +20,16 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
 }
 
 // The same launch for problems that are all in the benchmark's four formats: the lean code path, R rows per step (the
-// gate / up pair form always takes a pair).
-template <int THREADS, int R>
-__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void qgemv_lean_kernel(GemvArgs a) {
+// gate / up pair form always takes a pair).  PAIR: the kernel contains the pair form.  WPE: waves per SIMD the register
+// allocation is made for -- 4 (128 registers), or 5 (96 registers; the form without the pair form fits, with 640-thread
+// workgroups two of which fill a compute unit's twenty wave slots).
+template <int THREADS, int R, bool PAIR, int WPE>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void qgemv_lean_kernel(GemvArgs a) {
     RT_DYN_LDS(uint4, lds4);
     __shared__ float red[THREADS / 64];
     const int wg = blockIdx.x;
     RT_GEMV_PICK_PROBLEM(a, wg, P);
-    lean_dispatch<R>(P, wg - P.tile0, P.rows_per_tile, blockIdx.y, reinterpret_cast<uint32_t *>(lds4), red);
+    lean_dispatch<R, PAIR>(P, wg - P.tile0, P.rows_per_tile, blockIdx.y, reinterpret_cast<uint32_t *>(lds4), red);
 }
 
 }  // namespace
@@ -36,7 +38,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
 // every launch otherwise.
 static bool plan_launch(GemvArgs &a, int batch, GemvPlan &pl) {
     GemvPlanHints hints;
-    hints.lean = path_option(RT_HIP_OPT_GEMV_LEAN) == 1 ? 1 : 0;
+    const int lean = path_option(RT_HIP_OPT_GEMV_LEAN);
+    hints.lean = lean >= 1 ? 1 : 0;
+    hints.five_waves = lean == 2 ? 1 : 0;
     return plan_qgemv(a, batch, pl, hints);
 }
 
@@ -44,7 +48,8 @@ static bool plan_launch(GemvArgs &a, int batch, GemvPlan &pl) {
 bool describe_qgemv(GemvArgs &a, int batch, char *out, size_t out_bytes) {
     GemvPlan pl;
     if (!plan_launch(a, batch, pl)) return false;
-    int n = pl.lean ? snprintf(out, out_bytes, "qgemv_lean_kernel<%d,1>", pl.threads) : snprintf(out, out_bytes, "qgemv_kernel<%d>", pl.threads);
+    int n = pl.lean ? snprintf(out, out_bytes, "qgemv_lean_kernel<%d,1,%s,%d>", pl.threads, pl.pair ? "true" : "false", pl.threads == 640 ? 5 : 4)
+                    : snprintf(out, out_bytes, "qgemv_kernel<%d>", pl.threads);
     if (n < 0 || (size_t)n >= out_bytes) return true;
     n += snprintf(out + n, out_bytes - n, " grid %dx%d lds %zu%s shares", pl.wgs, batch, pl.lds, pl.lean ? "" : (pl.r2 ? " two rows per step" : " one row per step"));
     for (int i = 0; i < a.n && (size_t)n < out_bytes; i++)
@@ -66,8 +71,11 @@ hipError_t launch_qgemv(hipStream_t s, GemvArgs &a, int batch) {
         if (e != hipSuccess) return e;
     }
     if (pl.lean) {      // the planner gives this path one row per step
-        if (pl.threads == 512) qgemv_lean_kernel<512, 1><<<grid, 512, lds, s>>>(a);
-        else qgemv_lean_kernel<1024, 1><<<grid, 1024, lds, s>>>(a);
+        if (pl.threads == 640) qgemv_lean_kernel<640, 1, false, 5><<<grid, 640, lds, s>>>(a);      // only planned without a pair problem
+        else if (pl.threads == 512 && pl.pair) qgemv_lean_kernel<512, 1, true, 4><<<grid, 512, lds, s>>>(a);
+        else if (pl.threads == 512) qgemv_lean_kernel<512, 1, false, 4><<<grid, 512, lds, s>>>(a);
+        else if (pl.pair) qgemv_lean_kernel<1024, 1, true, 4><<<grid, 1024, lds, s>>>(a);
+        else qgemv_lean_kernel<1024, 1, false, 4><<<grid, 1024, lds, s>>>(a);
     } else if (pl.threads == 512) qgemv_kernel<512><<<grid, 512, lds, s>>>(a, pl.r2);
     else qgemv_kernel<1024><<<grid, 1024, lds, s>>>(a, pl.r2);
     return hipGetLastError();

@@ -179,8 +179,11 @@ __device__ __forceinline__ float lean_dot(const LeanLane<RT_GGML_Q4_0> &, const 
 // weights stay in flight behind it (requested the other way round, the wait for x would also be a wait for them, and
 // nothing would be on its way while the workgroup stages).  Values, arithmetic and LDS layout are those of stage_x.
 struct LeanStage {
-    static constexpr int NBQ = 6;      // trips of the ready-made form held in registers (5 words each)
-    static constexpr int NBF = 3;      // trips of the f32 forms (a float4 of x and one of gamma each)
+    // 4 and 2 trips hold a whole row of up to 8192 elements with 512 threads (10 240 with 640); longer rows finish in the
+    // loops below.  With 6 and 3 the kernel without the pair form needs 100 registers, with 4 and 2 it needs 91: under the 96
+    // that five waves per SIMD leave each wave.
+    static constexpr int NBQ = 4;      // trips of the ready-made form held in registers (5 words each)
+    static constexpr int NBF = 2;      // trips of the f32 forms (a float4 of x and one of gamma each)
     uint32_t h[NBQ], l[NBQ];
     float s[NBQ], b0[NBQ], b1[NBQ];
     float4 v[NBF], g[NBF];
@@ -518,9 +521,12 @@ __device__ __forceinline__ bool lean_type(int type) {
     return type == RT_GGML_Q4_K || type == RT_GGML_Q6_K || type == RT_GGML_Q8_0 || type == RT_GGML_Q4_0;
 }
 
-template <int R>
+// PAIR = false leaves the gate / up pair form out of the kernel (the launcher picks it when no problem of the launch has
+// the SwiGLU epilogue): the pair form holds two rows of weights twice over and sets the register budget of a kernel that
+// contains it, whether a launch reaches it or not.
+template <int R, bool PAIR>
 __device__ __forceinline__ void lean_dispatch(const GemvProb &P, int wg, int n_wg, int m, uint32_t *lds, float *red) {
-    if (P.epi == kEpiSwiglu) {
+    if (PAIR && P.epi == kEpiSwiglu) {
         switch (P.type) {
         case RT_GGML_Q4_K: lean_problem<RT_GGML_Q4_K, 2, true>(P, wg, n_wg, m, lds, red); break;
         case RT_GGML_Q6_K: lean_problem<RT_GGML_Q6_K, 2, true>(P, wg, n_wg, m, lds, red); break;

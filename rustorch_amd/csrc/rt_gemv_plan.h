@@ -16,7 +16,8 @@ namespace rt {
 #endif
 
 struct GemvPlan {
-    int threads = 0;      // workgroup size: 512 or 1024
+    int threads = 0;      // workgroup size: 512 or 1024 (640: the lean path's five-waves-per-SIMD form)
+    bool pair = false;    // some problem has the gate / up pair (SwiGLU) epilogue
     int r2 = 0;           // two rows per wave step (else one)
     int wgs = 0;          // grid.x
     size_t lds = 0;       // launch-sized LDS
@@ -28,6 +29,7 @@ struct GemvPlan {
 struct GemvPlanHints {
     int threads = -1, r2 = -1, budget = -1;
     int lean = -1;        // 0: never the lean path; 1 or -1: wherever every problem of the launch qualifies
+    int five_waves = 0;   // 1: lean launches without a pair problem use 640-thread workgroups, two per compute unit
 };
 
 // Gives every problem a share of the workgroups in proportion to its weight bytes (tile0 = first workgroup,
@@ -52,10 +54,13 @@ inline bool plan_qgemv(GemvArgs &a, int batch, GemvPlan &pl, const GemvPlanHints
         lean = lean && (p.res == nullptr || p.res == p.y) &&
                (p.type == RT_GGML_Q4_K || p.type == RT_GGML_Q6_K || p.type == RT_GGML_Q8_0 || p.type == RT_GGML_Q4_0);
     }
-    // 16 resident waves per CU over 256 CUs, as one or two workgroups
-    const int threads = hints.threads > 0 ? hints.threads : (total_bytes >= RT_GEMV_BIG_BYTES ? 512 : 1024);
+    bool pair = false;
+    for (int i = 0; i < a.n; i++) pair = pair || a.p[i].epi == kEpiSwiglu;
+    // 16 resident waves per CU over 256 CUs, as one or two workgroups; or 20 as two workgroups of ten
+    const bool five = lean && !pair && hints.five_waves == 1;
+    const int threads = hints.threads > 0 ? hints.threads : (five ? 640 : (total_bytes >= RT_GEMV_BIG_BYTES ? 512 : 1024));
     const int waves = threads / 64;
-    int budget = hints.budget > 0 ? hints.budget : 256 * (1024 / threads) / batch;
+    int budget = hints.budget > 0 ? hints.budget : 256 * (threads == 1024 ? 1 : 2) / batch;
     if (budget < a.n) budget = a.n;
     // General path: two rows per wave step once every wave has at least three steps of work, else one (two rows share one
     // read of x from LDS).  Lean path: one row per step at every size -- measured on the layer workload and on single
@@ -164,7 +169,7 @@ inline bool plan_qgemv(GemvArgs &a, int batch, GemvPlan &pl, const GemvPlanHints
         }
     }
     lds = lds_all;
-    pl.threads = threads; pl.r2 = r2; pl.wgs = wgs; pl.lds = lds; pl.lean = lean;
+    pl.threads = threads; pl.r2 = r2; pl.wgs = wgs; pl.lds = lds; pl.lean = lean; pl.pair = pair;
     return true;
 }
 

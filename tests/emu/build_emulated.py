@@ -154,6 +154,7 @@ SANITIZERS = {
     "address": ["-fsanitize=address,alignment,bounds,shift-exponent,signed-integer-overflow,float-cast-overflow,integer-divide-by-zero",
                 "-fno-sanitize-recover=all", "-shared-libasan"],
     "thread": ["-fsanitize=thread", "-shared-libsan", "-mllvm", "-tsan-instrument-func-entry-exit=0"],
+    "none": [],        # no checks: several times faster, for looking at the numerics of sizes the checked builds take hours over
 }
 
 
@@ -196,6 +197,8 @@ def build(out_dir: Path, verbose: bool = False, sanitizer: str = "address") -> P
 
 
 def sanitizer_runtime(sanitizer: str = "address") -> str:
+    if sanitizer == "none":
+        return ""
     name = {"address": "asan", "thread": "tsan"}[sanitizer]
     return subprocess.run([CLANG, "-print-file-name=libclang_rt.%s-x86_64.so" % name], capture_output=True, text=True, check=True).stdout.strip()
 
@@ -216,13 +219,15 @@ def environment(so: Path, sanitizer: str = "address") -> dict:
 
 if __name__ == "__main__":
     if len(sys.argv) < 2:
-        sys.exit("usage: python tests/emu/build_emulated.py OUT_DIR [--races] [--pytest PYTEST_ARGS... | --run SCRIPT ARGS...]\n"
+        sys.exit("usage: python tests/emu/build_emulated.py OUT_DIR [--races | --unchecked] [--pytest PYTEST_ARGS... | --run SCRIPT ARGS...]\n"
                  "  --races: the ThreadSanitizer build (a wave is a thread: unordered accesses of two waves are reported)\n"
+                 "  --unchecked: no sanitizer (faster; numerics only)\n"
                  "  builds the emulated library into OUT_DIR; with --pytest, then runs `pytest -m gpu PYTEST_ARGS` against it;\n"
                  "  with --run, a Python script (tests/emu/fuzz_shapes.py for one)")
-    kind = "thread" if "--races" in sys.argv else "address"
-    if "--races" in sys.argv:
-        sys.argv.remove("--races")
+    kind = "thread" if "--races" in sys.argv else ("none" if "--unchecked" in sys.argv else "address")
+    for flag in ("--races", "--unchecked"):
+        if flag in sys.argv:
+            sys.argv.remove(flag)
     lib = build(Path(sys.argv[1]), verbose="--pytest" not in sys.argv and "--run" not in sys.argv, sanitizer=kind)
     print(lib)
     if "--run" in sys.argv:

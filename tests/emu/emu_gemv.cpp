@@ -135,8 +135,9 @@ int run_case(const Case &c) {
                 const int wg = (int)blockIdx.x;
                 RT_GEMV_PICK_PROBLEM(a, wg, P);
                 if (path == 0) gemv_dispatch<false, true>(P, wg - P.tile0, P.rows_per_tile, m, pl.r2 != 0, lds, red);
-                else if (pl.r2) lean_dispatch<2>(P, wg - P.tile0, P.rows_per_tile, m, lds, red);
-                else lean_dispatch<1>(P, wg - P.tile0, P.rows_per_tile, m, lds, red);
+                else if (pl.r2) lean_dispatch<2, true>(P, wg - P.tile0, P.rows_per_tile, m, lds, red);
+                else if (pl.pair) lean_dispatch<1, true>(P, wg - P.tile0, P.rows_per_tile, m, lds, red);       // as the launcher: the kernel without
+                else lean_dispatch<1, false>(P, wg - P.tile0, P.rows_per_tile, m, lds, red);                   // the pair form when no problem is a pair
             });
             if (!ok) { printf("%s: path %d stalled\n", c.name, path); rc = 1; }
         }
@@ -224,8 +225,8 @@ int run_group(const char *name, const std::vector<GroupSpec> &specs, int budget)
             uint32_t *lds = reinterpret_cast<uint32_t *>(lds4);
             const int wg = (int)blockIdx.x;
             RT_GEMV_PICK_PROBLEM(a, wg, P);
-            if (pl.r2) lean_dispatch<2>(P, wg - P.tile0, P.rows_per_tile, 0, lds, red);
-            else lean_dispatch<1>(P, wg - P.tile0, P.rows_per_tile, 0, lds, red);
+            if (pl.r2) lean_dispatch<2, true>(P, wg - P.tile0, P.rows_per_tile, 0, lds, red);
+            else lean_dispatch<1, false>(P, wg - P.tile0, P.rows_per_tile, 0, lds, red);
         });
         if (!ok) { printf("%s: stalled\n", name); rc = 1; }
     };
@@ -325,6 +326,12 @@ int main(int argc, char **argv) {
         { "q4k 13x8192 rms, one row per step, residual", Q4K, 13, 8192, kStageRms, kEpiStore, true, 512, 0, 3, 1 },
         { "q8_0 9x4096 f32, one row per step, two vectors", Q80, 9, 4096, kStageF32, kEpiStore, false, 512, 0, 1, 2 },
         { "q4_0 5x11008 xq, planner's own choice", Q40, 5, 11008, kStageXq, kEpiStore, false, -1, -1, 2, 1 },
+        // 640-thread workgroups (ten waves: the five-waves-per-SIMD form of the lean path)
+        { "q4k 23x4096 xq, 640 threads", Q4K, 23, 4096, kStageXq, kEpiStore, false, 640, 0, 2, 1 },
+        { "q6k 21x11008 rms, 640 threads, residual (row longer than the staged trips)", Q6K, 21, 11008, kStageRms, kEpiStore, true, 640, 0, 2, 1 },
+        { "q4k 11x11008 xq, 640 threads", Q4K, 11, 11008, kStageXq, kEpiStore, false, 640, 0, 1, 1 },
+        { "q8_0 5x96 f32, 640 threads", Q80, 5, 96, kStageF32, kEpiStore, false, 640, 0, 1, 2 },
+        { "q4_0 9x11008 f32, 640 threads", Q40, 9, 11008, kStageF32, kEpiStore, false, 640, 0, 2, 1 },
         // formats of the general path alone
         { "q8_1 5x96 f32", Q81, 5, 96, kStageF32, kEpiStore, false, -1, -1, 2, 1, false },
         { "q8_1 13x4096 rms, two rows, residual", Q81, 13, 4096, kStageRms, kEpiStore, true, 512, 1, 1, 1, false },

@@ -14,11 +14,12 @@ pytestmark = pytest.mark.gpu
 LEAN_TYPES = (8, 2, 12, 14)
 
 
-@pytest.fixture
-def lean(ex):
-    ex.set_option(ex.OPT_GEMV_LEAN, 1)
-    assert ex.get_option(ex.OPT_GEMV_LEAN) == 1
-    yield
+@pytest.fixture(params=[1, 2], ids=["lean", "lean-five-waves"])
+def lean(ex, request):
+    """1: the lean kernel at four waves per SIMD; 2: launches without a gate / up pair run its 640-thread, five-wave form."""
+    ex.set_option(ex.OPT_GEMV_LEAN, request.param)
+    assert ex.get_option(ex.OPT_GEMV_LEAN) == request.param
+    yield request.param
     ex.set_option(ex.OPT_GEMV_LEAN, 0)
 
 
@@ -35,7 +36,9 @@ def test_options_are_refused_when_unknown(ex):
     with pytest.raises(InvalidParameters):
         ex.set_option(99, 1)
     with pytest.raises(InvalidParameters):
-        ex.set_option(ex.OPT_GEMV_LEAN, 7)
+        ex.set_option(ex.OPT_GEMV_LEAN, 3)
+    with pytest.raises(InvalidParameters):
+        ex.set_option(ex.OPT_DENSE_MFMA, 2)
     with pytest.raises(InvalidParameters):
         ex.get_option(0)
 
@@ -52,7 +55,8 @@ def test_lean_gemv_config_shapes(ex, orc, lean, name):
 
 
 @pytest.mark.parametrize("t,rows,cols", [(12, 4096, 4096), (14, 4096, 4096), (8, 4096, 2048), (2, 5504, 2048), (12, 77, 1024), (14, 5, 768), (8, 5, 96)])
-def test_lean_rows_of_one_pass_have_the_general_kernels_bits(ex, t, rows, cols):
+@pytest.mark.parametrize("value", [1, 2])
+def test_lean_rows_of_one_pass_have_the_general_kernels_bits(ex, t, rows, cols, value):
     """Same x layout and the same arithmetic per unit: a row of one pass (64 units: 4096 elements of Q4_K / Q6_K, 2048 of
     Q8_0 / Q4_0) must come out bit for bit as from the general kernel."""
     from rustorch_amd import synth
@@ -61,12 +65,13 @@ def test_lean_rows_of_one_pass_have_the_general_kernels_bits(ex, t, rows, cols):
     x = synth.normal(41, 2, 2 * cols).reshape(2, cols)
     ex.set_option(ex.OPT_GEMV_LEAN, 0)
     y_general = ex.qgemv(w, x)
-    ex.set_option(ex.OPT_GEMV_LEAN, 1)
+    ex.set_option(ex.OPT_GEMV_LEAN, value)
     try:
+        print("launch:", ex.qgemv_describe([w]), flush=True)
         y_lean = ex.qgemv(w, x)
     finally:
         ex.set_option(ex.OPT_GEMV_LEAN, 0)
-    print("lean vs general, type %d %d x %d: %d of %d elements differ" % (t, rows, cols, int((y_lean != y_general).sum()), y_lean.size), flush=True)
+    print("lean (%d) vs general, type %d %d x %d: %d of %d elements differ" % (value, t, rows, cols, int((y_lean != y_general).sum()), y_lean.size), flush=True)
     assert np.array_equal(y_lean, y_general)
 
 
@@ -87,6 +92,8 @@ def test_lean_long_rows_stay_within_the_held_bound_of_the_general_kernel(ex, orc
     ex.set_option(ex.OPT_GEMV_LEAN, 1)
     try:
         y_lean = ex.qgemv(w, x)
+        ex.set_option(ex.OPT_GEMV_LEAN, 2)
+        assert np.array_equal(ex.qgemv(w, x), y_lean)        # the cut of a launch (here: ten waves per workgroup) never changes a result
         other = ex.upload_qweight(12, 512, 4096, synth.blocks(12, 43, 3, 512, 4096))
         dx, dx2 = ex.to_device(x), ex.to_device(synth.normal(43, 4, 4096))
         dy, dy2 = ex.buffer(rows * 4), ex.buffer(512 * 4)
@@ -107,7 +114,7 @@ def test_lean_decode_steps_match_the_general_path_and_the_oracle(ex, orc):
     om = orc.OracleLlama(**cfg)
     toks = [3, 77, 100, 5, 319]
     logits = {}
-    for which in (0, 1):
+    for which in (0, 1, 2):
         ex.set_option(ex.OPT_GEMV_LEAN, which)
         try:
             gm = llama.HipLlama(ex, **cfg)
@@ -122,11 +129,11 @@ def test_lean_decode_steps_match_the_general_path_and_the_oracle(ex, orc):
         logits[which] = np.stack(out)
     want = om.forward(toks, 0)
     scale = np.abs(want).max(axis=1)[:, None]
-    for which in (0, 1):
+    for which in (0, 1, 2):
         err = np.abs(logits[which] - want).max()
         print("decode steps, lean %d: max |delta logit| %.3e (logit scale %.3e)" % (which, err, scale.max()), flush=True)
         assert np.all(np.abs(logits[which] - want) <= 1e-3 * scale + 1e-3)
-    assert np.all(np.abs(logits[1] - logits[0]) <= 2e-4 * scale + 1e-4)
+    assert np.all(np.abs(logits[1] - logits[0]) <= 2e-4 * scale + 1e-4) and np.all(np.abs(logits[2] - logits[0]) <= 2e-4 * scale + 1e-4)
 
 
 @pytest.mark.parametrize("batch,m,n,k", [(1, 128, 128, 16), (3, 200, 136, 72), (1, 130, 132, 20), (2, 64, 64, 260), (1, 257, 384, 128), (1, 96, 64, 64)])
