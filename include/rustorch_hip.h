@@ -72,6 +72,7 @@ typedef enum {
 typedef struct rt_hip_ctx rt_hip_ctx;         /* executor: device, stream, scratch */
 typedef struct rt_hip_qweight rt_hip_qweight; /* raw GGUF blocks resident in HBM */
 typedef struct rt_hip_llama rt_hip_llama;     /* weights + KV cache + decode-step state */
+typedef struct rt_hip_llama_batch rt_hip_llama_batch; /* KV caches and activations of several sequences decoded against one model */
 typedef struct rt_hip_event rt_hip_event;     /* timing marker on the context's stream */
 
 typedef struct {
@@ -288,6 +289,23 @@ RT_HIP_API int rt_hip_llama_logits(rt_hip_ctx *ctx, rt_hip_llama *m, float *logi
  * is not NULL -- teacher forcing).  out_tokens receives the n_steps picks.  Blocks at the end. */
 RT_HIP_API int rt_hip_llama_decode(rt_hip_ctx *ctx, rt_hip_llama *m, int first_token, int pos0, int n_steps,
                                    const int *forced, int *out_tokens);
+
+/* ---- several sequences at once: the generate loop (InferenceEngine::generate_with_gpt,
+ *      example-cli/src/model/inference.rs:135-192) run for up to 8 prompts side by side against one model's weights.  A
+ *      batch owns a cache of max_pos (1..8192) rows per sequence and the activations of one step; the model must outlive
+ *      it and must not change tensors while it exists.  One step feeds one token per sequence -- sequence i's token at
+ *      positions[i], which must equal the number of tokens fed to that sequence so far (sequences need not be at the same
+ *      position) -- and runs every weight matrix once for all sequences.  tokens[i] < 0 leaves sequence i idle for the
+ *      step (nothing is fed, its pick is reported as -1, its row of the logits is meaningless); at least one sequence must
+ *      be fed.  next_tokens (may be NULL; n_seq ints) receives the greedy picks (ties: lowest id) and makes the call block;
+ *      rt_hip_llama_batch_logits copies the [n_seq][vocab] logits of the last step to host.  reset forgets the cache of
+ *      sequence seq, or of every sequence when seq is -1 (a finished sequence's slot then takes a new prompt). */
+RT_HIP_API int rt_hip_llama_batch_create(rt_hip_ctx *ctx, rt_hip_llama *m, int n_seq, int max_pos, rt_hip_llama_batch **out);
+RT_HIP_API int rt_hip_llama_batch_destroy(rt_hip_ctx *ctx, rt_hip_llama_batch *b);
+RT_HIP_API int rt_hip_llama_batch_reset(rt_hip_ctx *ctx, rt_hip_llama_batch *b, int seq);
+RT_HIP_API int rt_hip_llama_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b, const int *tokens, const int *positions,
+                                       int *next_tokens);
+RT_HIP_API int rt_hip_llama_batch_logits(rt_hip_ctx *ctx, rt_hip_llama_batch *b, float *logits_host);
 
 /* ---- synthetic GGUF payloads (host only, no GPU needed): seeded, counter-based, so a tensor is a pure
  *      function of (seed, tensor_id).  Used by the tests, the bench and offline exercise of the CLI path. */

@@ -125,6 +125,12 @@ hipError_t launch_attn_decode_split(hipStream_t s, const float *q, const float *
                                     const float *inv_freq_dev, float *partials, float *out, uint8_t *xq);
 hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache,
                                 int pos0, size_t n_tok, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev);
+// several sequences in one step: row m of q / k / v is sequence m at position pos_rows_dev[m]; its cache starts m * seq_stride
+// elements into kcache / vcache
+hipError_t launch_rope_kv_rows(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache, const int *pos_rows_dev,
+                               size_t seq_stride, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev);
+hipError_t launch_attn_rows(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc, const int *pos_rows_dev, size_t seq_stride,
+                            int max_pos, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out);
 hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
                              const int *pos_dev, int n_pos, size_t n_queries, int n_heads, int n_kv_heads, int head_dim,
                              const float *inv_freq_dev, float *out, uint8_t *xq, bool fused);

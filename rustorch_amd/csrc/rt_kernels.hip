@@ -402,6 +402,98 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float *q, const float 
     }
 }
 
+// ---- several sequences in one step: row m of q / k / v belongs to sequence m, which has a position of its own
+// (pos_rows[m]) and a cache of its own (seq_stride elements after the one before it).
+// Rotate q in place, rotate k and store it and v as fp16 cache row pos_rows[m] of sequence m.  blockIdx.y = m.
+__global__ void rope_kv_rows_kernel(float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache, const int *pos_rows,
+                                    size_t seq_stride, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq) {
+    int half = head_dim / 2;
+    int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_heads * half) return;
+    int i = t % half;
+    const size_t row = (size_t)n_heads * head_dim, rowkv = (size_t)n_kv_heads * head_dim, m = blockIdx.y;
+    const int p = pos_rows[m];
+    float s, c;
+    sincosf((float)p * inv_freq[i], &s, &c);
+    float2 *qr = reinterpret_cast<float2 *>(q + m * row);
+    float2 qv = qr[t];
+    qr[t] = make_float2(qv.x * c - qv.y * s, qv.x * s + qv.y * c);
+    if (t >= n_kv_heads * half) return;          // fewer key / value heads than query heads
+    float2 kv = reinterpret_cast<const float2 *>(k + m * rowkv)[t];
+    float k0 = kv.x * c - kv.y * s, k1 = kv.x * s + kv.y * c;
+    float2 vv = reinterpret_cast<const float2 *>(v + m * rowkv)[t];
+    reinterpret_cast<uint32_t *>(kcache + m * seq_stride + (size_t)p * rowkv)[t] = (uint32_t)f2h_rne(k0) | ((uint32_t)f2h_rne(k1) << 16);
+    reinterpret_cast<uint32_t *>(vcache + m * seq_stride + (size_t)p * rowkv)[t] = (uint32_t)f2h_rne(vv.x) | ((uint32_t)f2h_rne(vv.y) << 16);
+}
+
+// One workgroup (256 threads) per (query head, sequence): the rotated query row m against rows [0, pos_rows[m]] of sequence
+// m's cache (the row of the step itself was stored by rope_kv_rows_kernel before).  Same arithmetic as the decode step's
+// kernel in its plain form: a thread per position for the scores (the whole dot in the thread), max-subtracted softmax over
+// the workgroup, values as 16-byte column chunks x position groups folded through LDS.  Dynamic LDS: max_pos floats.
+template <int HD>
+__global__ __launch_bounds__(256) void attn_rows_kernel(const float *q, const uint16_t *kc, const uint16_t *vc, const int *pos_rows,
+                                                        size_t seq_stride, int n_heads, int n_kv_heads, float *out) {
+    RT_DYN_LDS(float, sc);
+    __shared__ float red[4];
+    __shared__ __align__(16) float qs[HD];
+    __shared__ __align__(16) float part[2048];
+    constexpr int CH = HD / 8;          // 16-byte chunks per cache row of this head
+    constexpr int NG = 256 / CH;        // position groups in the value phase
+    const int h = blockIdx.x, tid = threadIdx.x;
+    const size_t m = blockIdx.y, row = (size_t)n_heads * HD, rowkv = (size_t)n_kv_heads * HD;
+    const int kvh = h / (n_heads / n_kv_heads);
+    const int n_pos = pos_rows[m] + 1;
+    kc += m * seq_stride + (size_t)kvh * HD;
+    vc += m * seq_stride + (size_t)kvh * HD;
+    const float scale = 1.0f / sqrtf((float)HD);
+    if (tid < HD) qs[tid] = q[m * row + (size_t)h * HD + tid];
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int j = tid; j < n_pos; j += 256) {
+        const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)j * rowkv);
+        float s = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < CH; cc++) {
+            float f[8];
+            unpack8(kr[cc], f);
+#pragma unroll
+            for (int e = 0; e < 8; e++) s += qs[8 * cc + e] * f[e];
+        }
+        s *= scale;
+        sc[j] = s;
+        mx = fmaxf(mx, s);
+    }
+    mx = block_max(mx, red);
+    float sum = 0.f;
+    for (int j = tid; j < n_pos; j += 256) {
+        float e = expf(sc[j] - mx);
+        sc[j] = e;
+        sum += e;
+    }
+    sum = block_sum(sum, red);
+    for (int j = tid; j < n_pos; j += 256) sc[j] = sc[j] / sum;
+    __syncthreads();
+    const int c = tid % CH, g = tid / CH;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] = 0.f;
+    for (int j = g; j < n_pos; j += NG) {
+        float f[8];
+        unpack8(reinterpret_cast<const uint4 *>(vc + (size_t)j * rowkv)[c], f);
+        const float p = sc[j];
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += p * f[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) part[g * HD + 8 * c + e] = acc[e];
+    __syncthreads();
+    if (tid < HD) {
+        float o = 0.f;
+        for (int gg = 0; gg < NG; gg++) o += part[gg * HD + tid];
+        out[m * row + (size_t)h * HD + tid] = o;
+    }
+}
+
 // ---- long contexts: the positions of a head are split over several workgroups
 // Workgroup (h, s) of the fused decode step covers positions [s * chunk, (s + 1) * chunk) of query head h and leaves
 // a partial result {m = max score, l = sum of exp(score - m), acc[HD] = sum of exp(score - m) * v} in
@@ -896,6 +988,26 @@ hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const f
     int pairs = n_heads * head_dim / 2;
     rope_kv_batch_kernel<<<dim3((unsigned)((pairs + 255) / 256), (unsigned)n_tok), 256, 0, s>>>(q, k, v, kcache, vcache, pos0, n_heads,
                                                                                                 n_kv_heads, head_dim, inv_freq_dev);
+    return hipGetLastError();
+}
+
+hipError_t launch_rope_kv_rows(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache, const int *pos_rows_dev,
+                               size_t seq_stride, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads != 0 || n_rows == 0 || n_rows > 65535) return hipErrorInvalidValue;
+    int pairs = n_heads * head_dim / 2;
+    rope_kv_rows_kernel<<<dim3((unsigned)((pairs + 255) / 256), (unsigned)n_rows), 256, 0, s>>>(q, k, v, kcache, vcache, pos_rows_dev, seq_stride,
+                                                                                                n_heads, n_kv_heads, head_dim, inv_freq_dev);
+    return hipGetLastError();
+}
+
+hipError_t launch_attn_rows(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc, const int *pos_rows_dev, size_t seq_stride,
+                            int max_pos, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads != 0 || n_rows == 0 || n_rows > 65535 || max_pos <= 0 || max_pos > 8192) return hipErrorInvalidValue;
+    const size_t lds = (size_t)max_pos * sizeof(float);      // at most 32 KB beside the 9 KB of static arrays: inside the default 64 KB
+    dim3 grid((unsigned)n_heads, (unsigned)n_rows);
+    if (head_dim == 128) attn_rows_kernel<128><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out);
+    else if (head_dim == 64) attn_rows_kernel<64><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out);
+    else return hipErrorInvalidValue;
     return hipGetLastError();
 }
 

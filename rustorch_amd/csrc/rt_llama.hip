@@ -66,6 +66,20 @@ struct rt_hip_llama {
     std::vector<void *> allocs;
 };
 
+// Several sequences decoded side by side against one model's weights (the model's own cache serves its own single
+// sequence): every sequence has a position and a cache of its own, one step feeds one token per sequence and runs every
+// matrix once for all of them.
+struct rt_hip_llama_batch {
+    rt_hip_llama *m = nullptr;
+    int n_seq = 0, max_pos = 0;
+    std::vector<int> fed;                     // tokens fed so far, per sequence
+    uint16_t *kcache = nullptr, *vcache = nullptr;      // [layer][sequence][max_pos][kv_dim] fp16
+    float *x = nullptr, *x2 = nullptr, *n = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *a = nullptr, *g = nullptr, *u = nullptr;
+    float *logits = nullptr;                  // [sequence][vocab]
+    int *tok = nullptr, *pos = nullptr, *pick = nullptr;
+    std::vector<void *> allocs;
+};
+
 namespace {
 
 #ifndef RT_ATTN_SPLIT_MIN
@@ -404,6 +418,61 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
     return RT_HIP_OK;
 }
 
+// One token of each of b->n_seq sequences (tokens and positions already in b->tok / b->pos) through all layers.  The
+// matrices see the sequences as rows of one activation matrix -- from three rows on, Q4_K / Q6_K weights are streamed once
+// for all of them on the integer matrix cores (rt_gemv_mb.hip), q / k / v and gate / up sharing one quantization of the
+// rows; RoPE, the cache append and the attention are per sequence.  Block order as in enqueue_step.  Enqueue only.
+int enqueue_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b) {
+    rt_hip_llama *m = b->m;
+    hipStream_t s = ctx->stream;
+    const rt_hip_llama_config &c = m->cfg;
+    const size_t H = (size_t)c.hidden, F = (size_t)c.ffn, M = (size_t)b->n_seq;
+    const size_t seq_stride = (size_t)b->max_pos * m->kv_dim;
+    size_t need = rt::qgemv_mb_scratch_bytes(std::max(H, F));
+    for (int l = 0; l < c.n_layers; l++)
+        for (const auto *t : { &m->wq[l], &m->wk[l], &m->wv[l], &m->wo[l], &m->wgate[l], &m->wup[l], &m->wdown[l] })
+            need = std::max(need, rt::qgemm_scratch_bytes(t->type, M, t->n_rows, t->n_cols));
+    need = std::max(need, rt::qgemm_scratch_bytes(m->output.type, M, m->output.n_rows, m->output.n_cols));
+    int rc = ensure_scratch(ctx, need);
+    if (rc) return rc;
+    float *x = b->x, *x2 = b->x2;
+    PrefillGemm gemm{ ctx, m };
+    RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, b->tok, M, c.vocab, x));
+    for (int l = 0; l < c.n_layers; l++) {
+        uint16_t *kc = b->kcache + (size_t)l * M * seq_stride;
+        uint16_t *vc = b->vcache + (size_t)l * M * seq_stride;
+        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->attn_norm[l], b->n, nullptr, M, H, c.rms_eps));
+        gemm.prepared = nullptr;
+        rt_hip_llama::T *qkv[3] = { &m->wq[l], &m->wk[l], &m->wv[l] };
+        float *qkv_y[3] = { b->q, b->k, b->v };
+        if ((rc = gemm.shared(qkv, qkv_y, 3, b->n, M))) return rc;
+        RT_TRY_HIP(ctx, rt::launch_rope_kv_rows(s, b->q, b->k, b->v, kc, vc, b->pos, seq_stride, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
+        RT_TRY_HIP(ctx, rt::launch_attn_rows(s, b->q, kc, vc, b->pos, seq_stride, b->max_pos, M, c.n_heads, m->n_kv, m->head_dim, b->a));
+        if ((rc = gemm(m->wo[l], b->a, M, x2, x))) return rc;
+        std::swap(x, x2);
+        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->ffn_norm[l], b->n, nullptr, M, H, c.rms_eps));
+        gemm.prepared = nullptr;
+        rt_hip_llama::T *gu[2] = { &m->wgate[l], &m->wup[l] };
+        float *gu_y[2] = { b->g, b->u };
+        if ((rc = gemm.shared(gu, gu_y, 2, b->n, M))) return rc;
+        RT_TRY_HIP(ctx, rt::launch_swiglu(s, b->g, b->u, b->g, nullptr, M * F));
+        gemm.prepared = nullptr;
+        if ((rc = gemm(m->wdown[l], b->g, M, x2, x))) return rc;
+        std::swap(x, x2);
+    }
+    RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->out_norm, b->n, nullptr, M, H, c.rms_eps));
+    gemm.prepared = nullptr;
+    if ((rc = gemm(m->output, b->n, M, b->logits, nullptr))) return rc;
+    for (size_t i = 0; i < M; i++)
+        RT_TRY_HIP(ctx, rt::launch_argmax(s, b->logits + i * (size_t)c.vocab, (size_t)c.vocab, b->pick + i));
+    return RT_HIP_OK;
+}
+
+void free_batch(rt_hip_llama_batch *b) {
+    for (void *p : b->allocs) (void)hipFree(p);
+    b->allocs.clear();
+}
+
 }  // namespace
 
 extern "C" {
@@ -707,6 +776,105 @@ int rt_hip_llama_decode(rt_hip_ctx *ctx, rt_hip_llama *m, int first_token, int p
     }
     m->n_fed = pos0 + n_steps;
     RT_TRY_HIP(ctx, hipMemcpyAsync(out_tokens, m->out_tokens_dev, (size_t)n_steps * sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+    RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_batch_create(rt_hip_ctx *ctx, rt_hip_llama *m, int n_seq, int max_pos, rt_hip_llama_batch **out) {
+    if (!ctx || !m || !out) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_batch_create: NULL argument");
+    *out = nullptr;
+    RT_REQUIRE(ctx, n_seq >= 1 && n_seq <= 8, RT_HIP_ERR_SHAPE, "a batch holds 1..8 sequences, got %d", n_seq);
+    RT_REQUIRE(ctx, max_pos >= 1 && max_pos <= 8192, RT_HIP_ERR_SHAPE, "max_pos=%d outside 1..8192", max_pos);
+    RT_REQUIRE(ctx, prefill_batchable(m), RT_HIP_ERR_SHAPE, "head_dim=%d (64 or 128 supported)", m->head_dim);
+    Guard g(ctx);
+    rt_hip_llama_batch *b = new (std::nothrow) rt_hip_llama_batch();
+    if (!b) return fail(ctx, RT_HIP_ERR_OOM, "host allocation failed");
+    b->m = m; b->n_seq = n_seq; b->max_pos = max_pos;
+    b->fed.assign((size_t)n_seq, 0);
+    const rt_hip_llama_config &c = m->cfg;
+    const size_t L = (size_t)c.n_layers, H = (size_t)c.hidden, F = (size_t)c.ffn, V = (size_t)c.vocab, M = (size_t)n_seq, P = (size_t)max_pos;
+    hipError_t e = hipSuccess;
+    auto A = [&](void **p, size_t bytes) {
+        if (e != hipSuccess) return;
+        e = hipMalloc(p, bytes ? bytes : 1);
+        if (e == hipSuccess) b->allocs.push_back(*p);
+    };
+    A((void **)&b->kcache, L * M * P * m->kv_dim * 2); A((void **)&b->vcache, L * M * P * m->kv_dim * 2);
+    A((void **)&b->x, M * H * 4); A((void **)&b->x2, M * H * 4); A((void **)&b->n, M * H * 4); A((void **)&b->q, M * H * 4);
+    A((void **)&b->k, M * m->kv_dim * 4); A((void **)&b->v, M * m->kv_dim * 4); A((void **)&b->a, M * H * 4);
+    A((void **)&b->g, M * F * 4); A((void **)&b->u, M * F * 4); A((void **)&b->logits, M * V * 4);
+    A((void **)&b->tok, M * sizeof(int)); A((void **)&b->pos, M * sizeof(int)); A((void **)&b->pick, M * sizeof(int));
+    if (e != hipSuccess) { free_batch(b); delete b; return hip_fail(ctx, e, "llama_batch_create"); }
+    *out = b;
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_batch_destroy(rt_hip_ctx *ctx, rt_hip_llama_batch *b) {
+    if (!b) return RT_HIP_OK;
+    if (!ctx) return fail(nullptr, RT_HIP_ERR_INVALID_ARG, "ctx is NULL");
+    Guard g(ctx);
+    (void)hipStreamSynchronize(ctx->stream);
+    free_batch(b);
+    delete b;
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_batch_reset(rt_hip_ctx *ctx, rt_hip_llama_batch *b, int seq) {
+    if (!ctx || !b) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_batch_reset: NULL argument");
+    RT_REQUIRE(ctx, seq >= -1 && seq < b->n_seq, RT_HIP_ERR_INVALID_ARG, "sequence %d of %d", seq, b->n_seq);
+    Guard g(ctx);
+    RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (seq < 0) b->fed.assign((size_t)b->n_seq, 0);
+    else b->fed[(size_t)seq] = 0;
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b, const int *tokens, const int *positions, int *next_tokens) {
+    if (!ctx || !b || !tokens || !positions) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_batch_step: NULL argument");
+    rt_hip_llama *m = b->m;
+    int tok[8], pos[8], active = 0;
+    for (int i = 0; i < b->n_seq; i++) {
+        const int fed = b->fed[(size_t)i];
+        if (tokens[i] < 0) {
+            // idle this step: the row still runs (token 0 at the row the sequence would write next, which its next real token
+            // overwrites); nothing is counted and its pick is reported as -1
+            tok[i] = 0;
+            pos[i] = std::min(fed, b->max_pos - 1);
+            continue;
+        }
+        RT_REQUIRE(ctx, tokens[i] < m->cfg.vocab, RT_HIP_ERR_INVALID_ARG, "sequence %d: token %d outside the vocabulary of %d", i, tokens[i], m->cfg.vocab);
+        RT_REQUIRE(ctx, positions[i] == fed, RT_HIP_ERR_INVALID_ARG, "sequence %d: pos=%d but %d tokens have been fed", i, positions[i], fed);
+        RT_REQUIRE(ctx, positions[i] < b->max_pos, RT_HIP_ERR_SHAPE, "sequence %d: pos=%d reaches max_pos=%d", i, positions[i], b->max_pos);
+        tok[i] = tokens[i];
+        pos[i] = positions[i];
+        active++;
+    }
+    RT_REQUIRE(ctx, active > 0, RT_HIP_ERR_INVALID_ARG, "batch step: every sequence is idle");
+    int rc = check_complete(ctx, m);
+    if (rc) return rc;
+    Guard g(ctx);
+    const size_t bytes = (size_t)b->n_seq * sizeof(int);
+    // (pageable host memory: the copies have left tok / pos when the calls return)
+    RT_TRY_HIP(ctx, hipMemcpyAsync(b->tok, tok, bytes, hipMemcpyHostToDevice, ctx->stream));
+    RT_TRY_HIP(ctx, hipMemcpyAsync(b->pos, pos, bytes, hipMemcpyHostToDevice, ctx->stream));
+    rc = enqueue_batch_step(ctx, b);
+    if (rc) return rc;
+    for (int i = 0; i < b->n_seq; i++)
+        if (tokens[i] >= 0) b->fed[(size_t)i]++;
+    if (next_tokens) {
+        RT_TRY_HIP(ctx, hipMemcpyAsync(next_tokens, b->pick, bytes, hipMemcpyDeviceToHost, ctx->stream));
+        RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        for (int i = 0; i < b->n_seq; i++)
+            if (tokens[i] < 0) next_tokens[i] = -1;
+    }
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_batch_logits(rt_hip_ctx *ctx, rt_hip_llama_batch *b, float *logits_host) {
+    if (!ctx || !b || !logits_host) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_batch_logits: NULL argument");
+    Guard g(ctx);
+    RT_TRY_HIP(ctx, hipMemcpyAsync(logits_host, b->logits, (size_t)b->n_seq * (size_t)b->m->cfg.vocab * sizeof(float), hipMemcpyDeviceToHost,
+                                   ctx->stream));
     RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return RT_HIP_OK;
 }

@@ -76,6 +76,83 @@ class HipLlama:
             pass
 
 
+class HipLlamaBatch:
+    """Up to 8 sequences decoded side by side against one model's weights (rt_hip_llama_batch_*): each sequence has its own
+    cache and position, a step feeds one token per sequence and streams every weight matrix once for all of them."""
+
+    def __init__(self, model: HipLlama, n_seq: int, max_pos: int):
+        self.model, self.ex, self.n_seq, self.max_pos = model, model.ex, n_seq, max_pos
+        self.h = C.c_void_p()
+        _lib.check(self.ex.lib.rt_hip_llama_batch_create(self.ex.ctx, model.h, n_seq, max_pos, C.byref(self.h)), self.ex.ctx)
+
+    def reset(self, seq: int = -1) -> None:
+        """Forget sequence `seq` (its slot can take a new prompt), or every sequence."""
+        _lib.check(self.ex.lib.rt_hip_llama_batch_reset(self.ex.ctx, self.h, seq), self.ex.ctx)
+
+    def step(self, tokens, positions, want_tokens: bool = True):
+        """tokens[i] at positions[i] for every sequence i (a negative token leaves the sequence idle for the step);
+        returns the greedy picks (-1 for idle sequences), or None."""
+        t = np.ascontiguousarray(np.asarray(tokens, dtype=np.int32))
+        p = np.ascontiguousarray(np.asarray(positions, dtype=np.int32))
+        if t.shape != (self.n_seq,) or p.shape != (self.n_seq,):
+            from .errors import ShapeMismatch
+            raise ShapeMismatch("batch step: %d tokens and %d positions for %d sequences" % (t.size, p.size, self.n_seq))
+        out = np.empty(self.n_seq, dtype=np.int32)
+        _lib.check(self.ex.lib.rt_hip_llama_batch_step(self.ex.ctx, self.h, t.ctypes.data_as(_lib.c_int_p), p.ctypes.data_as(_lib.c_int_p),
+                                                       out.ctypes.data_as(_lib.c_int_p) if want_tokens else None), self.ex.ctx)
+        return out if want_tokens else None
+
+    def logits(self) -> np.ndarray:
+        out = np.empty((self.n_seq, self.model.cfg.vocab), dtype=np.float32)
+        _lib.check(self.ex.lib.rt_hip_llama_batch_logits(self.ex.ctx, self.h, C.c_void_p(out.ctypes.data)), self.ex.ctx)
+        return out
+
+    def generate(self, prompts, max_new_tokens: int, eos_token: int | None = None):
+        """The generate loop (inference.rs:135-192) for n_seq prompts at once, greedy: feeds the prompts token by token
+        (a shorter prompt starts generating while longer ones are still being fed), stops a sequence at eos_token, after
+        max_new_tokens or at the end of its cache, and leaves finished sequences idle while the others go on.  Returns the
+        generated ids per sequence."""
+        prompts = [list(map(int, p)) for p in prompts]
+        if len(prompts) != self.n_seq or any(len(p) == 0 for p in prompts):
+            from .errors import ShapeMismatch
+            raise ShapeMismatch("generate: %d non-empty prompts wanted" % self.n_seq)
+        self.reset()
+        out = [[] for _ in prompts]
+        done = [False] * self.n_seq
+        cur = [p[0] for p in prompts]
+        pos = [0] * self.n_seq
+        while True:
+            for i in range(self.n_seq):
+                done[i] = done[i] or pos[i] >= self.max_pos
+            if all(done):
+                break
+            picks = self.step([-1 if done[i] else cur[i] for i in range(self.n_seq)], pos)
+            for i in range(self.n_seq):
+                if done[i]:
+                    continue
+                pos[i] += 1
+                if pos[i] < len(prompts[i]):
+                    cur[i] = prompts[i][pos[i]]                      # still feeding the prompt
+                    continue
+                tok = int(picks[i])
+                out[i].append(tok)
+                cur[i] = tok
+                if (eos_token is not None and tok == eos_token) or len(out[i]) >= max_new_tokens:
+                    done[i] = True
+        return out
+
+    def close(self) -> None:
+        if self.h and self.ex.ctx:
+            self.ex.lib.rt_hip_llama_batch_destroy(self.ex.ctx, self.h)
+            self.h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def synthetic_tensors(seed: int, n_layers: int, hidden: int, ffn: int, vocab: int, kv_dim: int | None = None):
     """Yield (slot, layer, ggml type, n_rows, n_cols, raw) of a random-init Llama: token embedding Q8_0,
     q/k/o/gate/up Q4_K, v/down and the output head Q6_K, RMSNorm weights f32 ~ 1 + N(0, 0.01)."""

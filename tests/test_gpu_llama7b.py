@@ -17,6 +17,7 @@ another rounding than the oracle's is one more such draw.  So the bound is held
 and the positions that exceed it are reported together with what the oracle's own draws did there.  Single-position checks
 (the prefill's last logits, the device loop's last logits) are asserted unless that position is sensitive in a stored
 draw or in this run's own stepping pass."""
+import os
 from pathlib import Path
 
 import numpy as np
@@ -24,7 +25,9 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-GOLD = Path(__file__).resolve().parent / "golden" / "llama7b_golden.npz"
+# RT_LLAMA_GOLDEN names another file of the same layout (make_llama7b_golden.py --small: a small model, to try this test's
+# own code where the full size is out of reach)
+GOLD = Path(os.environ.get("RT_LLAMA_GOLDEN") or Path(__file__).resolve().parent / "golden" / "llama7b_golden.npz")
 SENSITIVE_ABOVE = 0.25  # a position counts as sensitive when a conditioning draw moved the oracle's logits by more (in tolerances)
 MAX_OUTLIERS = 10       # of 256 positions that may exceed the tolerance in one pass (the oracle against itself: 1 to 5 per draw)
 
@@ -39,7 +42,8 @@ def test_full_size_model_matches_oracle_golden(ex):
           % (nl, h, f, v, n_prompt, n_pos - n_prompt, ids.size, g["top_ids"].shape[1]), flush=True)
     gm = llama.HipLlama(ex, nl, h, nh, f, v, n_pos)
     nbytes = llama.load_synthetic(gm, seed)
-    assert nbytes == 32 * 129_785_856 + 139_264_000 + 107_520_000
+    if (nl, h, f, v) == (32, 4096, 11008, 32000):
+        assert nbytes == 32 * 129_785_856 + 139_264_000 + 107_520_000
     tol_ids = 1e-3 * g["id_norm"] * np.sqrt(h)
     tol_top = 1e-3 * g["top_norm"] * np.sqrt(h)                 # [n_pos, n_top]
     moved = g["moved"].max(axis=0)                               # worst movement of the oracle's own logits per position, over the stored draws
