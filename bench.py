@@ -217,7 +217,26 @@ def bench_layer_batch8(ex, n_layers=4, reps=100):
             "launches_per_layer": 9}
 
 
-def bench_decode(ex, n_prompt, n_gen, shape="7b"):
+def bench_decode_batch(gm, n_seq, n_prompt, n_gen, vocab):
+    """Config C3's batch of eight as a loop: n_seq sequences decoded side by side against the model's weights (every matrix
+    streamed once per step for all of them), prompts of n_prompt tokens fed step by step, then n_gen greedy steps timed.
+    tokens/s counts the tokens of all sequences."""
+    from rustorch_amd import llama, synth
+    b = llama.HipLlamaBatch(gm, n_seq, n_prompt + n_gen)
+    prompts = [synth.tokens(SEED, 9500 + i, n_prompt, vocab) for i in range(n_seq)]
+    picks = None
+    for p in range(n_prompt):
+        picks = b.step([int(pr[p]) for pr in prompts], [p] * n_seq)
+    t0 = time.perf_counter()
+    for p in range(n_prompt, n_prompt + n_gen):
+        picks = b.step([int(t) for t in picks], [p] * n_seq)
+    dt = time.perf_counter() - t0
+    b.close()
+    return {"sequences": n_seq, "n_prompt": n_prompt, "n_generated": n_gen, "tokens_per_s": round(n_seq * n_gen / dt, 1),
+            "ms_per_step": round(1e3 * dt / n_gen, 4), "note": "one host round trip per step (the picks come back to be fed)"}
+
+
+def bench_decode(ex, n_prompt, n_gen, shape="7b", batch=0):
     from rustorch_amd import llama, synth
     sh = SHAPES[shape]
     NL, H, NH, NKV, F, V = sh["NL"], sh["H"], sh["NH"], sh["NKV"], sh["F"], sh["V"]
@@ -234,6 +253,7 @@ def bench_decode(ex, n_prompt, n_gen, shape="7b"):
     t0 = time.perf_counter()
     toks = gm.decode(int(prompt[-1]), n_prompt - 1, n_gen)
     t_dec = time.perf_counter() - t0
+    side_by_side = bench_decode_batch(gm, batch, 16, 64, V) if batch else None
     gm.close()
     kv_dim = NKV * (H // NH)
     per_layer = sum(t.row_bytes(c) * r for _, t, r, c in synth.layer_tensor_specs(H, F, kv_dim))
@@ -241,7 +261,7 @@ def bench_decode(ex, n_prompt, n_gen, shape="7b"):
     kv_avg = 2 * NL * kv_dim * 2 * (n_prompt + n_gen / 2)      # fp16 K and V rows read per token, averaged over the run
     return dict(shape=shape, tokens_per_s=n_gen / t_dec, ms_per_token=1e3 * t_dec / n_gen, prefill_tokens_per_s=(n_prompt - 1) / t_prefill,
                 bytes_per_token=int(tok_bytes + kv_avg), hbm_frac=(tok_bytes + kv_avg) * n_gen / t_dec / HBM_PEAK,
-                n_prompt=n_prompt, n_generated=n_gen, first_tokens=[int(t) for t in toks[:8]])
+                n_prompt=n_prompt, n_generated=n_gen, first_tokens=[int(t) for t in toks[:8]], **({"batch": side_by_side} if side_by_side else {}))
 
 
 def bench_prefill(ex, reps=20):
@@ -341,6 +361,8 @@ def main():
     ap.add_argument("--decode-prompt", type=int, default=128)
     ap.add_argument("--decode-gen", type=int, default=128)
     ap.add_argument("--decode-shape", choices=sorted(SHAPES), default="7b", help="model shape of the decode measurement (the benchmark's is 7b)")
+    ap.add_argument("--decode-batch", type=int, default=0,
+                    help="also decode this many sequences (1..8) side by side against the same model (rt_hip_llama_batch_*); off by default")
     ap.add_argument("--gemv-path", choices=("default", "general", "lean", "lean5"), default="default",
                     help="decode GEMV kernel of every leg: the library's default, the general kernel, the lean one, or the lean one with "
                          "five waves per SIMD where the launch allows it (rt_hip_set_option)")
@@ -425,7 +447,7 @@ def main():
         out["layer_batch8"] = bench_layer_batch8(ex)
         out["dense_f32"] = bench_dense_f32(ex)
     if not args.no_decode:
-        out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen, args.decode_shape)
+        out["decode"] = bench_decode(ex, args.decode_prompt, args.decode_gen, args.decode_shape, args.decode_batch)
     ex.close()
     if not args.no_cpu:
         wbytes, t1, tn, ncores = cpu_baseline(tensors, 3)

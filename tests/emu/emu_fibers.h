@@ -64,7 +64,14 @@ emu_switch_stack:
 namespace emu {
 
 enum State { RUNNABLE, AT_SYNC, AT_WAVE, AT_GATHER, AT_UNIFORM, SPIN, DONE };
-constexpr size_t kStack = 256 * 1024;      // above one guard page
+// EMU_STACK_BYTES: stack of a fiber (default 256 KB above one guard page).  EMU_STACK_ARENA = n: the stacks of up to n
+// fibers come out of one mapping without guard pages -- for grids of hundreds of thousands of fibers that are all alive at
+// once (a kernel whose workgroups wait for one another), where one mapping per fiber would exceed the kernel's limit on
+// mappings per process.
+#ifndef EMU_STACK_BYTES
+#define EMU_STACK_BYTES (256 * 1024)
+#endif
+constexpr size_t kStack = EMU_STACK_BYTES;
 
 struct Fiber {
     void *sp = nullptr;       // where the fiber's registers lie while it is not running
@@ -203,10 +210,21 @@ static char *take_stack() {
 #endif
         return s;
     }
+#ifdef EMU_STACK_ARENA
+    static char *arena = nullptr;
+    static size_t taken = 0;
+    if (!arena) {
+        arena = (char *)mmap(nullptr, (size_t)EMU_STACK_ARENA * kStack, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+        if (arena == (char *)MAP_FAILED) { perror("mmap"); exit(2); }
+    }
+    if (taken == (size_t)EMU_STACK_ARENA) { fprintf(stderr, "emu: more than EMU_STACK_ARENA fibers alive\n"); exit(2); }
+    return arena + kStack * taken++;
+#else
     char *s = (char *)mmap(nullptr, kStack + 4096, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
     if (s == (char *)MAP_FAILED) { perror("mmap"); exit(2); }
     mprotect(s, 4096, PROT_NONE);      // a fiber that outgrows its stack stops here instead of writing into another's
     return s + 4096;
+#endif
 }
 
 static void start_block(Block &b, int index) {

@@ -9,7 +9,9 @@ decode attention splits a head's positions over workgroups) and a way to cut a p
 take the batched pass, the grid-slice pass and the token-by-token pass, starting off multiples of 32), then steps a few
 tokens.  After every call the logits must be finite and within a loose multiple of
 the benchmark's bound of the oracle's -- the tiny models are ill conditioned in places, so this hunts for faults, NaNs and
-gross errors, not for the last bit -- and a second model fed token by token must agree with the first."""
+gross errors, not for the last bit -- and a second model fed token by token must agree with the first.  Last, a random
+number of sequences (1..8) is decoded side by side against the same weights (rt_hip_llama_batch_*), some of them starting
+late or sitting steps out, each against the oracle's forward of that sequence alone."""
 import sys
 
 import numpy as np
@@ -86,6 +88,37 @@ def one_case(ex, rng, seed):
     between = float((np.abs(g2.logits() - gm.logits()) / tol).max())
     say("   worst |delta| / bound: calls %.3f, token by token %.3f, between the two %.3f" % (worst, worst2, between))
     assert worst <= LOOSE and worst2 <= LOOSE and between <= LOOSE
+    # several sequences side by side against the same weights
+    n_seq = int(rng.integers(1, 9)); steps = int(rng.integers(3, 7))
+    seqs = [synth.tokens(seed, 500 + i, steps, vocab) for i in range(n_seq)]
+    wants = [om.forward(sq, 0) for sq in seqs]
+    start = [int(rng.integers(0, 3)) if i else 0 for i in range(n_seq)]      # sequence 0 always runs; the others may start late
+    b = llama.HipLlamaBatch(gm, n_seq, steps + 1)
+    fed = [0] * n_seq
+    worst3, step = 0.0, 0
+    while min(fed) < steps:
+        toks_b, pos_b = [], []
+        for i in range(n_seq):
+            idle = fed[i] >= steps or step < start[i] or (i and rng.random() < 0.15)
+            toks_b.append(-1 if idle else int(seqs[i][fed[i]])); pos_b.append(fed[i])
+        if all(t < 0 for t in toks_b):
+            toks_b[0] = int(seqs[0][min(fed[0], steps - 1)]) if fed[0] < steps else -1
+            if toks_b[0] < 0:
+                i = int(np.argmin(fed)); toks_b[i] = int(seqs[i][fed[i]])
+        picks = b.step(toks_b, pos_b)
+        lg = b.logits()
+        for i in range(n_seq):
+            if toks_b[i] < 0:
+                assert picks[i] == -1
+                continue
+            assert np.isfinite(lg[i]).all(), "batch step left non-finite logits for sequence %d" % i
+            assert picks[i] == int(np.argmax(lg[i]))
+            worst3 = max(worst3, float((np.abs(lg[i] - wants[i][fed[i]]) / tol).max()))
+            fed[i] += 1
+        step += 1
+    say("   %d sequences side by side, %d steps each (in %d batch steps): worst |delta| / bound %.3f" % (n_seq, steps, step, worst3))
+    assert worst3 <= LOOSE
+    b.close()
     gm.close(); g2.close()
 
 
