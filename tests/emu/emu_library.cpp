@@ -24,8 +24,8 @@ hipError_t hipMalloc(void **p, size_t n) {
     std::lock_guard<std::mutex> lock(g_mem_mu);
     *p = nullptr;
     if (n > kEmuDeviceBytes - g_mem_bytes) return hipErrorOutOfMemory;
-    *p = malloc(n ? n : 1);
-    if (!*p) return hipErrorOutOfMemory;
+    // 256-byte aligned like the device allocator's blocks (the launchers check the alignment of workspaces), exact size
+    if (posix_memalign(p, 256, n ? n : 1) != 0) { *p = nullptr; return hipErrorOutOfMemory; }
     memset(*p, 0xFF, n ? n : 1);      // undefined on the device; NaN patterns here, so that a read of it does not pass by luck
     g_mem[*p] = n;
     g_mem_bytes += n;

@@ -43,6 +43,8 @@ SELECTION = [
     "tests/test_gpu_gemm.py::test_three_to_fifteen_rows_go_eight_at_a_time[100-11008-12]",
     "tests/test_gpu_gemm.py::test_three_to_fifteen_rows_go_eight_at_a_time[100-11008-14]",
     "tests/test_gpu_llama.py::test_model_from_gguf_file_equals_direct_upload",
+    "tests/test_z_batch_decode.py::test_three_sequences_on_a_small_model",        # several sequences side by side
+    "tests/test_z_batch_decode.py::test_batch_arguments_are_checked",
 ]
 
 
@@ -66,7 +68,8 @@ RACE_SELECTION = [
     "tests/test_gpu_gemv.py::test_batches_of_two_to_eight_on_the_matrix_cores[300-11008-14]",
     "tests/test_z_optin_paths.py::test_dense_matmul_on_the_matrix_cores",
     "tests/test_z_optin_paths.py::test_lean_gemv_edge_inputs",
-    "tests/test_z_optin_paths.py::test_lean_gemv_config_shapes[C3_down]",
+    "tests/test_z_optin_paths.py::test_lean_gemv_config_shapes[lean-C3_down]",
+    "tests/test_z_optin_paths.py::test_lean_gemv_config_shapes[lean-five-waves-C3_down]",
     "tests/test_gpu_gemm.py::test_single_superblock_odd_counts_and_tiny_matrices",
     "tests/test_gpu_gemm.py::test_three_to_fifteen_rows_go_eight_at_a_time[100-11008-12]",
 ]

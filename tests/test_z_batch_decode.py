@@ -56,6 +56,28 @@ def test_batch_steps_match_the_oracle_and_the_single_sequence_step(ex, orc, n_se
     gm.close()
 
 
+def test_three_sequences_on_a_small_model(ex, orc):
+    """The whole step once at a size the CPU emulation of the library finishes in seconds: three rows, so the Q4_K / Q6_K
+    matrices take the matrix-core small-batch kernel."""
+    from rustorch_amd import llama
+    cfg = dict(n_layers=1, hidden=256, n_heads=2, ffn=256, vocab=64, max_pos=8)
+    gm, om, wn = build_pair(ex, orc, 59, **cfg)
+    seqs = sequences(59, 3, 4, cfg["vocab"])
+    want = [om.forward(s, 0) for s in seqs]
+    tol = logit_tol(wn, cfg["hidden"])
+    b = llama.HipLlamaBatch(gm, 3, 4)
+    ratios = []
+    for p in range(4):
+        picks = b.step([int(s[p]) for s in seqs], [p] * 3)
+        got = b.logits()
+        assert np.isfinite(got).all() and all(picks[i] == int(np.argmax(got[i])) for i in range(3))
+        ratios += [float((np.abs(got[i] - want[i][p]) / tol).max()) for i in range(3)]
+    print("small model, three sequences: median %.3f, max %.2f of the tolerance" % (np.median(ratios), max(ratios)), flush=True)
+    assert np.median(ratios) <= 0.1 and np.mean(np.array(ratios) <= 1) >= 0.9
+    b.close()
+    gm.close()
+
+
 def test_sequences_at_different_positions_and_refilled_slots(ex, orc):
     """Sequence 1 starts three steps after sequence 0 (idle steps), sequence 2 is reset in mid-run and takes a new prompt: every
     sequence's logits are those of that sequence fed alone."""
