@@ -187,7 +187,17 @@ template <> struct XRegs<RT_GGML_Q5_1> : XRegs<RT_GGML_Q4_0> {};
 //
 // The start is rounded down to a multiple of four bytes (rows of Q6_K at K = 11008 are 9030 bytes: only 2-byte aligned)
 // and the remainder goes into the scalar offset, with num_records lengthened by it: whether the range check counts the
-// scalar offset or not, every in-range lane passes it, and no lane gets more than 3 bytes past the piece.
+// scalar offset or not, every in-range lane passes it.  num_records is lengthened by kWindowSlack more, so that no rule a
+// range check may follow (the access as a whole, dword by dword, sub-dword loads widened to a dword) can refuse the last
+// bytes of a piece that is not a whole number of dwords -- a 2-byte scale at offset 9028 of a 9030-byte row.  A lane that
+// is out of range can then get kWindowSlack + 3 bytes past the piece and no further: inside the 64 bytes every upload
+// leaves behind a tensor.  (The CPU build of these sources sets the slack to zero: there a load ends the run the moment it
+// leaves the piece.)
+#ifdef RT_EMULATED
+constexpr uint32_t kWindowSlack = 0;
+#else
+constexpr uint32_t kWindowSlack = 16;
+#endif
 struct WRow {
     __amdgpu_buffer_rsrc_t rsrc;
     uint32_t soff;      // 0..3: what the rounding of the start took off
@@ -198,7 +208,7 @@ __device__ __forceinline__ WRow weight_window(const uint8_t *w, uint32_t nbytes,
     start = min(start, nbytes - span);      // unsigned: a start that went wrong in any direction lands inside the tensor
     const uint32_t rem = start & 3u;
     // raw buffer (stride 0), dword 3 as for 32-bit data
-    return WRow{ __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w) + (start - rem), 0, (int)(span + rem), 0x00020000), rem };
+    return WRow{ __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w) + (start - rem), 0, (int)(span + rem + kWindowSlack), 0x00020000), rem };
 }
 __device__ __forceinline__ uint4 bld16(WRow r, uint32_t off) {
     return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r.rsrc, off, r.soff, 0));

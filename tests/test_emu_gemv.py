@@ -19,7 +19,7 @@ def test_gemv_device_code_as_cpu_fibers_under_asan(tmp_path):
     obj = tmp_path / "rt_oracle.o"
     subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-fopenmp", "-c", str(ROOT / "oracle" / "rt_oracle.c"), "-o", str(obj)], check=True)
     exe = tmp_path / "emu_gemv"
-    subprocess.run([CLANG, "-std=c++17", "-O1", "-g", "-fsanitize=address", "-I", str(ROOT / "tests" / "emu"),
+    subprocess.run([CLANG, "-std=c++17", "-O1", "-g", "-fsanitize=address", "-DRT_EMULATED=1", "-I", str(ROOT / "tests" / "emu"),
                     "-I", str(ROOT / "rustorch_amd" / "csrc"), "-I", str(ROOT / "include"), str(ROOT / "tests" / "emu" / "emu_gemv.cpp"),
                     str(ROOT / "rustorch_amd" / "csrc" / "rt_synth.cpp"), str(obj), "-o", str(exe), "-fopenmp"], check=True)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")

@@ -17,7 +17,7 @@ def test_step_kernel_as_cpu_fibers_under_asan(tmp_path):
     obj = tmp_path / "rt_oracle.o"
     subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-fopenmp", "-c", str(ROOT / "oracle" / "rt_oracle.c"), "-o", str(obj)], check=True)
     exe = tmp_path / "emu_main"
-    subprocess.run([CLANG, "-std=c++17", "-O1", "-g", "-fsanitize=address", "-I", str(ROOT / "tests" / "emu"),
+    subprocess.run([CLANG, "-std=c++17", "-O1", "-g", "-fsanitize=address", "-DRT_EMULATED=1", "-I", str(ROOT / "tests" / "emu"),
                     "-I", str(ROOT / "rustorch_amd" / "csrc"), "-I", str(ROOT / "include"), str(ROOT / "tests" / "emu" / "emu_main.cpp"),
                     str(ROOT / "rustorch_amd" / "csrc" / "rt_synth.cpp"), str(obj), "-o", str(exe), "-fopenmp"], check=True)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
