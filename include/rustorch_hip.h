@@ -305,6 +305,11 @@ RT_HIP_API int rt_hip_llama_batch_destroy(rt_hip_ctx *ctx, rt_hip_llama_batch *b
 RT_HIP_API int rt_hip_llama_batch_reset(rt_hip_ctx *ctx, rt_hip_llama_batch *b, int seq);
 RT_HIP_API int rt_hip_llama_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b, const int *tokens, const int *positions,
                                        int *next_tokens);
+/* Feed n_tok (3 or more) tokens of sequence seq starting at pos0 (= the tokens fed to it so far) through the model's batched
+ * prefill passes (dense contractions on the matrix cores), into that sequence's cache; the other sequences are untouched.
+ * Its row of the logits then holds the last token's.  Blocks.  The call borrows the model's prefill workspace. */
+RT_HIP_API int rt_hip_llama_batch_prefill(rt_hip_ctx *ctx, rt_hip_llama_batch *b, int seq, const int *tokens, int n_tok,
+                                          int pos0);
 RT_HIP_API int rt_hip_llama_batch_logits(rt_hip_ctx *ctx, rt_hip_llama_batch *b, float *logits_host);
 
 /* ---- synthetic GGUF payloads (host only, no GPU needed): seeded, counter-based, so a tensor is a pure

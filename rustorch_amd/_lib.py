@@ -89,6 +89,7 @@ SIGNATURES = {
     "rt_hip_llama_batch_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
     "rt_hip_llama_batch_reset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "rt_hip_llama_batch_step": (C.c_int, [C.c_void_p, C.c_void_p, c_int_p, c_int_p, c_int_p]),
+    "rt_hip_llama_batch_prefill": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, c_int_p, C.c_int, C.c_int]),
     "rt_hip_llama_batch_logits": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "rt_synth_blocks": (C.c_int, [C.c_int, C.c_uint64, C.c_uint64, C.c_size_t, C.c_float, C.c_float, C.c_void_p]),
     "rt_synth_normal_f32": (C.c_int, [C.c_uint64, C.c_uint64, C.c_size_t, C.c_float, C.c_float, C.c_void_p]),

@@ -40,6 +40,10 @@ struct rt_hip_llama {
     std::vector<T> wq, wk, wv, wo, wgate, wup, wdown;
     std::vector<float *> attn_norm, ffn_norm;
     uint16_t *kcache = nullptr, *vcache = nullptr;
+    // the cache the batched prefill passes write and attend: the model's own ([layer][max_pos][kv_dim]), or for the length of one
+    // call a sequence of a batch object (rt_hip_llama_batch_prefill); layer l starts pf_layer_stride * l elements in
+    uint16_t *pf_kcache = nullptr, *pf_vcache = nullptr;
+    size_t pf_layer_stride = 0;
     float *x = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *g = nullptr, *u = nullptr, *logits = nullptr;
     uint8_t *xq_h = nullptr, *xq_a = nullptr, *xq_f = nullptr;
     float *inv_freq = nullptr;
@@ -341,8 +345,8 @@ int enqueue_prefill_chain(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
     rt::PlaneSum pending{ x, 0, 1 };             // what the next RMSNorm reads: first the embeddings themselves,
     const float *pending_res = nullptr;          // later the planes of a down-projection, to be added to x
     for (int l = 0; l < c.n_layers; l++) {
-        uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
-        uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
+        uint16_t *kc = m->pf_kcache + (size_t)l * m->pf_layer_stride;
+        uint16_t *vc = m->pf_vcache + (size_t)l * m->pf_layer_stride;
         rt::PlaneSum q, k, v, o, g, u, d;
         RT_TRY_HIP(ctx, rt::launch_xprep_rmsnorm(s, pending, pending_res, pending_res ? x : nullptr, m->attn_norm[l], c.rms_eps, M, H, m->pf_xp, m->pf_inv));
         if (same_kind(m->wq[l], m->wk[l])) {
@@ -393,8 +397,8 @@ int enqueue_prefill_batch(rt_hip_ctx *ctx, rt_hip_llama *m, size_t M, int pos0) 
     PrefillGemm gemm{ ctx, m };
     RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, m->pf_tok, M, c.vocab, x));
     for (int l = 0; l < c.n_layers; l++) {
-        uint16_t *kc = m->kcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
-        uint16_t *vc = m->vcache + (size_t)l * (size_t)c.max_pos * m->kv_dim;
+        uint16_t *kc = m->pf_kcache + (size_t)l * m->pf_layer_stride;
+        uint16_t *vc = m->pf_vcache + (size_t)l * m->pf_layer_stride;
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->attn_norm[l], m->pf_n, nullptr, M, H, c.rms_eps));
         gemm.prepared = nullptr;          // pf_n has new contents
         rt_hip_llama::T *qkv[3] = { &m->wq[l], &m->wk[l], &m->wv[l] };
@@ -512,6 +516,7 @@ int rt_hip_llama_create(rt_hip_ctx *ctx, const rt_hip_llama_config *cfg, rt_hip_
     m->attn_splits = cfg->max_pos >= RT_ATTN_SPLIT_MIN ? std::min(16, (cfg->max_pos + RT_ATTN_SPLIT_MIN / 4 - 1) / (RT_ATTN_SPLIT_MIN / 4)) : 1;
     A((void **)&m->attn_part, (size_t)cfg->n_heads * (size_t)m->attn_splits * (size_t)(hd + 2) * sizeof(float));
     A((void **)&m->kcache, L * P * m->kv_dim * 2); A((void **)&m->vcache, L * P * m->kv_dim * 2);
+    m->pf_kcache = m->kcache; m->pf_vcache = m->vcache; m->pf_layer_stride = P * m->kv_dim;
     A((void **)&m->x, H * 4); A((void **)&m->q, H * 4); A((void **)&m->k, H * 4); A((void **)&m->v, H * 4);
     A((void **)&m->g, F * 4); A((void **)&m->u, F * 4); A((void **)&m->logits, V * 4);
     A((void **)&m->xq_h, rt::xq_stride(H)); A((void **)&m->xq_a, rt::xq_stride(H)); A((void **)&m->xq_f, rt::xq_stride(F));
@@ -867,6 +872,54 @@ int rt_hip_llama_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b, const int *t
         for (int i = 0; i < b->n_seq; i++)
             if (tokens[i] < 0) next_tokens[i] = -1;
     }
+    return RT_HIP_OK;
+}
+
+int rt_hip_llama_batch_prefill(rt_hip_ctx *ctx, rt_hip_llama_batch *b, int seq, const int *tokens, int n_tok, int pos0) {
+    if (!ctx || !b || !tokens) return fail(ctx, RT_HIP_ERR_INVALID_ARG, "rt_hip_llama_batch_prefill: NULL argument");
+    rt_hip_llama *m = b->m;
+    RT_REQUIRE(ctx, seq >= 0 && seq < b->n_seq, RT_HIP_ERR_INVALID_ARG, "sequence %d of %d", seq, b->n_seq);
+    RT_REQUIRE(ctx, n_tok >= kPrefillMinRows, RT_HIP_ERR_SHAPE, "batch prefill takes %d tokens or more (fewer go through rt_hip_llama_batch_step), got %d",
+               kPrefillMinRows, n_tok);
+    RT_REQUIRE(ctx, pos0 == b->fed[(size_t)seq], RT_HIP_ERR_INVALID_ARG, "sequence %d: pos0=%d but %d tokens have been fed", seq, pos0, b->fed[(size_t)seq]);
+    RT_REQUIRE(ctx, pos0 + n_tok <= b->max_pos, RT_HIP_ERR_SHAPE, "pos0+n_tok=%d exceeds max_pos=%d", pos0 + n_tok, b->max_pos);
+    for (int i = 0; i < n_tok; i++)
+        RT_REQUIRE(ctx, tokens[i] >= 0 && tokens[i] < m->cfg.vocab, RT_HIP_ERR_INVALID_ARG, "token %d (index %d) outside the vocabulary", tokens[i], i);
+    int rc = check_complete(ctx, m);
+    if (rc) return rc;
+    Guard g(ctx);
+    rc = ensure_prefill_buffers(ctx, m, std::min((size_t)n_tok, kPrefillChunk));
+    if (rc) return rc;
+    // the model's own passes, writing and attending this sequence's cache for the length of the call
+    const size_t seq_stride = (size_t)b->max_pos * m->kv_dim;
+    m->pf_kcache = b->kcache + (size_t)seq * seq_stride;
+    m->pf_vcache = b->vcache + (size_t)seq * seq_stride;
+    m->pf_layer_stride = (size_t)b->n_seq * seq_stride;
+    struct Restore {
+        rt_hip_llama *m;
+        ~Restore() { m->pf_kcache = m->kcache; m->pf_vcache = m->vcache; m->pf_layer_stride = (size_t)m->cfg.max_pos * m->kv_dim; }
+    } restore{ m };
+    for (size_t t0 = 0; t0 < (size_t)n_tok;) {
+        size_t M = std::min(kPrefillChunk, (size_t)n_tok - t0);
+        const size_t left = (size_t)n_tok - t0 - M;
+        if (left > 0 && left < (size_t)kPrefillMinRows) M -= (size_t)kPrefillMinRows;      // no pass of one or two tokens: the last two share
+        RT_TRY_HIP(ctx, hipMemcpyAsync(m->pf_tok, tokens + t0, M * sizeof(int), hipMemcpyHostToDevice, ctx->stream));
+        rc = prefill_chainable(m, M) ? enqueue_prefill_chain(ctx, m, M, pos0 + (int)t0) : enqueue_prefill_batch(ctx, m, M, pos0 + (int)t0);
+        if (rc) return rc;
+        RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));       // `tokens` is the caller's buffer; pf_tok is reused by the next pass
+        t0 += M;
+    }
+    // logits of the last token into this sequence's row, and its greedy pick
+    float *row = b->logits + (size_t)seq * (size_t)m->cfg.vocab;
+    rt::GemvArgs a;
+    memset(&a, 0, sizeof a);
+    a.n = 1;
+    a.p[0] = make_prob(m->output, m->x, rt::kStageRms, row, nullptr);
+    a.p[0].gamma = m->out_norm; a.p[0].eps = m->cfg.rms_eps;
+    RT_TRY_HIP(ctx, rt::launch_qgemv(ctx->stream, a, 1));
+    RT_TRY_HIP(ctx, rt::launch_argmax(ctx->stream, row, (size_t)m->cfg.vocab, b->pick + seq));
+    RT_TRY_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    b->fed[(size_t)seq] = pos0 + n_tok;
     return RT_HIP_OK;
 }
 

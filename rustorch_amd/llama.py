@@ -102,6 +102,11 @@ class HipLlamaBatch:
                                                        out.ctypes.data_as(_lib.c_int_p) if want_tokens else None), self.ex.ctx)
         return out if want_tokens else None
 
+    def prefill(self, seq: int, tokens, pos0: int = 0) -> None:
+        """Three or more tokens of one sequence through the model's batched prefill passes, into that sequence's cache."""
+        t = np.ascontiguousarray(np.asarray(list(tokens), dtype=np.int32))
+        _lib.check(self.ex.lib.rt_hip_llama_batch_prefill(self.ex.ctx, self.h, seq, t.ctypes.data_as(_lib.c_int_p), t.size, pos0), self.ex.ctx)
+
     def logits(self) -> np.ndarray:
         out = np.empty((self.n_seq, self.model.cfg.vocab), dtype=np.float32)
         _lib.check(self.ex.lib.rt_hip_llama_batch_logits(self.ex.ctx, self.h, C.c_void_p(out.ctypes.data)), self.ex.ctx)
@@ -121,6 +126,10 @@ class HipLlamaBatch:
         done = [False] * self.n_seq
         cur = [p[0] for p in prompts]
         pos = [0] * self.n_seq
+        for i, p in enumerate(prompts):                      # all but the last prompt token in one prefill call where that is 3 tokens or more
+            if 4 <= len(p) <= self.max_pos:
+                self.prefill(i, p[:-1], 0)
+                pos[i], cur[i] = len(p) - 1, p[-1]
         while True:
             for i in range(self.n_seq):
                 done[i] = done[i] or pos[i] >= self.max_pos

@@ -123,6 +123,45 @@ def test_sequences_at_different_positions_and_refilled_slots(ex, orc):
     gm.close()
 
 
+def test_prompt_of_one_sequence_through_the_prefill_passes(ex, orc):
+    """A sequence's prompt in one prefill call (the model's batched passes, writing that sequence's cache) while another
+    sequence is in mid-run: the prompt's last logits and the steps that follow agree with the same tokens fed step by step and
+    with the oracle, and the other sequence is undisturbed."""
+    from rustorch_amd import llama, InvalidParameters, ShapeMismatch
+    gm, om, wn = build_pair(ex, orc, 69, **CFG)
+    s0, s1 = sequences(69, 2, 30, CFG["vocab"])
+    want0, want1 = om.forward(s0, 0), om.forward(s1, 0)
+    tol = logit_tol(wn, CFG["hidden"])
+    b, ref = llama.HipLlamaBatch(gm, 2, 32), llama.HipLlamaBatch(gm, 2, 32)
+    for p in range(4):                                           # sequence 0 runs four steps on its own first
+        b.step([int(s0[p]), -1], [p, 0]); ref.step([int(s0[p]), -1], [p, 0])
+    b.prefill(1, s1[:20], 0)                                     # 20 tokens: the dense-contraction pass
+    for p in range(20):
+        ref.step([-1, int(s1[p])], [0, p])
+    r_pf = float((np.abs(b.logits()[1] - want1[19]) / tol).max())
+    d_pf = float((np.abs(b.logits()[1] - ref.logits()[1]) / tol).max())
+    ratios, between = [], []
+    for k in range(6):                                           # both sequences go on together
+        toks, pos = [int(s0[4 + k]), int(s1[20 + k])], [4 + k, 20 + k]
+        b.step(toks, pos); ref.step(toks, pos)
+        got, other = b.logits(), ref.logits()
+        assert np.array_equal(got[0], other[0])                  # sequence 0 never met the prefill: the same bits as without it
+        ratios.append(float((np.abs(got[1] - want1[20 + k]) / tol).max()))
+        between.append(float((np.abs(got[1] - other[1]) / tol).max()))
+        ratios.append(float((np.abs(got[0] - want0[4 + k]) / tol).max()))
+    print("prefill of 20 tokens into sequence 1: %.3f of the tolerance against the oracle, %.3f against step by step; the steps after: "
+          "median %.3f max %.2f against the oracle, max %.3f against step by step" % (r_pf, d_pf, np.median(ratios), max(ratios), max(between)), flush=True)
+    assert np.median(ratios + [r_pf]) <= 0.1 and d_pf <= 0.5 and np.median(between) <= 0.1
+    with pytest.raises(ShapeMismatch):
+        b.prefill(0, s0[:2], 10)                                 # fewer than three tokens go through step
+    with pytest.raises(InvalidParameters):
+        b.prefill(0, s0[:5], 3)                                  # sequence 0 has been fed 10 tokens
+    with pytest.raises(ShapeMismatch):
+        b.prefill(0, s0[10:30].tolist() + [1, 2, 3], 10)         # past the end of the cache
+    b.close(); ref.close()
+    gm.close()
+
+
 def test_generate_for_several_prompts(ex, orc):
     """Greedy generation for three prompts of different lengths: what a manual loop over batch steps yields, end-of-sequence and
     the token budget honoured per sequence."""
@@ -132,10 +171,14 @@ def test_generate_for_several_prompts(ex, orc):
     b = llama.HipLlamaBatch(gm, 3, 24)
     out = b.generate(prompts, 6)
     assert [len(o) for o in out] == [6, 6, 6]
-    # the same by hand, one sequence per batch slot with the others idle
+    # the same by hand, one sequence per batch slot with the others idle (prompts of four tokens or more: all but the last
+    # token in one prefill call, as generate does)
     for i, prompt in enumerate(prompts):
         b.reset()
         toks, pos, pick = list(prompt), 0, None
+        if len(toks) >= 4:
+            b.prefill(i, toks[:-1], 0)
+            pos = len(toks) - 1
         gen = []
         while len(gen) < 6:
             t = toks[pos] if pos < len(toks) else gen[-1]
