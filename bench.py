@@ -219,14 +219,14 @@ def bench_layer_batch8(ex, n_layers=4, reps=100):
 
 def bench_decode_batch(gm, n_seq, n_prompt, n_gen, vocab):
     """Config C3's batch of eight as a loop: n_seq sequences decoded side by side against the model's weights (every matrix
-    streamed once per step for all of them), prompts of n_prompt tokens fed step by step, then n_gen greedy steps timed.
+    streamed once per step for all of them), prompts of n_prompt tokens through the prefill passes, then n_gen greedy steps timed.
     tokens/s counts the tokens of all sequences."""
     from rustorch_amd import llama, synth
     b = llama.HipLlamaBatch(gm, n_seq, n_prompt + n_gen)
     prompts = [synth.tokens(SEED, 9500 + i, n_prompt, vocab) for i in range(n_seq)]
-    picks = None
-    for p in range(n_prompt):
-        picks = b.step([int(pr[p]) for pr in prompts], [p] * n_seq)
+    for i, pr in enumerate(prompts):                    # all but the last prompt token through the prefill passes
+        b.prefill(i, pr[:-1], 0)
+    picks = b.step([int(pr[-1]) for pr in prompts], [n_prompt - 1] * n_seq)
     t0 = time.perf_counter()
     for p in range(n_prompt, n_prompt + n_gen):
         picks = b.step([int(t) for t in picks], [p] * n_seq)
