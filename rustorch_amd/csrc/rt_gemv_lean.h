@@ -24,6 +24,14 @@
 
 namespace rt {
 
+// After x has been staged, once per problem: wait for every outstanding load.  The two weight requests that are in flight
+// went out before the staging and its barrier, so they have landed or nearly.  What the wait buys is in the steady-state loop: the
+// compiler's wait-count bookkeeping follows every path through the staging code at once, ends up holding some staging
+// register for possibly still in flight, and -- where the loop reuses that register -- waits for *all* loads there, the
+// prefetch just issued included (seen in the generated code of the Q6_K loops: vmcnt(0) in the first of the two steps and no wait
+// in the second, against vmcnt(7), (6), (5) per step with this wait in place).
+__device__ __forceinline__ void lean_settle_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }      // vmcnt(0), the other counters untouched
+
 // The first product of an integer sum and the following ones.  (Through the compiler's own dot4, not inline assembly: the
 // result of a dot instruction may only be read by another kind of vector instruction a few issue slots later, and the
 // compiler keeps that distance only for instructions it can see.)
@@ -324,6 +332,7 @@ __device__ __forceinline__ void lean_problem_t(const GemvProb &P, int wg, int n_
 #ifndef RT_LEAN_NO_STAGE
     S.finish<TYPE>(P, m, lds, red);
 #endif
+    lean_settle_loads();
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
@@ -459,6 +468,7 @@ __device__ __forceinline__ void lean_problem_split(const GemvProb &P, int wg, in
 #ifndef RT_LEAN_NO_STAGE
     S.finish<TYPE>(P, m, lds, red);
 #endif
+    lean_settle_loads();
 
     auto consume = [&](const WRegs<TYPE> &wr, Pos s) {
         const int u = lane + 64 * s.p;
