@@ -24,7 +24,7 @@ def test_header_symbols_are_exported_and_bound(lib):
 
 
 def test_rust_binding_in_the_integration_notes_is_generated_from_the_header():
-    """INTEGRATION.md holds the Rust `extern "C"` module a maintainer would add; it is generated from the header, declares
+    """The integration notes hold the Rust `extern "C"` module a maintainer would add; it is generated from the header, declares
     every exported function with the header's argument count, pointer-ness and return kind, and agrees with the ctypes table."""
     import ctypes as C
     from rustorch_amd import _lib, ffi_gen
