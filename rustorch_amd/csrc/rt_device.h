@@ -251,4 +251,30 @@ __device__ __forceinline__ Q4Pack quantize4(float4 v) {
     return r;
 }
 
+// The operand form of the small-batch matrix-core GEMV (rt_gemv_mb.hip): up to 8 activation rows ("tokens") of K elements
+// in one workspace -- 16 K bytes of int8 planes, then xs[K / 32][8] (block scales) and xb[K / 32][8] (scale x block sum).
+// Per 32-element block 512 bytes in the order the GEMV's lanes load them: [k chunk c = 0..3][matrix row i = 8 * plane +
+// token][8 bytes].  Stores the four elements i4 * 4 .. + 3 of row `token`; the 8 lanes that hold a block must be
+// consecutive lanes of one wave, all active.  Rows that carry no token must be stored as zeros (the GEMV multiplies all 8).
+struct Xq8Work {
+    uint8_t *xq;
+    float *xs, *xb;
+};
+__device__ __host__ __forceinline__ Xq8Work xq8_work(void *work, size_t K) {
+    uint8_t *xq = static_cast<uint8_t *>(work);
+    float *xs = reinterpret_cast<float *>(xq + 16 * K);
+    return Xq8Work{ xq, xs, xs + K / 4 };
+}
+__device__ __forceinline__ void xq8_store4(float4 v, int i4, int token, const Xq8Work &w) {
+    const Q4Pack p = quantize4(v);
+    const int blk = i4 >> 3, l8 = i4 & 7;
+    uint8_t *base = w.xq + (size_t)blk * 512 + (l8 >> 1) * 128 + token * 8 + (l8 & 1) * 4;
+    *reinterpret_cast<uint32_t *>(base) = p.hi;
+    *reinterpret_cast<uint32_t *>(base + 64) = p.lo;
+    if (l8 == 0) {
+        w.xs[blk * 8 + token] = p.s;
+        w.xb[blk * 8 + token] = p.s * (float)p.sum32;
+    }
+}
+
 }  // namespace rt

@@ -42,15 +42,7 @@ __global__ __launch_bounds__(256) void xq8_prep_kernel(const float *__restrict__
     if (4 * i4 >= K) return;                               // K % 32 == 0: the lanes of a block leave together
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (t < batch) v = *reinterpret_cast<const float4 *>(X + (size_t)t * K + 4 * (size_t)i4);
-    const Q4Pack p = quantize4(v);
-    const int blk = i4 >> 3, l8 = i4 & 7;
-    uint8_t *base = xq + (size_t)blk * 512 + (l8 >> 1) * 128 + t * 8 + (l8 & 1) * 4;
-    *reinterpret_cast<uint32_t *>(base) = p.hi;
-    *reinterpret_cast<uint32_t *>(base + 64) = p.lo;
-    if (l8 == 0) {
-        xs[blk * 8 + t] = p.s;
-        xb[blk * 8 + t] = p.s * (float)p.sum32;
-    }
+    xq8_store4(v, i4, t, Xq8Work{ xq, xs, xb });
 }
 
 constexpr int kMbMaxProbs = 4;             // weight matrices of one format that meet the same prepared rows in one launch

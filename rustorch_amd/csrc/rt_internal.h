@@ -130,7 +130,11 @@ hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const f
 hipError_t launch_rope_kv_rows(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache, const int *pos_rows_dev,
                                size_t seq_stride, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev);
 hipError_t launch_attn_rows(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc, const int *pos_rows_dev, size_t seq_stride,
-                            int max_pos, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out);
+                            int max_pos, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out, void *xq8_work_buf);
+// producers that write the operand form of the small-batch matrix-core GEMV (launch_qgemv_mb_group's `work`) directly:
+// rows <= 8, n a multiple of 256; launch_attn_rows does the same with out == nullptr
+hipError_t launch_rmsnorm_xq8(hipStream_t s, const float *x, const float *gamma, size_t rows, size_t n, float eps, void *work);
+hipError_t launch_swiglu_xq8(hipStream_t s, const float *gate, const float *up, size_t rows, size_t n, void *work);
 hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,
                              const int *pos_dev, int n_pos, size_t n_queries, int n_heads, int n_kv_heads, int head_dim,
                              const float *inv_freq_dev, float *out, uint8_t *xq, bool fused);
@@ -141,6 +145,7 @@ hipError_t launch_embed_rows(hipStream_t s, int type, const uint8_t *w, size_t r
                              const int *tokens_dev, size_t n_tok, int vocab, float *out);
 hipError_t launch_add(hipStream_t s, float *x, const float *y, size_t n);
 hipError_t launch_stream_read(hipStream_t s, const void *p, size_t nbytes, unsigned *sink);
+hipError_t launch_argmax_rows(hipStream_t s, const float *v, size_t rows, size_t n, int *out_dev);     // out_dev[row] = pick of v[row][0..n)
 hipError_t launch_argmax(hipStream_t s, const float *v, size_t n, int *out_dev);
 // the greedy pick and the end of the decode step (as launch_step_advance) in one launch
 hipError_t launch_argmax_advance(hipStream_t s, const float *v, size_t n, int *pick_dev, int *pos_dev, int *token_dev, const int *forced_dev,

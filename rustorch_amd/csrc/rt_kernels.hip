@@ -126,6 +126,50 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const float *gate, const fl
     }
 }
 
+// ---- the same two operations writing the operand form of the small-batch matrix-core GEMV (xq8_store4) instead of f32:
+// the step of several sequences runs them in front of q / k / v, gate / up and the down-projection, which saves those
+// contractions their quantizing launch.  Arithmetic as in rmsnorm_kernel / swiglu_kernel, then the quantization step the
+// stand-alone pre-pass applies to their f32 result.  n % 32 == 0.  All 8 rows of the operand are written: zeros from row
+// `batch` on.
+__global__ __launch_bounds__(1024) void rmsnorm_xq8_kernel(const float *x, const float *gamma, size_t n, float eps, int batch, Xq8Work w) {
+    __shared__ float red[16];
+    const int m = blockIdx.x;
+    const size_t n4 = n / 4;
+    if (m >= batch) {
+        for (size_t i = threadIdx.x; i < n4; i += blockDim.x) xq8_store4(make_float4(0.f, 0.f, 0.f, 0.f), (int)i, m, w);
+        return;
+    }
+    const float4 *x4 = reinterpret_cast<const float4 *>(x + (size_t)m * n);
+    const float4 *g4 = reinterpret_cast<const float4 *>(gamma);
+    float ss = 0.f;
+    for (size_t i = threadIdx.x; i < n4; i += blockDim.x) {
+        float4 v = x4[i];
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = block_sum(ss, red);
+    float rms = sqrtf(ss / (float)n + eps);
+    for (size_t i = threadIdx.x; i < n4; i += blockDim.x) {
+        float4 v = x4[i], g = g4[i];
+        xq8_store4(make_float4(g.x * (v.x / rms), g.y * (v.y / rms), g.z * (v.z / rms), g.w * (v.w / rms)), (int)i, m, w);
+    }
+}
+
+// grid (n / 4 / 256 rounded up, 8): blockIdx.y = row
+__global__ __launch_bounds__(256) void swiglu_xq8_kernel(const float *gate, const float *up, size_t n, int batch, Xq8Work w) {
+    const int t = blockIdx.y;
+    const size_t i4 = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i4 * 4 >= n) return;          // whole 8-lane groups leave together because n % 32 == 0
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (t < batch) {
+        float4 g = reinterpret_cast<const float4 *>(gate + (size_t)t * n)[i4], u = reinterpret_cast<const float4 *>(up + (size_t)t * n)[i4];
+        o.x = u.x * (g.x * (1.0f / (1.0f + expf(-g.x))));
+        o.y = u.y * (g.y * (1.0f / (1.0f + expf(-g.y))));
+        o.z = u.z * (g.z * (1.0f / (1.0f + expf(-g.z))));
+        o.w = u.w * (g.w * (1.0f / (1.0f + expf(-g.w))));
+    }
+    xq8_store4(o, (int)i4, t, w);
+}
+
 // --------------------------------------------------------------------- RoPE
 // Interleaved pairs: (x[2i], x[2i+1]) turned by pos * inv_freq[i].  One thread per pair.
 __global__ void rope_kernel(float *x, int n_heads, int head_dim, const int *pos_dev, int pos, const float *inv_freq,
@@ -430,9 +474,11 @@ __global__ void rope_kv_rows_kernel(float *q, const float *k, const float *v, ui
 // m's cache (the row of the step itself was stored by rope_kv_rows_kernel before).  Same arithmetic as the decode step's
 // kernel in its plain form: a thread per position for the scores (the whole dot in the thread), max-subtracted softmax over
 // the workgroup, values as 16-byte column chunks x position groups folded through LDS.  Dynamic LDS: max_pos floats.
+// With xw.xq set the result goes out in the operand form of the small-batch matrix-core GEMV (the o-projection's input; out
+// is not written) and the grid has 8 rows: the rows from n_rows on are stored as zeros.
 template <int HD>
 __global__ __launch_bounds__(256) void attn_rows_kernel(const float *q, const uint16_t *kc, const uint16_t *vc, const int *pos_rows,
-                                                        size_t seq_stride, int n_heads, int n_kv_heads, float *out) {
+                                                        size_t seq_stride, int n_heads, int n_kv_heads, float *out, Xq8Work xw, int n_rows) {
     RT_DYN_LDS(float, sc);
     __shared__ float red[4];
     __shared__ __align__(16) float qs[HD];
@@ -441,6 +487,10 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const float *q, const ui
     constexpr int NG = 256 / CH;        // position groups in the value phase
     const int h = blockIdx.x, tid = threadIdx.x;
     const size_t m = blockIdx.y, row = (size_t)n_heads * HD, rowkv = (size_t)n_kv_heads * HD;
+    if ((int)m >= n_rows) {             // only in the operand form: a row without a sequence
+        if (tid < HD / 4) xq8_store4(make_float4(0.f, 0.f, 0.f, 0.f), h * (HD / 4) + tid, (int)m, xw);
+        return;
+    }
     const int kvh = h / (n_heads / n_kv_heads);
     const int n_pos = pos_rows[m] + 1;
     kc += m * seq_stride + (size_t)kvh * HD;
@@ -490,7 +540,12 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const float *q, const ui
     if (tid < HD) {
         float o = 0.f;
         for (int gg = 0; gg < NG; gg++) o += part[gg * HD + tid];
-        out[m * row + (size_t)h * HD + tid] = o;
+        if (xw.xq) qs[tid] = o;         // the query row has done its work
+        else out[m * row + (size_t)h * HD + tid] = o;
+    }
+    if (xw.xq) {
+        __syncthreads();
+        if (tid < HD / 4) xq8_store4(reinterpret_cast<const float4 *>(qs)[tid], h * (HD / 4) + tid, (int)m, xw);
     }
 }
 
@@ -677,9 +732,8 @@ struct StepAdvance {
     const int *forced_dev;
     int enabled;
 };
-__global__ __launch_bounds__(1024) void argmax_kernel(const float *v, size_t n, int *out, StepAdvance adv) {
-    __shared__ float bv[1024];
-    __shared__ int bi[1024];
+// The pick of one workgroup of 1024 threads over v[0..n); valid in thread 0.
+__device__ __forceinline__ int block_argmax(const float *v, size_t n, float *bv, int *bi) {
     float best = -INFINITY;
     int idx = 0x7fffffff;
     for (size_t i0 = threadIdx.x; i0 < n; i0 += 8 * (size_t)blockDim.x) {
@@ -707,8 +761,22 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *v, size_t n, 
         }
         __syncthreads();
     }
+    return bi[0] == 0x7fffffff ? 0 : bi[0];
+}
+
+// One workgroup per row of v[rows][n]: out[row] = its pick (the step of several sequences).
+__global__ __launch_bounds__(1024) void argmax_rows_kernel(const float *v, size_t n, int *out) {
+    __shared__ float bv[1024];
+    __shared__ int bi[1024];
+    const int pick = block_argmax(v + (size_t)blockIdx.x * n, n, bv, bi);
+    if (threadIdx.x == 0) out[blockIdx.x] = pick;
+}
+
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *v, size_t n, int *out, StepAdvance adv) {
+    __shared__ float bv[1024];
+    __shared__ int bi[1024];
+    const int pick = block_argmax(v, n, bv, bi);
     if (threadIdx.x == 0) {
-        const int pick = bi[0] == 0x7fffffff ? 0 : bi[0];
         *out = pick;
         if (adv.enabled) {
             const int step = *adv.step_dev;
@@ -1000,14 +1068,35 @@ hipError_t launch_rope_kv_rows(hipStream_t s, float *q, const float *k, const fl
     return hipGetLastError();
 }
 
+// out: [n_rows][n_heads * head_dim] f32 -- or, with out == nullptr and xq8_work set, the operand form of the small-batch
+// matrix-core GEMV in that workspace (n_rows <= 8, n_heads * head_dim a multiple of 256)
 hipError_t launch_attn_rows(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc, const int *pos_rows_dev, size_t seq_stride,
-                            int max_pos, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out) {
+                            int max_pos, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out, void *xq8_work_buf) {
     if (n_kv_heads <= 0 || n_heads % n_kv_heads != 0 || n_rows == 0 || n_rows > 65535 || max_pos <= 0 || max_pos > 8192) return hipErrorInvalidValue;
+    if ((out == nullptr) == (xq8_work_buf == nullptr)) return hipErrorInvalidValue;
+    const size_t H = (size_t)n_heads * (size_t)head_dim;
+    if (xq8_work_buf && (n_rows > 8 || H % 256 != 0 || ((uintptr_t)xq8_work_buf & 255))) return hipErrorInvalidValue;
     const size_t lds = (size_t)max_pos * sizeof(float);      // at most 32 KB beside the 9 KB of static arrays: inside the default 64 KB
-    dim3 grid((unsigned)n_heads, (unsigned)n_rows);
-    if (head_dim == 128) attn_rows_kernel<128><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out);
-    else if (head_dim == 64) attn_rows_kernel<64><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out);
+    const Xq8Work xw = xq8_work_buf ? xq8_work(xq8_work_buf, H) : Xq8Work{ nullptr, nullptr, nullptr };
+    dim3 grid((unsigned)n_heads, xq8_work_buf ? 8u : (unsigned)n_rows);
+    if (head_dim == 128) attn_rows_kernel<128><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out, xw, (int)n_rows);
+    else if (head_dim == 64) attn_rows_kernel<64><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out, xw, (int)n_rows);
     else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+// RMSNorm / SwiGLU of `rows` <= 8 rows of n elements (n % 256 == 0) into the operand form of the small-batch matrix-core GEMV
+hipError_t launch_rmsnorm_xq8(hipStream_t s, const float *x, const float *gamma, size_t rows, size_t n, float eps, void *work) {
+    if (!x || !gamma || !work || rows < 1 || rows > 8 || n < 256 || n % 256 != 0) return hipErrorInvalidValue;
+    if (((uintptr_t)x & 15) || ((uintptr_t)gamma & 15) || ((uintptr_t)work & 255)) return hipErrorInvalidValue;
+    rmsnorm_xq8_kernel<<<8, 1024, 0, s>>>(x, gamma, n, eps, (int)rows, xq8_work(work, n));
+    return hipGetLastError();
+}
+
+hipError_t launch_swiglu_xq8(hipStream_t s, const float *gate, const float *up, size_t rows, size_t n, void *work) {
+    if (!gate || !up || !work || rows < 1 || rows > 8 || n < 256 || n % 256 != 0) return hipErrorInvalidValue;
+    if (((uintptr_t)gate & 15) || ((uintptr_t)up & 15) || ((uintptr_t)work & 255)) return hipErrorInvalidValue;
+    swiglu_xq8_kernel<<<dim3((unsigned)((n / 4 + 255) / 256), 8), 256, 0, s>>>(gate, up, n, (int)rows, xq8_work(work, n));
     return hipGetLastError();
 }
 
@@ -1078,6 +1167,12 @@ hipError_t launch_stream_read(hipStream_t s, const void *p, size_t nbytes, unsig
     const size_t n_chunks = nbytes / 2048;       // whole pieces only: nothing past p + nbytes is touched
     if (n_chunks == 0) return hipSuccess;
     stream_read_kernel<<<512, 512, 0, s>>>(reinterpret_cast<const uint4 *>(p), n_chunks, sink);
+    return hipGetLastError();
+}
+
+hipError_t launch_argmax_rows(hipStream_t s, const float *v, size_t rows, size_t n, int *out_dev) {
+    if (rows == 0 || rows > 65535) return hipErrorInvalidValue;
+    argmax_rows_kernel<<<(unsigned)rows, 1024, 0, s>>>(v, n, out_dev);
     return hipGetLastError();
 }
 

@@ -442,16 +442,51 @@ int enqueue_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b) {
     float *x = b->x, *x2 = b->x2;
     PrefillGemm gemm{ ctx, m };
     RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, b->tok, M, c.vocab, x));
+    // Every matrix of a layer on the small-batch matrix-core GEMV (3..8 sequences, Q4_K / Q6_K): the kernel in front of
+    // each contraction writes the GEMV's operand form itself -- RMSNorm for q / k / v and for gate / up, the attention for the
+    // o-projection, SwiGLU for the down-projection -- so no contraction needs a quantizing launch of its own (four launches
+    // fewer per layer), and no f32 copy of those activations is written or read.
+    auto mb = [&](const rt_hip_llama::T &t, size_t K) { return t.n_cols == K && rt::qgemv_mb_serves(t.type, t.n_rows, K, (int)M); };
+    auto mb_group = [&](std::initializer_list<const rt_hip_llama::T *> ts, std::initializer_list<float *> ys, const float *res, size_t K) {
+        for (int type : { (int)RT_GGML_Q4_K, (int)RT_GGML_Q6_K }) {
+            rt::MbProb probs[4];
+            int k = 0;
+            auto y = ys.begin();
+            for (const rt_hip_llama::T *t : ts) {
+                if (t->type == type) probs[k++] = rt::MbProb{ t->dev, t->row_bytes, t->n_rows, *y, res };
+                ++y;
+            }
+            if (k) RT_TRY_HIP(ctx, rt::launch_qgemv_mb_group(s, type, probs, k, K, (int)M, ctx->scratch));
+        }
+        return (int)RT_HIP_OK;
+    };
     for (int l = 0; l < c.n_layers; l++) {
         uint16_t *kc = b->kcache + (size_t)l * M * seq_stride;
         uint16_t *vc = b->vcache + (size_t)l * M * seq_stride;
+        const bool fused = M >= (size_t)rt::kGemvMbMinBatch && M <= 8 && ((uintptr_t)ctx->scratch & 255) == 0 &&
+                           ctx->scratch_bytes >= rt::qgemv_mb_scratch_bytes(std::max(H, F)) && mb(m->wq[l], H) && mb(m->wk[l], H) &&
+                           mb(m->wv[l], H) && mb(m->wo[l], H) && mb(m->wgate[l], H) && mb(m->wup[l], H) && mb(m->wdown[l], F);
+        if (fused) {
+            RT_TRY_HIP(ctx, rt::launch_rmsnorm_xq8(s, x, m->attn_norm[l], M, H, c.rms_eps, ctx->scratch));
+            if ((rc = mb_group({ &m->wq[l], &m->wk[l], &m->wv[l] }, { b->q, b->k, b->v }, nullptr, H))) return rc;
+            RT_TRY_HIP(ctx, rt::launch_rope_kv_rows(s, b->q, b->k, b->v, kc, vc, b->pos, seq_stride, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
+            RT_TRY_HIP(ctx, rt::launch_attn_rows(s, b->q, kc, vc, b->pos, seq_stride, b->max_pos, M, c.n_heads, m->n_kv, m->head_dim, nullptr, ctx->scratch));
+            if ((rc = mb_group({ &m->wo[l] }, { x2 }, x, H))) return rc;
+            std::swap(x, x2);
+            RT_TRY_HIP(ctx, rt::launch_rmsnorm_xq8(s, x, m->ffn_norm[l], M, H, c.rms_eps, ctx->scratch));
+            if ((rc = mb_group({ &m->wgate[l], &m->wup[l] }, { b->g, b->u }, nullptr, H))) return rc;
+            RT_TRY_HIP(ctx, rt::launch_swiglu_xq8(s, b->g, b->u, M, F, ctx->scratch));
+            if ((rc = mb_group({ &m->wdown[l] }, { x2 }, x, F))) return rc;
+            std::swap(x, x2);
+            continue;
+        }
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->attn_norm[l], b->n, nullptr, M, H, c.rms_eps));
         gemm.prepared = nullptr;
         rt_hip_llama::T *qkv[3] = { &m->wq[l], &m->wk[l], &m->wv[l] };
         float *qkv_y[3] = { b->q, b->k, b->v };
         if ((rc = gemm.shared(qkv, qkv_y, 3, b->n, M))) return rc;
         RT_TRY_HIP(ctx, rt::launch_rope_kv_rows(s, b->q, b->k, b->v, kc, vc, b->pos, seq_stride, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
-        RT_TRY_HIP(ctx, rt::launch_attn_rows(s, b->q, kc, vc, b->pos, seq_stride, b->max_pos, M, c.n_heads, m->n_kv, m->head_dim, b->a));
+        RT_TRY_HIP(ctx, rt::launch_attn_rows(s, b->q, kc, vc, b->pos, seq_stride, b->max_pos, M, c.n_heads, m->n_kv, m->head_dim, b->a, nullptr));
         if ((rc = gemm(m->wo[l], b->a, M, x2, x))) return rc;
         std::swap(x, x2);
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->ffn_norm[l], b->n, nullptr, M, H, c.rms_eps));
@@ -464,11 +499,16 @@ int enqueue_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b) {
         if ((rc = gemm(m->wdown[l], b->g, M, x2, x))) return rc;
         std::swap(x, x2);
     }
-    RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->out_norm, b->n, nullptr, M, H, c.rms_eps));
-    gemm.prepared = nullptr;
-    if ((rc = gemm(m->output, b->n, M, b->logits, nullptr))) return rc;
-    for (size_t i = 0; i < M; i++)
-        RT_TRY_HIP(ctx, rt::launch_argmax(s, b->logits + i * (size_t)c.vocab, (size_t)c.vocab, b->pick + i));
+    if (M >= (size_t)rt::kGemvMbMinBatch && M <= 8 && ((uintptr_t)ctx->scratch & 255) == 0 && ctx->scratch_bytes >= rt::qgemv_mb_scratch_bytes(H) &&
+        mb(m->output, H)) {
+        RT_TRY_HIP(ctx, rt::launch_rmsnorm_xq8(s, x, m->out_norm, M, H, c.rms_eps, ctx->scratch));
+        if ((rc = mb_group({ &m->output }, { b->logits }, nullptr, H))) return rc;
+    } else {
+        RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->out_norm, b->n, nullptr, M, H, c.rms_eps));
+        gemm.prepared = nullptr;
+        if ((rc = gemm(m->output, b->n, M, b->logits, nullptr))) return rc;
+    }
+    RT_TRY_HIP(ctx, rt::launch_argmax_rows(s, b->logits, M, (size_t)c.vocab, b->pick));
     return RT_HIP_OK;
 }
 
