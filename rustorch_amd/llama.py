@@ -112,11 +112,17 @@ class HipLlamaBatch:
         _lib.check(self.ex.lib.rt_hip_llama_batch_logits(self.ex.ctx, self.h, C.c_void_p(out.ctypes.data)), self.ex.ctx)
         return out
 
-    def generate(self, prompts, max_new_tokens: int, eos_token: int | None = None):
-        """The generate loop (inference.rs:135-192) for n_seq prompts at once, greedy: feeds the prompts token by token
-        (a shorter prompt starts generating while longer ones are still being fed), stops a sequence at eos_token, after
-        max_new_tokens or at the end of its cache, and leaves finished sequences idle while the others go on.  Returns the
-        generated ids per sequence."""
+    def generate(self, prompts, max_new_tokens: int, eos_token: int | None = None, config=None, rng=None):
+        """The generate loop (inference.rs:135-192) for n_seq prompts at once: feeds the prompts (a shorter prompt starts
+        generating while longer ones are still being fed), stops a sequence at eos_token, after max_new_tokens or at the end
+        of its cache, and leaves finished sequences idle while the others go on.  Greedy by default (the pick is made on the
+        device); with a sampling configuration (sampling.rs:8-80) that is not greedy, every step's logits are read back and
+        each live sequence draws on the host from its own row, with its own history for the repetition penalty.  Returns
+        the generated ids per sequence."""
+        from .sampling import SamplingConfig, sample_token
+        config = config or SamplingConfig.greedy()
+        config.validate()
+        on_host = not (config.is_greedy and config.repetition_penalty == 1.0)
         prompts = [list(map(int, p)) for p in prompts]
         if len(prompts) != self.n_seq or any(len(p) == 0 for p in prompts):
             from .errors import ShapeMismatch
@@ -135,7 +141,8 @@ class HipLlamaBatch:
                 done[i] = done[i] or pos[i] >= self.max_pos
             if all(done):
                 break
-            picks = self.step([-1 if done[i] else cur[i] for i in range(self.n_seq)], pos)
+            picks = self.step([-1 if done[i] else cur[i] for i in range(self.n_seq)], pos, want_tokens=not on_host)
+            rows = self.logits() if on_host else None
             for i in range(self.n_seq):
                 if done[i]:
                     continue
@@ -143,7 +150,7 @@ class HipLlamaBatch:
                 if pos[i] < len(prompts[i]):
                     cur[i] = prompts[i][pos[i]]                      # still feeding the prompt
                     continue
-                tok = int(picks[i])
+                tok = int(sample_token(rows[i], config, prompts[i] + out[i], rng)) if on_host else int(picks[i])
                 out[i].append(tok)
                 cur[i] = tok
                 if (eos_token is not None and tok == eos_token) or len(out[i]) >= max_new_tokens:

@@ -193,6 +193,14 @@ def test_generate_for_several_prompts(ex, orc):
     assert stopped[0] == out[0][:out[0].index(eos) + 1]
     short = llama.HipLlamaBatch(gm, 3, 9)                       # the longest prompt leaves room for two new tokens
     assert [len(o) for o in short.generate(prompts, 6)] == [5, 6, 2]
+    # sampling on the host from each sequence's own row of logits: a greedy configuration that has to take that way (a
+    # repetition penalty, here one that changes nothing) repeats the device's picks; a seeded draw repeats itself
+    from rustorch_amd.sampling import SamplingConfig
+    assert b.generate(prompts, 6, config=SamplingConfig(temperature=0.0, top_k=1, repetition_penalty=1.0 + 1e-12)) == out
+    warm = SamplingConfig(temperature=0.9, top_k=20, top_p=0.95, repetition_penalty=1.1)
+    drawn = b.generate(prompts, 6, config=warm, rng=np.random.default_rng(5))
+    assert drawn == b.generate(prompts, 6, config=warm, rng=np.random.default_rng(5))
+    assert [len(o) for o in drawn] == [6, 6, 6] and all(0 <= t < CFG["vocab"] for o in drawn for t in o)
     b.close(); short.close()
     gm.close()
 
