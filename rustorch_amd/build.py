@@ -50,7 +50,8 @@ def find_hipcc() -> str:
 # one of them a scratch frame (register spills or an array it could not keep in registers).  One spilling variant
 # inside such a kernel slows every launch of it, also the ones that never reach the variant.
 NO_SCRATCH = {"rt_gemv.hip": ("qgemv_kernel", "qgemv_lean_kernel"), "rt_gemm.hip": ("qgemm_kernel",), "rt_attn_prefill.hip": ("attn_causal_kernel",),
-              "rt_hgemm.hip": ("hgemm_kernel",), "rt_gemv_mb.hip": ("qgemv_mb_q4k_kernel", "qgemv_mb_q6k_kernel")}
+              "rt_hgemm.hip": ("hgemm_kernel",), "rt_gemv_mb.hip": ("qgemv_mb_q4k_kernel", "qgemv_mb_q6k_kernel"),
+              "rt_kernels.hip": ("attn_decode_kernel", "attn_split_kernel", "attn_rows_kernel", "matmul_f32_mfma_kernel")}
 RESOURCE_FLAG = "-Rpass-analysis=kernel-resource-usage"
 
 
