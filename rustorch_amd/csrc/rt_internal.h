@@ -129,10 +129,11 @@ hipError_t launch_rope_kv_batch(hipStream_t s, float *q, const float *k, const f
 // elements into kcache / vcache
 hipError_t launch_rope_kv_rows(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kcache, uint16_t *vcache, const int *pos_rows_dev,
                                size_t seq_stride, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, const float *inv_freq_dev);
-hipError_t launch_attn_rows(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc, const int *pos_rows_dev, size_t seq_stride,
-                            int max_pos, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out, void *xq8_work_buf);
+hipError_t launch_attn_rows(hipStream_t s, const float *q, uint16_t *kc, uint16_t *vc, const int *pos_rows_dev, size_t seq_stride, int max_pos,
+                            size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out, void *xq8_work_buf, const float *k_new,
+                            const float *v_new, const float *inv_freq_dev);
 // producers that write the operand form of the small-batch matrix-core GEMV (launch_qgemv_mb_group's `work`) directly:
-// rows <= 8, n a multiple of 256; launch_attn_rows does the same with out == nullptr
+// rows <= 8, n a multiple of 256; launch_attn_rows does the same with out == nullptr (and then rotates and appends itself)
 hipError_t launch_rmsnorm_xq8(hipStream_t s, const float *x, const float *gamma, size_t rows, size_t n, float eps, void *work);
 hipError_t launch_swiglu_xq8(hipStream_t s, const float *gate, const float *up, size_t rows, size_t n, void *work);
 hipError_t launch_attn_batch(hipStream_t s, float *q, const float *k, const float *v, uint16_t *kc, uint16_t *vc,

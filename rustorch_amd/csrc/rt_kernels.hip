@@ -474,38 +474,74 @@ __global__ void rope_kv_rows_kernel(float *q, const float *k, const float *v, ui
 // m's cache (the row of the step itself was stored by rope_kv_rows_kernel before).  Same arithmetic as the decode step's
 // kernel in its plain form: a thread per position for the scores (the whole dot in the thread), max-subtracted softmax over
 // the workgroup, values as 16-byte column chunks x position groups folded through LDS.  Dynamic LDS: max_pos floats.
-// With xw.xq set the result goes out in the operand form of the small-batch matrix-core GEMV (the o-projection's input; out
-// is not written) and the grid has 8 rows: the rows from n_rows on are stored as zeros.
+// With xw.xq set the kernel is the whole attention block of the step of several sequences: q, k_new and v_new are the
+// projections as the contractions left them; the workgroup rotates its query head and the step's key row by the sequence's
+// position (rope_kv_rows_kernel's arithmetic), the first query head of a key / value group stores the rotated key and the
+// value as the cache's row of that position, and every workgroup takes that row from its own LDS copy (rounded to fp16 as the
+// cache holds it) instead of waiting for the store of another workgroup.  The result goes out in the operand form of the
+// small-batch matrix-core GEMV (the o-projection's input; out is not written) and the grid has 8 rows: the rows from
+// n_rows on are stored as zeros.
 template <int HD>
-__global__ __launch_bounds__(256) void attn_rows_kernel(const float *q, const uint16_t *kc, const uint16_t *vc, const int *pos_rows,
-                                                        size_t seq_stride, int n_heads, int n_kv_heads, float *out, Xq8Work xw, int n_rows) {
+__global__ __launch_bounds__(256) void attn_rows_kernel(const float *q, uint16_t *kc, uint16_t *vc, const int *pos_rows, size_t seq_stride,
+                                                        int n_heads, int n_kv_heads, float *out, Xq8Work xw, int n_rows, const float *k_new,
+                                                        const float *v_new, const float *inv_freq) {
     RT_DYN_LDS(float, sc);
     __shared__ float red[4];
     __shared__ __align__(16) float qs[HD];
+    __shared__ __align__(16) float knew[HD], vnew[HD];
     __shared__ __align__(16) float part[2048];
     constexpr int CH = HD / 8;          // 16-byte chunks per cache row of this head
     constexpr int NG = 256 / CH;        // position groups in the value phase
     const int h = blockIdx.x, tid = threadIdx.x;
     const size_t m = blockIdx.y, row = (size_t)n_heads * HD, rowkv = (size_t)n_kv_heads * HD;
+    const bool whole = xw.xq != nullptr;
     if ((int)m >= n_rows) {             // only in the operand form: a row without a sequence
         if (tid < HD / 4) xq8_store4(make_float4(0.f, 0.f, 0.f, 0.f), h * (HD / 4) + tid, (int)m, xw);
         return;
     }
-    const int kvh = h / (n_heads / n_kv_heads);
-    const int n_pos = pos_rows[m] + 1;
+    const int group = n_heads / n_kv_heads, kvh = h / group;
+    const int last = pos_rows[m], n_pos = last + 1;
     kc += m * seq_stride + (size_t)kvh * HD;
     vc += m * seq_stride + (size_t)kvh * HD;
     const float scale = 1.0f / sqrtf((float)HD);
-    if (tid < HD) qs[tid] = q[m * row + (size_t)h * HD + tid];
+    if (whole) {
+        if (tid < HD / 2) {
+            float s, c;
+            sincosf((float)last * inv_freq[tid], &s, &c);
+            const float2 qv = reinterpret_cast<const float2 *>(q + m * row + (size_t)h * HD)[tid];
+            qs[2 * tid] = qv.x * c - qv.y * s;
+            qs[2 * tid + 1] = qv.x * s + qv.y * c;
+            const float2 kv = reinterpret_cast<const float2 *>(k_new + m * rowkv + (size_t)kvh * HD)[tid];
+            const float k0 = kv.x * c - kv.y * s, k1 = kv.x * s + kv.y * c;
+            const float2 vv = reinterpret_cast<const float2 *>(v_new + m * rowkv + (size_t)kvh * HD)[tid];
+            const uint32_t kh = (uint32_t)f2h_rne(k0) | ((uint32_t)f2h_rne(k1) << 16), vh = (uint32_t)f2h_rne(vv.x) | ((uint32_t)f2h_rne(vv.y) << 16);
+            knew[2 * tid] = h2f(kh & 0xFFFF);
+            knew[2 * tid + 1] = h2f(kh >> 16);
+            vnew[2 * tid] = h2f(vh & 0xFFFF);
+            vnew[2 * tid + 1] = h2f(vh >> 16);
+            if (h == kvh * group) {
+                reinterpret_cast<uint32_t *>(kc + (size_t)last * rowkv)[tid] = kh;
+                reinterpret_cast<uint32_t *>(vc + (size_t)last * rowkv)[tid] = vh;
+            }
+        }
+    } else if (tid < HD) {
+        qs[tid] = q[m * row + (size_t)h * HD + tid];
+    }
     __syncthreads();
     float mx = -INFINITY;
     for (int j = tid; j < n_pos; j += 256) {
         const uint4 *kr = reinterpret_cast<const uint4 *>(kc + (size_t)j * rowkv);
+        const bool own = whole && j == last;      // this step's row: from LDS, the cache's copy may not be there yet
         float s = 0.f;
 #pragma unroll
         for (int cc = 0; cc < CH; cc++) {
             float f[8];
-            unpack8(kr[cc], f);
+            if (own) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) f[e] = knew[8 * cc + e];
+            } else {
+                unpack8(kr[cc], f);
+            }
 #pragma unroll
             for (int e = 0; e < 8; e++) s += qs[8 * cc + e] * f[e];
         }
@@ -529,7 +565,12 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const float *q, const ui
     for (int e = 0; e < 8; e++) acc[e] = 0.f;
     for (int j = g; j < n_pos; j += NG) {
         float f[8];
-        unpack8(reinterpret_cast<const uint4 *>(vc + (size_t)j * rowkv)[c], f);
+        if (whole && j == last) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) f[e] = vnew[8 * c + e];
+        } else {
+            unpack8(reinterpret_cast<const uint4 *>(vc + (size_t)j * rowkv)[c], f);
+        }
         const float p = sc[j];
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] += p * f[e];
@@ -1068,19 +1109,24 @@ hipError_t launch_rope_kv_rows(hipStream_t s, float *q, const float *k, const fl
     return hipGetLastError();
 }
 
-// out: [n_rows][n_heads * head_dim] f32 -- or, with out == nullptr and xq8_work set, the operand form of the small-batch
-// matrix-core GEMV in that workspace (n_rows <= 8, n_heads * head_dim a multiple of 256)
-hipError_t launch_attn_rows(hipStream_t s, const float *q, const uint16_t *kc, const uint16_t *vc, const int *pos_rows_dev, size_t seq_stride,
-                            int max_pos, size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out, void *xq8_work_buf) {
+// Two forms.  (1) out set: q rotated, the caches hold the step's rows (launch_rope_kv_rows before); result [n_rows][n_heads *
+// head_dim] f32.  (2) out == nullptr, xq8_work_buf, k_new, v_new and inv_freq_dev set: q, k_new, v_new as projected; the launch
+// rotates, appends to the caches and leaves the result in the operand form of the small-batch matrix-core GEMV in that
+// workspace (n_rows <= 8, n_heads * head_dim a multiple of 256).
+hipError_t launch_attn_rows(hipStream_t s, const float *q, uint16_t *kc, uint16_t *vc, const int *pos_rows_dev, size_t seq_stride, int max_pos,
+                            size_t n_rows, int n_heads, int n_kv_heads, int head_dim, float *out, void *xq8_work_buf, const float *k_new,
+                            const float *v_new, const float *inv_freq_dev) {
     if (n_kv_heads <= 0 || n_heads % n_kv_heads != 0 || n_rows == 0 || n_rows > 65535 || max_pos <= 0 || max_pos > 8192) return hipErrorInvalidValue;
     if ((out == nullptr) == (xq8_work_buf == nullptr)) return hipErrorInvalidValue;
     const size_t H = (size_t)n_heads * (size_t)head_dim;
-    if (xq8_work_buf && (n_rows > 8 || H % 256 != 0 || ((uintptr_t)xq8_work_buf & 255))) return hipErrorInvalidValue;
-    const size_t lds = (size_t)max_pos * sizeof(float);      // at most 32 KB beside the 9 KB of static arrays: inside the default 64 KB
+    if (xq8_work_buf && (n_rows > 8 || H % 256 != 0 || ((uintptr_t)xq8_work_buf & 255) || !k_new || !v_new || !inv_freq_dev)) return hipErrorInvalidValue;
+    const size_t lds = (size_t)max_pos * sizeof(float);      // at most 32 KB beside the 10 KB of static arrays: inside the default 64 KB
     const Xq8Work xw = xq8_work_buf ? xq8_work(xq8_work_buf, H) : Xq8Work{ nullptr, nullptr, nullptr };
     dim3 grid((unsigned)n_heads, xq8_work_buf ? 8u : (unsigned)n_rows);
-    if (head_dim == 128) attn_rows_kernel<128><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out, xw, (int)n_rows);
-    else if (head_dim == 64) attn_rows_kernel<64><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out, xw, (int)n_rows);
+    if (head_dim == 128)
+        attn_rows_kernel<128><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out, xw, (int)n_rows, k_new, v_new, inv_freq_dev);
+    else if (head_dim == 64)
+        attn_rows_kernel<64><<<grid, 256, lds, s>>>(q, kc, vc, pos_rows_dev, seq_stride, n_heads, n_kv_heads, out, xw, (int)n_rows, k_new, v_new, inv_freq_dev);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }

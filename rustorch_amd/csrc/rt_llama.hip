@@ -443,9 +443,9 @@ int enqueue_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b) {
     PrefillGemm gemm{ ctx, m };
     RT_TRY_HIP(ctx, rt::launch_embed_rows(s, m->tok_embd.type, m->tok_embd.dev, m->tok_embd.row_bytes, H, b->tok, M, c.vocab, x));
     // Every matrix of a layer on the small-batch matrix-core GEMV (3..8 sequences, Q4_K / Q6_K): the kernel in front of
-    // each contraction writes the GEMV's operand form itself -- RMSNorm for q / k / v and for gate / up, the attention for the
-    // o-projection, SwiGLU for the down-projection -- so no contraction needs a quantizing launch of its own (four launches
-    // fewer per layer), and no f32 copy of those activations is written or read.
+    // each contraction writes the GEMV's operand form itself -- RMSNorm for q / k / v and for gate / up, the attention (which
+    // then also rotates and appends) for the o-projection, SwiGLU for the down-projection -- so no contraction needs a
+    // quantizing launch of its own (five launches fewer per layer), and no f32 copy of those activations is written or read.
     auto mb = [&](const rt_hip_llama::T &t, size_t K) { return t.n_cols == K && rt::qgemv_mb_serves(t.type, t.n_rows, K, (int)M); };
     auto mb_group = [&](std::initializer_list<const rt_hip_llama::T *> ts, std::initializer_list<float *> ys, const float *res, size_t K) {
         for (int type : { (int)RT_GGML_Q4_K, (int)RT_GGML_Q6_K }) {
@@ -469,8 +469,8 @@ int enqueue_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b) {
         if (fused) {
             RT_TRY_HIP(ctx, rt::launch_rmsnorm_xq8(s, x, m->attn_norm[l], M, H, c.rms_eps, ctx->scratch));
             if ((rc = mb_group({ &m->wq[l], &m->wk[l], &m->wv[l] }, { b->q, b->k, b->v }, nullptr, H))) return rc;
-            RT_TRY_HIP(ctx, rt::launch_rope_kv_rows(s, b->q, b->k, b->v, kc, vc, b->pos, seq_stride, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
-            RT_TRY_HIP(ctx, rt::launch_attn_rows(s, b->q, kc, vc, b->pos, seq_stride, b->max_pos, M, c.n_heads, m->n_kv, m->head_dim, nullptr, ctx->scratch));
+            RT_TRY_HIP(ctx, rt::launch_attn_rows(s, b->q, kc, vc, b->pos, seq_stride, b->max_pos, M, c.n_heads, m->n_kv, m->head_dim, nullptr, ctx->scratch,
+                                                 b->k, b->v, m->inv_freq));
             if ((rc = mb_group({ &m->wo[l] }, { x2 }, x, H))) return rc;
             std::swap(x, x2);
             RT_TRY_HIP(ctx, rt::launch_rmsnorm_xq8(s, x, m->ffn_norm[l], M, H, c.rms_eps, ctx->scratch));
@@ -486,7 +486,7 @@ int enqueue_batch_step(rt_hip_ctx *ctx, rt_hip_llama_batch *b) {
         float *qkv_y[3] = { b->q, b->k, b->v };
         if ((rc = gemm.shared(qkv, qkv_y, 3, b->n, M))) return rc;
         RT_TRY_HIP(ctx, rt::launch_rope_kv_rows(s, b->q, b->k, b->v, kc, vc, b->pos, seq_stride, M, c.n_heads, m->n_kv, m->head_dim, m->inv_freq));
-        RT_TRY_HIP(ctx, rt::launch_attn_rows(s, b->q, kc, vc, b->pos, seq_stride, b->max_pos, M, c.n_heads, m->n_kv, m->head_dim, b->a, nullptr));
+        RT_TRY_HIP(ctx, rt::launch_attn_rows(s, b->q, kc, vc, b->pos, seq_stride, b->max_pos, M, c.n_heads, m->n_kv, m->head_dim, b->a, nullptr, nullptr, nullptr, nullptr));
         if ((rc = gemm(m->wo[l], b->a, M, x2, x))) return rc;
         std::swap(x, x2);
         RT_TRY_HIP(ctx, rt::launch_rmsnorm(s, x, m->ffn_norm[l], b->n, nullptr, M, H, c.rms_eps));
