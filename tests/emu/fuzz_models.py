@@ -39,11 +39,16 @@ def one_case(ex, rng, seed):
     n_tok = int(rng.integers(20, 60)); max_pos = n_tok + 4
     if rng.random() < 0.3:
         max_pos = int(rng.integers(512, 700))      # from 512 positions on the decode attention is split over several workgroups
-    uniform = rng.random() < 0.4
+    kind = rng.random()
+    uniform = kind < 0.35
+    k_quants = 0.35 <= kind < 0.6       # Q4_K / Q6_K throughout, as the common 4-bit files are: several sequences then take the fused step
     fmts = {}
     base = str(rng.choice(MATRIX_FORMATS))
     for slot in ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"):
-        fmts[slot] = base if uniform else str(rng.choice(MATRIX_FORMATS[:6] if rng.random() < 0.7 else MATRIX_FORMATS))
+        if k_quants:
+            fmts[slot] = str(rng.choice(["Q4_K", "Q6_K"]))
+        else:
+            fmts[slot] = base if uniform else str(rng.choice(MATRIX_FORMATS[:6] if rng.random() < 0.7 else MATRIX_FORMATS))
     cfg = dict(n_layers=n_layers, hidden=hidden, n_heads=nh, ffn=ffn, vocab=vocab, max_pos=max_pos)
     say("model", cfg, "kv heads", n_kv, "formats", fmts, "tokens", n_tok)
     gm = llama.HipLlama(ex, n_kv_heads=n_kv, **cfg)
